@@ -1,0 +1,141 @@
+/*
+ * mdattn.h -- C ABI of the MI355X (gfx950) DiT attention hot path.
+ *
+ * One shared library (libmdattn.so).  Every entry point
+ *   - takes a HIP stream (hipStream_t passed as void*; NULL = the default stream),
+ *   - only enqueues work on that stream: never synchronises, never allocates,
+ *   - validates its arguments on the host BEFORE any launch and returns a negative
+ *     MDATTN_E_* code instead of launching a kernel that could fault,
+ *   - is re-entrant (no mutable global state).
+ * All pointers are device pointers owned by the caller.  "bf16" tensors hold
+ * bfloat16 bit patterns (uint16_t); the innermost (head_dim) axis is contiguous and
+ * every other axis is described by an element stride, so [B,S,H,D] (= the
+ * reference's rank-3 [B,S,H*D]) and [B,H,S,D] are both accepted without a copy.
+ *
+ * The reference these replace is Python (paths relative to src/maxdiffusion/ of
+ * AI-Hypercomputer/maxdiffusion); each declaration cites the code it stands in for.
+ */
+#ifndef MDATTN_H_
+#define MDATTN_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MDATTN_VERSION 100 /* major*10000 + minor*100 + patch */
+
+enum {
+  MDATTN_OK = 0,
+  MDATTN_E_BADARG = -1,      /* null pointer, non-positive size, inconsistent shape   */
+  MDATTN_E_UNSUPPORTED = -2, /* well-formed request this build has no kernel for      */
+  MDATTN_E_ALIGN = -3,       /* pointer or stride not aligned as the kernels require  */
+  MDATTN_E_LAUNCH = -4       /* the HIP runtime rejected the launch                   */
+};
+
+/* Element strides of one rank-4 tensor [batch, seq, head, dim] with dim contiguous. */
+typedef struct mdattn_strides {
+  int64_t batch;
+  int64_t seq;
+  int64_t head;
+} mdattn_strides;
+
+int mdattn_version(void);
+const char* mdattn_strerror(int code);
+
+/*
+ * Fused RMSNorm over the FULL inner dimension H*D + 3-axis RoPE, for q and k in one pass.
+ * Replaces: FlaxWanAttention.__call__'s norm_q / norm_k (models/attention_flax.py:2657,
+ * :2669; module definition :2529-2553), _unflatten_heads (:2673-2675) and _apply_rope
+ * (:2596-2620, called :2677).
+ *   q_in, k_in   bf16 [B,S,H*D]; k_in may be NULL (only q is processed: the cached-text-KV
+ *                case, attention_flax.py:2659-2660)
+ *   q_out,k_out  bf16, strides out_strides (any of [B,S,H,D] / [B,H,S,D]); may alias the inputs
+ *                when the layouts are identical
+ *   wq, wk       bf16 [H*D] RMSNorm scales
+ *   cos, sin     f32 [S, D/2]: real/imaginary part of the rotary table the unchanged host
+ *                code builds (WanRotaryPosEmbed, models/wan/transformers/transformer_wan.py:63-95);
+ *                both NULL = norm only (cross-attention, rotary_emb is None, attention_flax.py:2671)
+ * Arithmetic: statistics, scale and rotation in f32, ONE rounding to bf16.
+ * Requires D % 8 == 0, H*D <= 8192, 16-byte aligned pointers, strides % 8 == 0.
+ */
+int mdattn_norm_rope_fullrow(void* stream, const void* q_in, const void* k_in, void* q_out, void* k_out,
+                             const void* wq, const void* wk, const float* cos, const float* sin,
+                             int B, int S, int H, int D, float eps,
+                             int64_t in_stride_batch, int64_t in_stride_seq,
+                             const mdattn_strides* out_strides);
+
+/*
+ * Fused per-head RMSNorm (over D) + 3-axis RoPE, for q and k in one pass.
+ * Replaces: FlaxFluxAttention's query_norm / key_norm / encoder_*_norm
+ * (models/attention_flax.py:2947-2967, applied :2989-2990 and :3002-3003; single blocks
+ * models/flux/transformers/transformer_flux_flax.py:192-193) and apply_rope
+ * (models/attention_flax.py:2079-2115, called :3018).
+ *   q_in, k_in   bf16 [B,S,H,D] described by in_strides (k_in may be NULL)
+ *   wq, wk       bf16 [D]; wq_txt / wk_txt (nullable) are used for tokens [0, n_txt)
+ *   cos, sin     f32 [S, D/2] from FluxPosEmbed (models/embeddings_flax.py:437-469); NULL = norm only
+ * Requires D in {64,128,256}.
+ */
+int mdattn_norm_rope_perhead(void* stream, const void* q_in, const void* k_in, void* q_out, void* k_out,
+                             const void* wq, const void* wk, const void* wq_txt, const void* wk_txt, int n_txt,
+                             const float* cos, const float* sin, int B, int S, int H, int D, float eps,
+                             const mdattn_strides* in_strides, const mdattn_strides* out_strides);
+
+/*
+ * Non-causal softmax attention forward, bf16 MFMA, online softmax in f32, optional LSE.
+ * Replaces: the kernel a KERNEL_REGISTRY entry dispatches to (models/attention_flax.py:1589-1597,
+ * :1965-1966), i.e. what _tpu_flash_attention (:563-809) / kernels/custom_splash_attention.py:69-320
+ * compute, with results matching `_apply_attention_dot` (:1487-1567).
+ *   q            bf16 [B,Sq,H,D] by q_strides;  k, v  bf16 [B,Skv,H,D] by k_/v_strides
+ *   out          bf16 [B,Sq,H,D] by o_strides
+ *   lse          f32 [B,H,Sq] contiguous or NULL: natural-log logsumexp of scale*q.k
+ *                (kernels/splash_attention/base.py:103-105)
+ *   scale        applied to q.k inside the kernel (the reference pre-multiplies k, :1783)
+ * Requires D == 128.  Any Sq, Skv >= 1 (ragged tails handled in-kernel).
+ */
+int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* out, float* lse,
+                    int B, int H, int Sq, int Skv, int D,
+                    const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                    const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale);
+
+/*
+ * Per-tensor absmax quantisation bf16 -> OCP float8 e4m3fn (BASELINE configs[4]; no reference
+ * counterpart: the reference's fp8 is qwix quantisation of dense layers, pipelines/wan/wan_pipeline.py:581-626).
+ *   x_bf16 [n] contiguous, x_fp8 [n] bytes,
+ *   scale_out f32[2] device: [0] = absmax/448 (x ~= x_fp8 * scale_out[0]), [1] = absmax (scratch of the reduction)
+ * n % 16 == 0.
+ */
+int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, float* scale_out, int64_t n);
+
+/*
+ * fp8-e4m3 attention forward: q8/k8/v8 are e4m3 bytes [B,S,H,D] by strides, *_scale device f32[1]
+ * de-quantisation factors; P is re-quantised to e4m3 per tile before the PV MFMA; f32 accumulation;
+ * bf16 out; lse as above.  Requires D == 128.
+ */
+int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, const void* v8, void* out, float* lse,
+                   int B, int H, int Sq, int Skv, int D,
+                   const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                   const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
+                   const float* q_scale, const float* k_scale, const float* v_scale);
+
+/*
+ * In-place LSE-space merge of a normalised partial (o_cur, lse_cur) into the running
+ * (o_run f32, lse_run f32); start from o_run = 0, lse_run = -1e30.
+ * Replaces: kernels/splash_attention/ring_attention_kernel.py:1062-1073 (same result as the
+ * (m,l,o) forms :1120-1130 and models/attention_flax.py:753-772).
+ *   o_run  f32 [B,S,H,D] by run_strides; o_cur bf16 (cur_is_f32 == 0) or f32 by cur_strides
+ *   lse_run, lse_cur f32 [B,H,S] contiguous
+ */
+int mdattn_merge(void* stream, float* o_run, float* lse_run, const void* o_cur, const float* lse_cur,
+                 int cur_is_f32, int B, int H, int S, int D,
+                 const mdattn_strides* run_strides, const mdattn_strides* cur_strides);
+
+/* f32 -> bf16 cast of the merged numerator (the `.astype(q.dtype)` of ring_attention_kernel.py:1130).
+ * n % 8 == 0, both contiguous. */
+int mdattn_finalize(void* stream, const float* o_run, void* out_bf16, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MDATTN_H_ */

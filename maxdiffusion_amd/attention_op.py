@@ -1,0 +1,304 @@
+"""Host-side mirror of maxdiffusion's attention plug-in surface for the `hip_flash` kernel.
+
+Same names, argument meaning and error behaviour as the reference (paths relative to
+``src/maxdiffusion/``):
+
+  KERNEL_REGISTRY / register_kernel   models/attention_flax.py:1589-1597
+  _check_attention_inputs             models/attention_flax.py:99-106
+  _apply_attention                    models/attention_flax.py:1870-1968
+  AttentionOp.apply_attention         models/attention_flax.py:2241-2273 (NNXAttentionOp)
+
+Arrays are torch tensors in device memory (the image has no JAX); `jax_plugin.py` registers
+the same kernels with a live maxdiffusion install.  Only the MI355X kernels are registered:
+an unknown name raises ValueError exactly like the reference, and no name is ever demoted
+to a CPU implementation.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+
+__all__ = [
+    "KERNEL_REGISTRY", "register_kernel", "AttentionOp", "hip_flash_kernel", "hip_flash_fp8_kernel",
+    "hip_norm_rope", "HIP_KERNEL_NAMES",
+]
+
+KERNEL_REGISTRY = {}
+
+# Names chosen to contain none of "ring", "ulysses", "custom", "tokamax": the reference keys axis-rule
+# injection and block-size plumbing on those substrings (pyconfig.py:237-238, max_utils.py:781-786).
+HIP_KERNEL_NAMES = ("hip_flash", "hip_flash_fp8")
+
+# Kernel names the reference demotes to dot_product below flash_min_seq_length
+# (attention_flax.py:1905-1912).  The HIP kernels are not in the list: they serve every length.
+_FLASH_MIN_LENGTH_GATED = ("flash", "tokamax_flash", "ulysses", "ulysses_custom", "ulysses_custom_fixed_m", "ulysses_ring")
+
+
+def register_kernel(name: str):
+  def decorator(func):
+    KERNEL_REGISTRY[name] = func
+    return func
+
+  return decorator
+
+
+def _check_attention_inputs(query, key, value) -> None:
+  assert key.ndim == value.ndim, "k, v must have same rank."
+  assert query.shape[:-3] == key.shape[:-3] == value.shape[:-3], "q, k, v batch dims must match."
+  assert key.shape[-2] == value.shape[-2], "k, v num_kv_heads must match."
+  assert key.shape[-3] == value.shape[-3], "k, v lengths must match."
+  assert query.shape[-1] == key.shape[-1], "q, k depths must match."
+
+
+def _as_bshd(x: torch.Tensor, heads: int) -> torch.Tensor:
+  """[B,S,H*D] -> view [B,S,H,D];  [B,H,S,D] -> view [B,S,H,D] (what _reshape_data_for_flash,
+  attention_flax.py:200-220, does with a transpose; here it is a stride change)."""
+  if x.dim() == 3:
+    b, s, n = x.shape
+    if n % heads:
+      raise ValueError(f"inner dim {n} is not divisible by heads={heads}")
+    if x.stride(2) != 1:
+      x = x.contiguous()
+    return x.view(b, s, heads, n // heads) if x.is_contiguous() else x.unflatten(2, (heads, n // heads))
+  if x.dim() == 4:
+    if x.stride(3) != 1:
+      x = x.contiguous()
+    return x.permute(0, 2, 1, 3)
+  raise ValueError(f"attention inputs must have rank 3 or 4, got {x.dim()}")
+
+
+def _reject_unsupported(context) -> None:
+  # The custom kernels of the reference raise NotImplementedError for masks they cannot honour
+  # (attention_flax.py:850-854, :1300-1304); this kernel is non-causal, FullMask only.
+  if context.get("attention_mask") is not None:
+    raise NotImplementedError("hip_flash does not take an attention_mask (non-causal, unmasked DiT attention only)")
+  if context.get("is_causal"):
+    raise NotImplementedError("hip_flash is non-causal")
+
+
+@register_kernel("hip_flash")
+def hip_flash_kernel(q, k, v, context):
+  """KERNEL_REGISTRY entry: fn(q, k, v, context) -> [B, Sq, H*D] in q's dtype.
+
+  Unlike the reference's flash entries, which pass k * scale (attention_flax.py:1783), the scale goes
+  to the kernel and is folded into the exp2 argument; `flash_block_sizes`, `mesh` and the axis names
+  are accepted and ignored (one GPU, tiles fixed by the kernel).
+  """
+  _reject_unsupported(context)
+  heads = context["heads"]
+  qv, kv, vv = _as_bshd(q, heads), _as_bshd(k, heads), _as_bshd(v, heads)
+  cast = q.dtype != torch.bfloat16
+  if cast:  # LTX2 hands f32 q/k (attention_ltx2.py:415-432); the MFMA operands are bf16
+    qv, kv, vv = qv.to(torch.bfloat16), kv.to(torch.bfloat16), vv.to(torch.bfloat16)
+  out = ops.flash_attention(qv, kv, vv, scale=context["scale"])
+  b, s, h, d = out.shape
+  out = out.reshape(b, s, h * d)
+  return out.to(q.dtype) if cast else out
+
+
+@register_kernel("hip_flash_fp8")
+def hip_flash_fp8_kernel(q, k, v, context):
+  """fp8-e4m3 variant: per-tensor absmax quantisation of q, k, v on the device, then the fp8 kernel."""
+  _reject_unsupported(context)
+  heads = context["heads"]
+  qv, kv, vv = (_as_bshd(t, heads).to(torch.bfloat16).contiguous() for t in (q, k, v))
+  q8, sq = ops.quant_e4m3(qv)
+  k8, sk = ops.quant_e4m3(kv)
+  v8, sv = ops.quant_e4m3(vv)
+  out = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=context["scale"])
+  b, s, h, d = out.shape
+  return out.reshape(b, s, h * d).to(q.dtype)
+
+
+def _apply_attention(
+    query,
+    key,
+    value,
+    heads: int,
+    dim_head: int,
+    split_head_dim: bool,
+    float32_qk_product: bool,
+    attention_kernel: str,
+    flash_min_seq_length: int,
+    use_memory_efficient_attention: bool,
+    scale: float,
+    dtype,
+    mesh,
+    axis_names_q,
+    axis_names_kv,
+    flash_block_sizes,
+    dpa_layer,
+    mask_padding_tokens: bool = True,
+    residual_checkpoint_name: str | None = None,
+    attention_mask=None,
+    use_base2_exp: bool = False,
+    use_experimental_scheduler: bool = False,
+    ulysses_shards: int = -1,
+    ulysses_attention_chunks: int = 1,
+    is_causal: bool = False,
+):
+  """Routes to an attention kernel through the module-level registry (attention_flax.py:1870-1968)."""
+  _check_attention_inputs(query, key, value)
+  seq_len_idx = 2 if query.ndim == 4 else 1
+
+  can_use_flash_attention = True
+  if attention_kernel in _FLASH_MIN_LENGTH_GATED:
+    can_use_flash_attention = (
+        query.shape[seq_len_idx] >= flash_min_seq_length
+        and key.shape[seq_len_idx] >= flash_min_seq_length
+        and value.shape[seq_len_idx] >= flash_min_seq_length
+    )
+
+  effective_attention_kernel = attention_kernel
+  if attention_kernel == "dot_product" or use_memory_efficient_attention or not can_use_flash_attention:
+    effective_attention_kernel = "dot_product"
+
+  if attention_mask is not None:
+    if attention_mask.ndim != 2:
+      raise ValueError(f"attention_mask must have shape [batch, kv_length], got {tuple(attention_mask.shape)}.")
+    attention_mask = attention_mask.to(torch.bool)
+
+  context = {
+      "heads": heads,
+      "mesh": mesh,
+      "axis_names_q": axis_names_q,
+      "axis_names_kv": axis_names_kv,
+      "flash_block_sizes": flash_block_sizes,
+      "dtype": dtype,
+      "mask_padding_tokens": mask_padding_tokens,
+      "residual_checkpoint_name": residual_checkpoint_name,
+      "attention_mask": attention_mask,
+      "scale": scale,
+      "use_base2_exp": use_base2_exp,
+      "use_experimental_scheduler": use_experimental_scheduler,
+      "ulysses_shards": ulysses_shards,
+      "ulysses_attention_chunks": ulysses_attention_chunks,
+      "dim_head": dim_head,
+      "split_head_dim": split_head_dim,
+      "float32_qk_product": float32_qk_product,
+      "use_memory_efficient_attention": use_memory_efficient_attention,
+      "dpa_layer": dpa_layer,
+      "is_causal": is_causal,
+  }
+
+  if effective_attention_kernel in KERNEL_REGISTRY:
+    return KERNEL_REGISTRY[effective_attention_kernel](query, key, value, context)
+
+  raise ValueError(f"Unexpected attention kernel {effective_attention_kernel=}.")
+
+
+class AttentionOp:
+  """Same constructor arguments and `apply_attention` signature as NNXAttentionOp
+  (attention_flax.py:2172-2273); `mesh`, axis names and block sizes are carried, not used."""
+
+  def __init__(
+      self,
+      mesh=None,
+      attention_kernel: str = "hip_flash",
+      scale: float = 1.0,
+      heads: int = 1,
+      dim_head: int = 128,
+      use_memory_efficient_attention: bool = False,
+      split_head_dim: bool = True,
+      float32_qk_product: bool = True,
+      axis_names_q=("activation_batch", "activation_heads", "activation_length", "activation_kv"),
+      axis_names_kv=("activation_batch", "activation_heads", "activation_kv_length", "activation_kv"),
+      flash_min_seq_length: int = 0,
+      flash_block_sizes=None,
+      dtype=torch.float32,
+      quant=None,
+      mask_padding_tokens: bool = True,
+      residual_checkpoint_name: str | None = None,
+      use_base2_exp: bool = False,
+      use_experimental_scheduler: bool = False,
+      ulysses_shards: int = -1,
+      ulysses_attention_chunks: int = 1,
+  ):
+    self.dpa_layer = None
+    self.mesh = mesh
+    self.scale = scale
+    self.heads = heads
+    self.dim_head = dim_head
+    self.attention_kernel = attention_kernel
+    self.use_memory_efficient_attention = use_memory_efficient_attention
+    self.split_head_dim = split_head_dim
+    self.float32_qk_product = float32_qk_product
+    self.axis_names_q = axis_names_q
+    self.axis_names_kv = axis_names_kv
+    self.flash_min_seq_length = flash_min_seq_length
+    self.flash_block_sizes = flash_block_sizes
+    self.dtype = dtype
+    self.quant = quant
+    self.mask_padding_tokens = mask_padding_tokens
+    self.residual_checkpoint_name = residual_checkpoint_name
+    self.use_base2_exp = use_base2_exp
+    self.use_experimental_scheduler = use_experimental_scheduler
+    self.ulysses_shards = ulysses_shards
+    self.ulysses_attention_chunks = ulysses_attention_chunks
+
+  def apply_attention(self, query, key, value, attention_mask=None):
+    return _apply_attention(
+        query=query,
+        key=key,
+        value=value,
+        heads=self.heads,
+        dim_head=self.dim_head,
+        split_head_dim=self.split_head_dim,
+        float32_qk_product=self.float32_qk_product,
+        attention_kernel=self.attention_kernel,
+        flash_min_seq_length=self.flash_min_seq_length,
+        use_memory_efficient_attention=self.use_memory_efficient_attention,
+        scale=self.scale,
+        dtype=self.dtype,
+        mesh=self.mesh,
+        axis_names_q=self.axis_names_q,
+        axis_names_kv=self.axis_names_kv,
+        flash_block_sizes=self.flash_block_sizes,
+        dpa_layer=self.dpa_layer,
+        mask_padding_tokens=self.mask_padding_tokens,
+        residual_checkpoint_name=self.residual_checkpoint_name,
+        attention_mask=attention_mask,
+        use_base2_exp=self.use_base2_exp,
+        use_experimental_scheduler=self.use_experimental_scheduler,
+        ulysses_shards=self.ulysses_shards,
+        ulysses_attention_chunks=self.ulysses_attention_chunks,
+    )
+
+
+def _split_table(freqs_cis, seq: int, d: int):
+  """Accepts the reference's rotary tables and returns contiguous f32 (cos, sin) [S, D/2]:
+  complex [1,1,S,D/2] (WanRotaryPosEmbed), (cos, sin) tuples with D or D/2 columns
+  (FluxPosEmbed return_tuple, repeated pairwise), or the [S, D/2, 2, 2] matrix form."""
+  if freqs_cis is None:
+    return None, None
+  if isinstance(freqs_cis, (tuple, list)):
+    cos, sin = freqs_cis
+    cos, sin = cos.reshape(seq, -1), sin.reshape(seq, -1)
+    if cos.shape[1] == d:  # each angle repeated for both members of the pair
+      cos, sin = cos[:, 0::2], sin[:, 0::2]
+  elif torch.is_complex(freqs_cis):
+    t = freqs_cis.reshape(seq, d // 2)
+    cos, sin = t.real, t.imag
+  else:
+    t = freqs_cis.reshape(seq, d // 2, 2, 2)
+    cos, sin = t[:, :, 0, 0], t[:, :, 1, 0]
+  return cos.to(torch.float32).contiguous(), sin.to(torch.float32).contiguous()
+
+
+def hip_norm_rope(q, k, wq, wk, freqs_cis, heads: int, eps: float = 1e-6, per_head: bool = False,
+                  wq_txt=None, wk_txt=None, n_txt: int = 0, out_layout: str = "bshd"):
+  """The fused prologue the attention modules call in place of their inline norm + rope.
+
+  per_head=False: FlaxWanAttention.__call__ lines attention_flax.py:2655-2677 (q, k are [B,S,H*D]).
+  per_head=True : FlaxFluxAttention.__call__ lines :2989-3020 (q, k are [B,S,H,D] views).
+  freqs_cis=None is the norm-only mode of the cross-attention (:2671).  Returns logical [B,S,H,D]
+  views laid out as `out_layout`, ready for `hip_flash` with no transpose in between.
+  """
+  if per_head:
+    b, s, h, d = q.shape
+    cos, sin = _split_table(freqs_cis, s, d)
+    return ops.norm_rope_perhead(q, k, wq, wk, cos, sin, eps, wq_txt, wk_txt, n_txt, out_layout)
+  b, s, n = q.shape
+  cos, sin = _split_table(freqs_cis, s, n // heads)
+  return ops.norm_rope_fullrow(q, k, wq, wk, cos, sin, heads, eps, out_layout)

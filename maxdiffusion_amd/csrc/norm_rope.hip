@@ -1,0 +1,267 @@
+// Fused q/k RMSNorm + interleaved-pair RoPE for gfx950.  HBM-bound: every q and k element is
+// read once (16-byte loads) and written once (16-byte stores); statistics, scale and rotation
+// are f32 in registers with a single rounding to bf16.
+#include "mdattn_common.h"
+
+namespace mdattn {
+
+struct NormRopeFullArgs {
+  const uint4* x_in[2];   // q, k  (k may be null)
+  uint4* x_out[2];
+  const uint4* w[2];
+  const float4* cos;
+  const float4* sin;
+  int S, H, D, N;         // N = H*D
+  float eps, inv_n;
+  int64_t in_sb, in_ss;
+  int64_t out_sb, out_ss, out_sh;
+};
+
+// One workgroup (256 lanes) per token row; lane t owns 16-byte chunks t, t+256, ... (<= MAXC).
+template <int MAXC>
+__global__ __launch_bounds__(256) void norm_rope_fullrow_kernel(NormRopeFullArgs a) {
+  const int tid = threadIdx.x;
+  const int s = blockIdx.x, b = blockIdx.y;
+  const int nchunks = a.N >> 3;
+  const int ntens = a.x_in[1] ? 2 : 1;
+  __shared__ float red[2][16];
+
+  uint4 raw[2][MAXC];
+  float ss[2] = {0.f, 0.f};
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    if (t < ntens) {
+      const uint4* row = a.x_in[t] + ((b * a.in_sb + s * a.in_ss) >> 3);
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = tid + i * 256;
+        if (c < nchunks) raw[t][i] = ld_nt(row + c);
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    if (t < ntens) {
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = tid + i * 256;
+        if (c < nchunks) {
+          float f[8];
+          unpack8(raw[t][i], f);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) ss[t] = __builtin_fmaf(f[j], f[j], ss[t]);
+        }
+      }
+      ss[t] = row16_sum(ss[t]);
+      if ((tid & 15) == 0) red[t][tid >> 4] = ss[t];
+    }
+  }
+  __syncthreads();
+  float inv[2] = {0.f, 0.f};
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    if (t < ntens) {
+      float tot = 0.f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) tot += red[t][j];
+      const float x = tot * a.inv_n + a.eps;
+      const float y = __builtin_amdgcn_rsqf(x);
+      // one Newton step brings v_rsq_f32 (1 ulp) to f32 round-off: y*(1.5 - 0.5*x*y*y)
+      inv[t] = y * (1.5f - 0.5f * x * y * y);
+    }
+  }
+
+  const bool rope = a.cos != nullptr;
+  const int halfd4 = a.D >> 3;  // float4 chunks per table row
+#pragma unroll
+  for (int i = 0; i < MAXC; ++i) {
+    const int c = tid + i * 256;
+    if (c < nchunks) {
+      const int e = c << 3;
+      const int h = e / a.D, d = e - h * a.D;
+      float4 cs = {1.f, 1.f, 1.f, 1.f}, sn = {0.f, 0.f, 0.f, 0.f};
+      if (rope) {
+        cs = a.cos[(int64_t)s * halfd4 + (d >> 3)];
+        sn = a.sin[(int64_t)s * halfd4 + (d >> 3)];
+      }
+      const float cc[4] = {cs.x, cs.y, cs.z, cs.w}, sv[4] = {sn.x, sn.y, sn.z, sn.w};
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        if (t < ntens) {
+          float f[8], w[8], o[8];
+          unpack8(raw[t][i], f);
+          unpack8(a.w[t][c], w);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) f[j] = f[j] * inv[t] * w[j];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            o[2 * j] = f[2 * j] * cc[j] - f[2 * j + 1] * sv[j];
+            o[2 * j + 1] = f[2 * j] * sv[j] + f[2 * j + 1] * cc[j];
+          }
+          uint4* dst = a.x_out[t] + ((b * a.out_sb + s * a.out_ss + h * a.out_sh + d) >> 3);
+          st_nt(dst, pack8(o));
+        }
+      }
+    }
+  }
+}
+
+struct NormRopeHeadArgs {
+  const uint4* x_in[2];
+  uint4* x_out[2];
+  const uint4* w[2];
+  const uint4* w_txt[2];
+  const float4* cos;
+  const float4* sin;
+  int S, H, n_txt;
+  int64_t rows;  // B*S*H
+  float eps;
+  int64_t in_sb, in_ss, in_sh, out_sb, out_ss, out_sh;
+};
+
+// LPR = D/8 lanes per (token, head) row; each lane owns one 16-byte chunk; RPT rows per lane group
+// in flight so that enough bytes are outstanding per CU.
+template <int LPR, int RPT>
+__global__ __launch_bounds__(256) void norm_rope_perhead_kernel(NormRopeHeadArgs a) {
+  constexpr int D = LPR * 8;
+  constexpr int GROUPS = 256 / LPR;
+  const int tid = threadIdx.x;
+  const int lane = tid % LPR;
+  const int64_t row0 = ((int64_t)blockIdx.x * GROUPS + tid / LPR) * RPT;
+  const int ntens = a.x_in[1] ? 2 : 1;
+  const bool rope = a.cos != nullptr;
+
+  uint4 raw[2][RPT];
+  int64_t oofs[RPT];
+  int tok[RPT];
+#pragma unroll
+  for (int r = 0; r < RPT; ++r) {
+    int64_t row = row0 + r;
+    if (row >= a.rows) row = a.rows - 1;  // clamp loads; stores are predicated below
+    const int h = (int)(row % a.H);
+    const int64_t bs = row / a.H;
+    const int s = (int)(bs % a.S);
+    const int64_t b = bs / a.S;
+    tok[r] = s;
+    oofs[r] = b * a.out_sb + s * a.out_ss + h * a.out_sh;
+    const int64_t iofs = b * a.in_sb + s * a.in_ss + h * a.in_sh;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+      if (t < ntens) raw[t][r] = ld_nt(a.x_in[t] + (iofs >> 3) + lane);
+  }
+#pragma unroll
+  for (int r = 0; r < RPT; ++r) {
+    float4 cs = {1.f, 1.f, 1.f, 1.f}, sn = {0.f, 0.f, 0.f, 0.f};
+    if (rope) {
+      cs = a.cos[(int64_t)tok[r] * LPR + lane];
+      sn = a.sin[(int64_t)tok[r] * LPR + lane];
+    }
+    const float cc[4] = {cs.x, cs.y, cs.z, cs.w}, sv[4] = {sn.x, sn.y, sn.z, sn.w};
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      if (t < ntens) {
+        float f[8], w[8], o[8];
+        unpack8(raw[t][r], f);
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(f[j], f[j], ss);
+        if (LPR >= 16) {
+          ss = row16_sum(ss);
+          if (LPR == 32) ss += __shfl_xor(ss, 16);
+        } else {  // LPR == 8
+          ss += __shfl_xor(ss, 1); ss += __shfl_xor(ss, 2); ss += __shfl_xor(ss, 4);
+        }
+        const float x = ss * (1.0f / D) + a.eps;
+        float inv = __builtin_amdgcn_rsqf(x);
+        inv = inv * (1.5f - 0.5f * x * inv * inv);
+        const uint4* wp = (a.w_txt[t] && tok[r] < a.n_txt) ? a.w_txt[t] : a.w[t];
+        unpack8(wp[lane], w);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] = f[j] * inv * w[j];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          o[2 * j] = f[2 * j] * cc[j] - f[2 * j + 1] * sv[j];
+          o[2 * j + 1] = f[2 * j] * sv[j] + f[2 * j + 1] * cc[j];
+        }
+        if (row0 + r < a.rows) st_nt(a.x_out[t] + (oofs[r] >> 3) + lane, pack8(o));
+      }
+    }
+  }
+}
+
+}  // namespace mdattn
+
+using namespace mdattn;
+
+extern "C" int mdattn_norm_rope_fullrow(void* stream, const void* q_in, const void* k_in, void* q_out, void* k_out,
+                                        const void* wq, const void* wk, const float* cos, const float* sin,
+                                        int B, int S, int H, int D, float eps,
+                                        int64_t in_stride_batch, int64_t in_stride_seq,
+                                        const mdattn_strides* out_strides) {
+  if (!q_in || !q_out || !wq || B <= 0 || S <= 0 || H <= 0 || D <= 0 || !out_strides) return MDATTN_E_BADARG;
+  if ((k_in == nullptr) != (k_out == nullptr) || (k_in && !wk)) return MDATTN_E_BADARG;
+  if ((cos == nullptr) != (sin == nullptr)) return MDATTN_E_BADARG;
+  if (!(eps >= 0.f)) return MDATTN_E_BADARG;
+  const int64_t N = (int64_t)H * D;
+  if (D % 8 != 0 || N > 8192) return MDATTN_E_UNSUPPORTED;
+  if (B > 65535) return MDATTN_E_UNSUPPORTED;
+  if (in_stride_seq < N || in_stride_batch < 0) return MDATTN_E_BADARG;
+  if (!aligned16(q_in) || !aligned16(q_out) || !aligned16(wq) || !aligned16(k_in) || !aligned16(k_out) ||
+      !aligned16(wk) || !aligned16(cos) || !aligned16(sin))
+    return MDATTN_E_ALIGN;
+  if (in_stride_batch % 8 || in_stride_seq % 8 || !strides_ok(out_strides, 8)) return MDATTN_E_ALIGN;
+
+  NormRopeFullArgs a;
+  a.x_in[0] = (const uint4*)q_in; a.x_in[1] = (const uint4*)k_in;
+  a.x_out[0] = (uint4*)q_out; a.x_out[1] = (uint4*)k_out;
+  a.w[0] = (const uint4*)wq; a.w[1] = (const uint4*)wk;
+  a.cos = (const float4*)cos; a.sin = (const float4*)sin;
+  a.S = S; a.H = H; a.D = D; a.N = (int)N; a.eps = eps; a.inv_n = 1.0f / (float)N;
+  a.in_sb = in_stride_batch; a.in_ss = in_stride_seq;
+  a.out_sb = out_strides->batch; a.out_ss = out_strides->seq; a.out_sh = out_strides->head;
+  dim3 grid(S, B), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  const int nchunks = (int)(N / 8);
+  if (nchunks <= 256) hipLaunchKernelGGL(norm_rope_fullrow_kernel<1>, grid, block, 0, st, a);
+  else if (nchunks <= 512) hipLaunchKernelGGL(norm_rope_fullrow_kernel<2>, grid, block, 0, st, a);
+  else if (nchunks <= 768) hipLaunchKernelGGL(norm_rope_fullrow_kernel<3>, grid, block, 0, st, a);
+  else hipLaunchKernelGGL(norm_rope_fullrow_kernel<4>, grid, block, 0, st, a);
+  return launch_status();
+}
+
+extern "C" int mdattn_norm_rope_perhead(void* stream, const void* q_in, const void* k_in, void* q_out, void* k_out,
+                                        const void* wq, const void* wk, const void* wq_txt, const void* wk_txt,
+                                        int n_txt, const float* cos, const float* sin, int B, int S, int H, int D,
+                                        float eps, const mdattn_strides* in_strides,
+                                        const mdattn_strides* out_strides) {
+  if (!q_in || !q_out || !wq || B <= 0 || S <= 0 || H <= 0 || D <= 0 || !in_strides || !out_strides) return MDATTN_E_BADARG;
+  if ((k_in == nullptr) != (k_out == nullptr) || (k_in && !wk)) return MDATTN_E_BADARG;
+  if ((cos == nullptr) != (sin == nullptr)) return MDATTN_E_BADARG;
+  if (n_txt < 0 || n_txt > S || !(eps >= 0.f)) return MDATTN_E_BADARG;
+  if (D != 64 && D != 128 && D != 256) return MDATTN_E_UNSUPPORTED;
+  if (!aligned16(q_in) || !aligned16(q_out) || !aligned16(wq) || !aligned16(k_in) || !aligned16(k_out) ||
+      !aligned16(wk) || !aligned16(wq_txt) || !aligned16(wk_txt) || !aligned16(cos) || !aligned16(sin))
+    return MDATTN_E_ALIGN;
+  if (!strides_ok(in_strides, 8) || !strides_ok(out_strides, 8)) return MDATTN_E_ALIGN;
+
+  NormRopeHeadArgs a;
+  a.x_in[0] = (const uint4*)q_in; a.x_in[1] = (const uint4*)k_in;
+  a.x_out[0] = (uint4*)q_out; a.x_out[1] = (uint4*)k_out;
+  a.w[0] = (const uint4*)wq; a.w[1] = (const uint4*)wk;
+  a.w_txt[0] = (const uint4*)wq_txt; a.w_txt[1] = k_in ? (const uint4*)wk_txt : nullptr;
+  a.cos = (const float4*)cos; a.sin = (const float4*)sin;
+  a.S = S; a.H = H; a.n_txt = n_txt; a.rows = (int64_t)B * S * H; a.eps = eps;
+  a.in_sb = in_strides->batch; a.in_ss = in_strides->seq; a.in_sh = in_strides->head;
+  a.out_sb = out_strides->batch; a.out_ss = out_strides->seq; a.out_sh = out_strides->head;
+  constexpr int RPT = 4;
+  const int lpr = D / 8;
+  const int64_t rows_per_block = (256 / lpr) * RPT;
+  const int64_t nblocks = (a.rows + rows_per_block - 1) / rows_per_block;
+  if (nblocks > 0x7FFFFFFF) return MDATTN_E_UNSUPPORTED;
+  dim3 grid((unsigned)nblocks), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  if (lpr == 8) hipLaunchKernelGGL((norm_rope_perhead_kernel<8, RPT>), grid, block, 0, st, a);
+  else if (lpr == 16) hipLaunchKernelGGL((norm_rope_perhead_kernel<16, RPT>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((norm_rope_perhead_kernel<32, RPT>), grid, block, 0, st, a);
+  return launch_status();
+}

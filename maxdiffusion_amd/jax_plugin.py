@@ -1,0 +1,112 @@
+"""Registers the HIP kernels with a live maxdiffusion + JAX (ROCm) install.
+
+`install()` (1) registers the XLA-FFI targets exported by libmdattn_ffi.so with
+``jax.ffi.register_ffi_target(..., platform="ROCM")`` and (2) adds ``hip_flash`` to
+maxdiffusion's own KERNEL_REGISTRY (models/attention_flax.py:1589-1597), after which
+``attention: hip_flash`` in any Wan / Flux / LTX config reaches the MI355X kernel through
+the unchanged `_apply_attention` (models/attention_flax.py:1965-1966).
+
+Nothing here runs at import time: jax, jaxlib's FFI headers and maxdiffusion are absent from
+the build image, so this module is exercised only where they exist.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+from .build import FFI_LIB_PATH, build_ffi_library
+
+FFI_TARGETS = {
+    "mdattn_fwd_bf16": "MdattnFwdBf16",
+    "mdattn_norm_rope_fullrow": "MdattnNormRopeFullrow",
+    "mdattn_norm_rope_perhead": "MdattnNormRopePerhead",
+    "mdattn_merge": "MdattnMerge",
+}
+
+_installed = False
+
+
+def _require_jax():
+  try:
+    import jax  # noqa: F401
+    import jax.ffi  # noqa: F401
+    import jax.numpy as jnp  # noqa: F401
+  except ImportError as e:  # pragma: no cover - jax is not in the build image
+    raise RuntimeError("maxdiffusion_amd.jax_plugin needs jax with ROCm support") from e
+  return jax, jnp
+
+
+def register_ffi_targets():
+  jax, _ = _require_jax()
+  if not os.path.exists(FFI_LIB_PATH) and build_ffi_library() is None:
+    raise RuntimeError("libmdattn_ffi.so is missing and jaxlib's FFI headers were not found to build it")
+  lib = ctypes.CDLL(FFI_LIB_PATH)
+  for target, symbol in FFI_TARGETS.items():
+    jax.ffi.register_ffi_target(target, jax.ffi.pycapsule(getattr(lib, symbol)), platform="ROCM")
+
+
+def hip_flash_attention(q, k, v, scale: float, layout: int):
+  """q [B,Sq,H,D] (layout 0) or [B,H,Sq,D] (layout 1) bf16 -> (out [B,Sq,H,D] bf16, lse [B,H,Sq] f32)."""
+  jax, jnp = _require_jax()
+  if layout == 0:
+    b, sq, h, d = q.shape
+  else:
+    b, h, sq, d = q.shape
+  call = jax.ffi.ffi_call(
+      "mdattn_fwd_bf16",
+      (jax.ShapeDtypeStruct((b, sq, h, d), jnp.bfloat16), jax.ShapeDtypeStruct((b, h, sq), jnp.float32)),
+      vmap_method="sequential",
+  )
+  import numpy as np
+
+  return call(q, k, v, scale=np.float32(scale), layout=np.int64(layout))
+
+
+def hip_norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6):
+  """q, k [B,S,H*D] bf16; cos/sin f32 [S,D/2] or None -> (q_out, k_out) [B,S,H,D] bf16."""
+  jax, jnp = _require_jax()
+  import numpy as np
+
+  b, s, n = q.shape
+  d = n // heads
+  rope = cos is not None
+  if not rope:
+    cos = sin = jnp.zeros((1, 1), jnp.float32)
+  out = jax.ShapeDtypeStruct((b, s, heads, d), jnp.bfloat16)
+  call = jax.ffi.ffi_call("mdattn_norm_rope_fullrow", (out, out), vmap_method="sequential")
+  return call(q, k, wq, wk, cos, sin, eps=np.float32(eps), heads=np.int64(heads), rope=np.int64(rope))
+
+
+def hip_flash_kernel(q, k, v, context):
+  """The KERNEL_REGISTRY entry: fn(q, k, v, context) -> [B, Sq, H*D] in q's dtype."""
+  _, jnp = _require_jax()
+  if context.get("attention_mask") is not None:
+    raise NotImplementedError("hip_flash does not take an attention_mask (non-causal, unmasked DiT attention only)")
+  if context.get("is_causal"):
+    raise NotImplementedError("hip_flash is non-causal")
+  heads = context["heads"]
+  if q.ndim == 3:
+    b, sq, n = q.shape
+    d = n // heads
+    q4 = q.reshape(b, sq, heads, d)
+    k4 = k.reshape(b, k.shape[1], heads, d)
+    v4 = v.reshape(b, v.shape[1], heads, d)
+    layout = 0
+  else:
+    q4, k4, v4, layout = q, k, v, 1
+  dt = q.dtype
+  out, _ = hip_flash_attention(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"], layout)
+  b, sq, h, d = out.shape
+  return out.reshape(b, sq, h * d).astype(dt)
+
+
+def install():
+  """Idempotent: FFI targets + maxdiffusion KERNEL_REGISTRY['hip_flash']."""
+  global _installed
+  if _installed:
+    return
+  register_ffi_targets()
+  from maxdiffusion.models import attention_flax  # type: ignore
+
+  attention_flax.register_kernel("hip_flash")(hip_flash_kernel)
+  _installed = True

@@ -1,0 +1,199 @@
+"""Host-side operators of the DiT attention hot path (torch tensors in HBM -> libmdattn.so).
+
+torch is used for device memory and the current HIP stream only; every computation below is
+a hand-written HIP kernel reached through the C ABI.  Tensors are logical [B, S, H, D] views
+(any strides, D contiguous), so a [B, H, S, D] buffer is passed as ``x.permute(0, 2, 1, 3)``
+and the reference's rank-3 [B, S, H*D] as ``x.view(B, S, H, D)`` -- never copied.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+
+import torch
+
+from . import _lib
+from ._lib import Strides
+
+__all__ = [
+    "norm_rope_fullrow", "norm_rope_perhead", "flash_attention", "flash_attention_fp8", "quant_e4m3",
+    "merge_partial", "finalize", "new_merge_state", "LSE_INIT",
+]
+
+LSE_INIT = -1e30
+
+
+def _ptr(t):
+  return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+  return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check_dev(*ts):
+  for t in ts:
+    if t is not None and not t.is_cuda:
+      raise ValueError("mdattn operators need tensors in device memory (cuda/HIP); there is no CPU path")
+
+
+def _strides(t: torch.Tensor) -> Strides:
+  if t.dim() != 4 or t.stride(3) != 1:
+    raise ValueError(f"expected a [B,S,H,D] view with contiguous D, got shape {tuple(t.shape)} strides {t.stride()}")
+  return Strides(t.stride(0), t.stride(1), t.stride(2))
+
+
+def _alloc_like_layout(b, s, h, d, layout: str, dtype, device):
+  """Returns a logical [B,S,H,D] view over a fresh buffer laid out as `layout`."""
+  if layout == "bshd":
+    return torch.empty((b, s, h, d), dtype=dtype, device=device)
+  if layout == "bhsd":
+    return torch.empty((b, h, s, d), dtype=dtype, device=device).permute(0, 2, 1, 3)
+  raise ValueError(f"unknown layout {layout!r} (want 'bshd' or 'bhsd')")
+
+
+def _table(t, s, d, name):
+  if t is None:
+    return None
+  if t.dtype != torch.float32 or tuple(t.shape) != (s, d // 2) or not t.is_contiguous():
+    raise ValueError(f"{name} must be a contiguous float32 [S, D/2] = [{s}, {d // 2}] tensor, got {tuple(t.shape)} {t.dtype}")
+  return t
+
+
+def norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6, out_layout: str = "bshd"):
+  """q, k: bf16 [B, S, H*D] (k may be None) -> (q_out, k_out) logical [B,S,H,D] views in `out_layout`.
+
+  RMSNorm over H*D, then rotation of interleaved pairs by the [S, D/2] table (cos/sin None: norm only).
+  """
+  _check_dev(q, k, wq, wk, cos, sin)
+  if q.dim() != 3 or q.dtype != torch.bfloat16 or q.stride(2) != 1:
+    raise ValueError("q must be bf16 [B, S, H*D] with a contiguous last axis")
+  b, s, n = q.shape
+  if n % heads:
+    raise ValueError(f"inner dim {n} is not divisible by heads={heads}")
+  d = n // heads
+  if k is not None and (k.shape != q.shape or k.dtype != q.dtype or k.stride() != q.stride()):
+    raise ValueError("k must match q in shape, dtype and strides")
+  cos, sin = _table(cos, s, d, "cos"), _table(sin, s, d, "sin")
+  q_out = _alloc_like_layout(b, s, heads, d, out_layout, torch.bfloat16, q.device)
+  k_out = _alloc_like_layout(b, s, heads, d, out_layout, torch.bfloat16, q.device) if k is not None else None
+  st = _strides(q_out)
+  rc = _lib.load().mdattn_norm_rope_fullrow(
+      _stream(), _ptr(q), _ptr(k), _ptr(q_out), _ptr(k_out), _ptr(wq), _ptr(wk), _ptr(cos), _ptr(sin),
+      b, s, heads, d, eps, q.stride(0), q.stride(1), ctypes.byref(st))
+  _lib.check(rc, "mdattn_norm_rope_fullrow")
+  return q_out, k_out
+
+
+def norm_rope_perhead(q, k, wq, wk, cos, sin, eps: float = 1e-6, wq_txt=None, wk_txt=None, n_txt: int = 0,
+                      out_layout: str = "bshd"):
+  """q, k: bf16 logical [B, S, H, D] views (k may be None); RMSNorm over D per head, then RoPE."""
+  _check_dev(q, k, wq, wk, wq_txt, wk_txt, cos, sin)
+  if q.dtype != torch.bfloat16:
+    raise ValueError("q must be bf16")
+  b, s, h, d = q.shape
+  if k is not None and (k.shape != q.shape or k.stride() != q.stride() or k.dtype != q.dtype):
+    raise ValueError("k must match q in shape, dtype and strides")
+  cos, sin = _table(cos, s, d, "cos"), _table(sin, s, d, "sin")
+  q_out = _alloc_like_layout(b, s, h, d, out_layout, torch.bfloat16, q.device)
+  k_out = _alloc_like_layout(b, s, h, d, out_layout, torch.bfloat16, q.device) if k is not None else None
+  si, so = _strides(q), _strides(q_out)
+  rc = _lib.load().mdattn_norm_rope_perhead(
+      _stream(), _ptr(q), _ptr(k), _ptr(q_out), _ptr(k_out), _ptr(wq), _ptr(wk), _ptr(wq_txt), _ptr(wk_txt), n_txt,
+      _ptr(cos), _ptr(sin), b, s, h, d, eps, ctypes.byref(si), ctypes.byref(so))
+  _lib.check(rc, "mdattn_norm_rope_perhead")
+  return q_out, k_out
+
+
+def flash_attention(q, k, v, scale: float | None = None, return_lse: bool = False, out_layout: str = "bshd", out=None):
+  """softmax(scale * q k^T) v, non-causal.  q [B,Sq,H,D], k/v [B,Skv,H,D] logical views, bf16.
+
+  Returns out (logical [B,Sq,H,D] in `out_layout`) and, if asked, lse f32 [B,H,Sq] (natural log).
+  """
+  _check_dev(q, k, v)
+  if not (q.dtype == k.dtype == v.dtype == torch.bfloat16):
+    raise ValueError("flash_attention needs bf16 q, k, v")
+  b, sq, h, d = q.shape
+  if k.shape != v.shape or k.shape[0] != b or k.shape[2] != h or k.shape[3] != d:
+    raise ValueError(f"inconsistent shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)}")
+  skv = k.shape[1]
+  if scale is None:
+    scale = 1.0 / math.sqrt(d)
+  if out is None:
+    out = _alloc_like_layout(b, sq, h, d, out_layout, torch.bfloat16, q.device)
+  lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device) if return_lse else None
+  sq_, sk_, sv_, so_ = _strides(q), _strides(k), _strides(v), _strides(out)
+  rc = _lib.load().mdattn_fwd_bf16(
+      _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), b, h, sq, skv, d,
+      ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale))
+  _lib.check(rc, "mdattn_fwd_bf16")
+  return (out, lse) if return_lse else out
+
+
+def quant_e4m3(x: torch.Tensor):
+  """Per-tensor absmax quantisation of a contiguous bf16 tensor -> (uint8 e4m3 bytes, f32[2] scale buffer)."""
+  _check_dev(x)
+  if x.dtype != torch.bfloat16 or not x.is_contiguous():
+    raise ValueError("quant_e4m3 needs a contiguous bf16 tensor")
+  x8 = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+  scale = torch.empty(2, dtype=torch.float32, device=x.device)
+  rc = _lib.load().mdattn_quant_e4m3(_stream(), _ptr(x), _ptr(x8), _ptr(scale), x.numel())
+  _lib.check(rc, "mdattn_quant_e4m3")
+  return x8, scale
+
+
+def flash_attention_fp8(q8, k8, v8, q_scale, k_scale, v_scale, scale: float | None = None, return_lse: bool = False,
+                        out_layout: str = "bshd"):
+  """fp8-e4m3 variant: q8/k8/v8 uint8 logical [B,S,H,D] views, *_scale device f32 tensors (element 0 is used)."""
+  _check_dev(q8, k8, v8, q_scale, k_scale, v_scale)
+  b, sq, h, d = q8.shape
+  skv = k8.shape[1]
+  if scale is None:
+    scale = 1.0 / math.sqrt(d)
+  out = _alloc_like_layout(b, sq, h, d, out_layout, torch.bfloat16, q8.device)
+  lse = torch.empty((b, h, sq), dtype=torch.float32, device=q8.device) if return_lse else None
+  sq_, sk_, sv_, so_ = _strides(q8), _strides(k8), _strides(v8), _strides(out)
+  rc = _lib.load().mdattn_fwd_fp8(
+      _stream(), _ptr(q8), _ptr(k8), _ptr(v8), _ptr(out), _ptr(lse), b, h, sq, skv, d,
+      ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale),
+      _ptr(q_scale), _ptr(k_scale), _ptr(v_scale))
+  _lib.check(rc, "mdattn_fwd_fp8")
+  return (out, lse) if return_lse else out
+
+
+def new_merge_state(b, s, h, d, device, layout: str = "bshd"):
+  """(o_run f32 zeros as a logical [B,S,H,D] view, lse_run f32 [B,H,S] filled with -1e30)."""
+  o = _alloc_like_layout(b, s, h, d, layout, torch.float32, device)
+  o.zero_()
+  lse = torch.full((b, h, s), LSE_INIT, dtype=torch.float32, device=device)
+  return o, lse
+
+
+def merge_partial(o_run, lse_run, o_cur, lse_cur):
+  """In-place LSE-space merge of (o_cur, lse_cur) into (o_run, lse_run)."""
+  _check_dev(o_run, lse_run, o_cur, lse_cur)
+  b, s, h, d = o_run.shape
+  if o_run.dtype != torch.float32 or o_cur.shape != o_run.shape or o_cur.dtype not in (torch.bfloat16, torch.float32):
+    raise ValueError("o_run must be f32 and o_cur bf16/f32 of the same logical shape")
+  for t in (lse_run, lse_cur):
+    if t.dtype != torch.float32 or tuple(t.shape) != (b, h, s) or not t.is_contiguous():
+      raise ValueError("lse tensors must be contiguous f32 [B,H,S]")
+  sr, sc = _strides(o_run), _strides(o_cur)
+  rc = _lib.load().mdattn_merge(
+      _stream(), _ptr(o_run), _ptr(lse_run), _ptr(o_cur), _ptr(lse_cur), int(o_cur.dtype == torch.float32),
+      b, h, s, d, ctypes.byref(sr), ctypes.byref(sc))
+  _lib.check(rc, "mdattn_merge")
+  return o_run, lse_run
+
+
+def finalize(o_run: torch.Tensor) -> torch.Tensor:
+  """f32 -> bf16 cast of a merged accumulator, same memory layout."""
+  _check_dev(o_run)
+  if o_run.dtype != torch.float32:
+    raise ValueError("finalize needs an f32 tensor")
+  out = torch.empty_like(o_run, dtype=torch.bfloat16)  # preserves strides of dense permuted views
+  if out.stride() != o_run.stride():
+    raise ValueError("finalize needs a dense tensor")
+  rc = _lib.load().mdattn_finalize(_stream(), _ptr(o_run), _ptr(out), o_run.numel())
+  _lib.check(rc, "mdattn_finalize")
+  return out

@@ -1,0 +1,394 @@
+"""numpy restatement of maxdiffusion's DiT attention hot path (CPU oracle).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py, never by the product package.
+
+Reference paths are relative to ``src/maxdiffusion/`` of the reference tree.
+
+Pinning status of each function (what fixes it besides its own formula):
+
+  bf16_round / to_bf16_bits      torch.bfloat16 casts on CPU (library routine)
+  e4m3_round                     torch.float8_e4m3fn casts on CPU (library routine)
+  rmsnorm                        torch.nn.functional.rms_norm, closed forms
+                                 (constant row, w=1/eps=0 unit RMS)
+  wan_rope_angles / table        shape fixture (1,1,75600,64) and split 22/21/21
+                                 from tests/wan/wan_transformer_test.py:51-78,
+                                 brute-force (f,h,w) loop, unit modulus
+  flux_rope_angles / table       text ids -> identity, pair split 8/28/28,
+                                 tuple form == matrix form of apply_rope
+  apply_rope_interleaved         complex128 multiply, composition, inverse,
+                                 relative-position property
+  attention / attention_rows     scipy logsumexp, torch SDPA (fp32, CPU),
+                                 invariants (K=0 -> mean(V), lse=ln Skv; ...),
+                                 hand fixtures of tests/ltx2/test_attention_ltx2.py:38-116
+  merge_lse / merge_mlo /        attention over a union of KV chunks equals the
+  merge_scan_ring                merge of per-chunk results (brute force)
+  attention_dot_product_bf16     PARITY UNPINNED at bit level: the rounding points
+                                 of XLA-CPU's bf16 einsum/softmax are not fixed by
+                                 any reference test; it is pinned only to tolerance
+                                 (2e-2) against `attention`, like the reference's
+                                 own tests do (tests/attention_test.py:90-147).
+  attention_fp8_emulated         no reference counterpart (BASELINE configs[4]);
+                                 defined by this file, pinned only through
+                                 e4m3_round and cosine vs `attention`.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+__all__ = [
+    "bf16_round", "to_bf16_bits", "from_bf16_bits", "e4m3_round", "E4M3_MAX",
+    "rmsnorm", "wan_rope_angles", "wan_rope_table", "wan_rope_table_complex",
+    "flux_ids", "flux_rope_angles", "flux_rope_table", "flux_rope_table_matrix",
+    "apply_rope_interleaved", "apply_rope_matrix_form", "norm_rope_fullrow", "norm_rope_perhead",
+    "norm_rope_wan_reference_flow", "attention", "attention_rows", "attention_dot_product_bf16",
+    "merge_lse", "merge_mlo", "merge_scan_ring", "ring_replay", "quant_e4m3", "attention_fp8_emulated",
+    "LSE_INIT",
+]
+
+E4M3_MAX = 448.0
+LSE_INIT = -1e30  # finite "empty" lse, ring_attention_kernel.py:944-946
+
+
+# --------------------------------------------------------------------------- dtype helpers
+def to_bf16_bits(x: np.ndarray) -> np.ndarray:
+  """float32 -> bf16 bit pattern (uint16), round-to-nearest-even, NaN kept quiet."""
+  x = np.ascontiguousarray(x, dtype=np.float32)
+  u = x.view(np.uint32)
+  bias = ((u >> 16) & 1) + np.uint32(0x7FFF)
+  r = ((u + bias) >> 16).astype(np.uint16)
+  nan = np.isnan(x)
+  if nan.any():
+    r = np.where(nan, np.uint16(0x7FC0), r)
+  return r
+
+
+def from_bf16_bits(b: np.ndarray) -> np.ndarray:
+  return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def bf16_round(x: np.ndarray) -> np.ndarray:
+  """Round float values to the nearest bf16, returned as float32."""
+  return from_bf16_bits(to_bf16_bits(np.asarray(x, dtype=np.float32)))
+
+
+def e4m3_round(x: np.ndarray) -> np.ndarray:
+  """Round to OCP float8 e4m3fn (bias 7, max 448, no inf), saturating, as float32.
+
+  Values are rounded to nearest-even on a grid of 3 mantissa bits; the subnormal
+  grid is 2**-9.
+  """
+  x = np.asarray(x, dtype=np.float32)
+  a = np.minimum(np.abs(x).astype(np.float64), E4M3_MAX)
+  with np.errstate(divide="ignore"):
+    e = np.floor(np.log2(np.where(a > 0, a, 1.0)))
+  e = np.maximum(e, -6.0)  # subnormals share the exponent of the smallest normal
+  q = np.exp2(e - 3.0)  # grid spacing
+  r = np.rint(a / q) * q  # np.rint is round-half-even
+  r = np.minimum(r, E4M3_MAX)
+  return (np.sign(x) * r).astype(np.float32)
+
+
+# --------------------------------------------------------------------------- A1 RMSNorm
+def rmsnorm(x: np.ndarray, w: np.ndarray, eps: float = 1e-6, dtype=np.float64) -> np.ndarray:
+  """y = x * rsqrt(mean(x^2, last axis) + eps) * w, un-rounded.
+
+  Wan: full inner dim H*D (attention_flax.py:2529-2553, applied :2657 and :2669).
+  Flux: last axis D per head (attention_flax.py:2947-2967, applied :2989-2990).
+  flax RMSNorm keeps statistics in float32; `dtype` selects the oracle's precision.
+  """
+  xf = np.asarray(x, dtype=dtype)
+  ms = np.mean(xf * xf, axis=-1, keepdims=True)
+  return xf / np.sqrt(ms + dtype(eps)) * np.asarray(w, dtype=dtype)
+
+
+# --------------------------------------------------------------------------- A2 Wan rotary table
+def _inv_freq(dim: int, theta: float) -> np.ndarray:
+  # embeddings_flax.py:239  1 / theta ** (arange(0, dim, 2) / dim), float32
+  return (1.0 / (np.float32(theta) ** (np.arange(0, dim, 2, dtype=np.float32)[: dim // 2] / np.float32(dim)))).astype(np.float32)
+
+
+def wan_rope_angles(grid: tuple[int, int, int], head_dim: int = 128, theta: float = 10000.0) -> np.ndarray:
+  """Angles [S, head_dim/2] (float32) for a post-patch token grid (ppf, pph, ppw).
+
+  transformer_wan.py:43-60: h_dim = w_dim = 2*(D//6), t_dim = D - h_dim - w_dim; the
+  first t_dim/2 pairs rotate with the frame index, the next h_dim/2 with the row, the
+  last w_dim/2 with the column.  transformer_wan.py:77-95: token order is row-major
+  over (ppf, pph, ppw).
+  """
+  ppf, pph, ppw = grid
+  h_dim = w_dim = 2 * (head_dim // 6)
+  t_dim = head_dim - h_dim - w_dim
+  f = np.arange(ppf, dtype=np.float32)[:, None] * _inv_freq(t_dim, theta)[None, :]
+  h = np.arange(pph, dtype=np.float32)[:, None] * _inv_freq(h_dim, theta)[None, :]
+  w = np.arange(ppw, dtype=np.float32)[:, None] * _inv_freq(w_dim, theta)[None, :]
+  ang = np.concatenate(
+      [
+          np.broadcast_to(f[:, None, None, :], (ppf, pph, ppw, t_dim // 2)),
+          np.broadcast_to(h[None, :, None, :], (ppf, pph, ppw, h_dim // 2)),
+          np.broadcast_to(w[None, None, :, :], (ppf, pph, ppw, w_dim // 2)),
+      ],
+      axis=-1,
+  )
+  return np.ascontiguousarray(ang.reshape(ppf * pph * ppw, head_dim // 2), dtype=np.float32)
+
+
+def wan_rope_table(grid, head_dim: int = 128, theta: float = 10000.0):
+  """(cos, sin), each float32 [S, head_dim/2]: real and imaginary part of exp(1j*angle)."""
+  ang = wan_rope_angles(grid, head_dim, theta).astype(np.float64)
+  return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+
+def wan_rope_table_complex(grid, head_dim: int = 128, theta: float = 10000.0) -> np.ndarray:
+  """complex64 [1, 1, S, head_dim/2], the shape WanRotaryPosEmbed returns (transformer_wan.py:94)."""
+  c, s = wan_rope_table(grid, head_dim, theta)
+  return (c + 1j * s).astype(np.complex64)[None, None]
+
+
+# --------------------------------------------------------------------------- A3 Flux rotary table
+def flux_ids(n_txt: int, height: int, width: int) -> np.ndarray:
+  """ids [n_txt + height*width, 3]: text rows (0,0,0); image rows (0,row,col) row-major.
+
+  transformer_flux_flax.py:622-629 (text ids first), :687-693 (image ids).
+  """
+  img = np.zeros((height, width, 3), dtype=np.float32)
+  img[..., 1] = np.arange(height, dtype=np.float32)[:, None]
+  img[..., 2] = np.arange(width, dtype=np.float32)[None, :]
+  return np.concatenate([np.zeros((n_txt, 3), np.float32), img.reshape(-1, 3)], axis=0)
+
+
+def flux_rope_angles(ids: np.ndarray, axes_dim=(16, 56, 56), theta: float = 10000.0) -> np.ndarray:
+  """Angles [L, sum(axes_dim)/2] float32: axis a owns axes_dim[a]/2 consecutive pairs.
+
+  embeddings_flax.py:437-469 with get_1d_rotary_pos_embed :222-250.
+  """
+  cols = []
+  for a, dim in enumerate(axes_dim):
+    cols.append(np.asarray(ids[:, a], dtype=np.float32)[:, None] * _inv_freq(dim, theta)[None, :])
+  return np.concatenate(cols, axis=1).astype(np.float32)
+
+
+def flux_rope_table(ids, axes_dim=(16, 56, 56), theta: float = 10000.0, table_dtype: str = "f32"):
+  """(cos, sin) float32 [L, 64].  table_dtype="bf16" rounds the table entries to bf16, the
+  precision FluxPosEmbed produces when the model dtype is bf16 (transformer_flux_flax.py:434)."""
+  ang = flux_rope_angles(ids, axes_dim, theta).astype(np.float64)
+  c, s = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+  if table_dtype == "bf16":
+    c, s = bf16_round(c), bf16_round(s)
+  return c, s
+
+
+def flux_rope_table_matrix(ids, axes_dim=(16, 56, 56), theta: float = 10000.0) -> np.ndarray:
+  """[L, 64, 2, 2] table packed [cos, -sin, sin, cos] (embeddings_flax.py:246)."""
+  c, s = flux_rope_table(ids, axes_dim, theta)
+  return np.stack([c, -s, s, c], axis=-1).reshape(c.shape[0], c.shape[1], 2, 2)
+
+
+# --------------------------------------------------------------------------- A4 RoPE application
+def apply_rope_interleaved(x: np.ndarray, cos: np.ndarray, sin: np.ndarray, seq_axis: int = -3) -> np.ndarray:
+  """Rotate interleaved pairs: o[2j] = x[2j] c - x[2j+1] s; o[2j+1] = x[2j] s + x[2j+1] c.
+
+  attention_flax.py:2596-2620 (Wan), :2079-2107 (Flux tuple form).  `x` is [..., S, H, D]
+  (seq_axis=-3) or [..., H, S, D] (seq_axis=-2); cos/sin are [S, D/2], shared by all heads.
+  """
+  x = np.asarray(x)
+  dt = np.result_type(x.dtype, np.float32)
+  xr = x.astype(dt).reshape(*x.shape[:-1], x.shape[-1] // 2, 2)
+  shape = [1] * xr.ndim
+  shape[seq_axis - 1] = cos.shape[0]  # one more trailing axis after the reshape
+  shape[-2] = cos.shape[1]
+  c = np.asarray(cos, dtype=dt).reshape(shape[:-1])
+  s = np.asarray(sin, dtype=dt).reshape(shape[:-1])
+  x0, x1 = xr[..., 0], xr[..., 1]
+  out = np.stack([x0 * c - x1 * s, x0 * s + x1 * c], axis=-1)
+  return out.reshape(x.shape)
+
+
+def apply_rope_matrix_form(x: np.ndarray, table: np.ndarray) -> np.ndarray:
+  """Matrix form of the same rotation (attention_flax.py:2109-2115): x [H, L, D], table [L, D/2, 2, 2]."""
+  x_ = np.asarray(x, np.float64).reshape(*x.shape[:-1], -1, 1, 2)
+  out = table[..., 0] * x_[..., 0] + table[..., 1] * x_[..., 1]
+  return out.reshape(x.shape)
+
+
+def norm_rope_fullrow(x, w, cos, sin, heads: int, eps: float = 1e-6, dtype=np.float64):
+  """Fused prologue, Wan flavour: x [B, S, H*D] -> RMSNorm over H*D -> rope -> [B, S, H, D].
+
+  attention_flax.py:2655-2677 (norm_q/norm_k, unflatten heads, _apply_rope).  Everything
+  in `dtype`, no intermediate rounding; cos=None gives the norm-only mode used by the
+  cross-attention (rotary_emb is None, attention_flax.py:2671).
+  """
+  b, s, hd = x.shape
+  y = rmsnorm(x, w, eps, dtype).reshape(b, s, heads, hd // heads)
+  if cos is None:
+    return y
+  return apply_rope_interleaved(y, cos, sin, seq_axis=-3)
+
+
+def norm_rope_perhead(x, w, cos, sin, eps: float = 1e-6, dtype=np.float64, w_txt=None, n_txt: int = 0):
+  """Fused prologue, Flux flavour: x [B, L, H, D] -> RMSNorm over D -> rope -> [B, L, H, D].
+
+  attention_flax.py:2989-3020.  Tokens [0, n_txt) use `w_txt` when given (the text stream's
+  own encoder_*_norm weights in the double blocks, :3002-3003).
+  """
+  y = rmsnorm(x, w, eps, dtype)
+  if w_txt is not None and n_txt > 0:
+    y[:, :n_txt] = rmsnorm(x[:, :n_txt], w_txt, eps, dtype)
+  if cos is None:
+    return y
+  return apply_rope_interleaved(y, cos, sin, seq_axis=-3)
+
+
+def norm_rope_wan_reference_flow(x_bf16, w_bf16, cos, sin, heads: int, eps: float = 1e-6):
+  """The reference's rounding sequence for bf16 activations (returns bf16 values as float32).
+
+  RMSNorm statistics in f32, result cast to bf16 (attention_flax.py:2529-2553); cos/sin cast
+  to bf16 (:2598-2599); each product and each sum rounded to bf16 (:2609-2613, the
+  un-fused reading; XLA may keep wider intermediates).
+  """
+  b, s, hd = x_bf16.shape
+  y = bf16_round(rmsnorm(x_bf16, w_bf16, eps, np.float32)).reshape(b, s, heads, hd // heads)
+  c = bf16_round(cos)[None, :, None, :]
+  sn = bf16_round(sin)[None, :, None, :]
+  yr = y.reshape(b, s, heads, -1, 2)
+  y0, y1 = yr[..., 0], yr[..., 1]
+  o0 = bf16_round(bf16_round(y0 * c) - bf16_round(y1 * sn))
+  o1 = bf16_round(bf16_round(y0 * sn) + bf16_round(y1 * c))
+  return np.stack([o0, o1], axis=-1).reshape(b, s, heads, hd // heads)
+
+
+# --------------------------------------------------------------------------- A5 attention + LSE
+def attention(q, k, v, scale: float, dtype=np.float64, kv_mask=None):
+  """Dense non-causal softmax attention with natural-log LSE over the scaled logits.
+
+  q [H, Sq, D], k/v [H, Skv, D] -> (out [H, Sq, D], lse [H, Sq]); the f32 oracle of
+  kernels/splash_attention/base.py:70-106 (logsumexp = m + log(l)) with the `scale`
+  the dispatcher supplies (attention_flax.py:1549).  kv_mask [Skv] bool keeps keys;
+  rows with no kept key return out=0 (attention_flax.py:1552-1554) and lse=-inf.
+  """
+  q = np.asarray(q, dtype)
+  k = np.asarray(k, dtype)
+  v = np.asarray(v, dtype)
+  s = np.matmul(q, np.swapaxes(k, -1, -2)) * dtype(scale)
+  if kv_mask is not None:
+    s = np.where(np.asarray(kv_mask, bool)[None, None, :], s, -np.inf)
+  m = s.max(axis=-1)
+  m_safe = np.where(np.isfinite(m), m, 0.0)
+  p = np.exp(s - m_safe[..., None])
+  l = p.sum(axis=-1)
+  with np.errstate(divide="ignore", invalid="ignore"):
+    out = np.where(l[..., None] > 0, np.matmul(p, v) / l[..., None], 0.0)
+    lse = np.where(l > 0, m_safe + np.log(l), -np.inf)
+  return out, lse
+
+
+def attention_rows(q_rows, k, v, scale: float, dtype=np.float64):
+  """Same as `attention` for a sample of query rows of ONE head: q_rows [R, D], k/v [Skv, D]."""
+  out, lse = attention(np.asarray(q_rows)[None], np.asarray(k)[None], np.asarray(v)[None], scale, dtype)
+  return out[0], lse[0]
+
+
+def attention_dot_product_bf16(q, k, v, scale: float):
+  """dtype flow of `_apply_attention_dot` for bf16 inputs (attention_flax.py:1487-1567).
+
+  float32_qk_product=False: scores are produced in bf16 (:1546), scaled in bf16 (:1549),
+  softmax in bf16 storage (:1551), probabilities cast to `dtype` (:1556), PV einsum with
+  bf16 result (:1564).  Each stage is computed in f32 and rounded to bf16 where the
+  reference stores bf16.  q [H,Sq,D], k/v [H,Skv,D] (bf16 values held in float32).
+  """
+  q = np.asarray(q, np.float32)
+  k = np.asarray(k, np.float32)
+  v = np.asarray(v, np.float32)
+  s = bf16_round(np.matmul(q, np.swapaxes(k, -1, -2)))
+  s = bf16_round(s * bf16_round(np.float32(scale)))
+  m = s.max(axis=-1, keepdims=True)
+  e = np.exp(s - m)
+  p = bf16_round(e / e.sum(axis=-1, keepdims=True))
+  return bf16_round(np.matmul(p, v))
+
+
+# --------------------------------------------------------------------------- A6 merges
+def merge_lse(o_run, lse_run, o_cur, lse_cur, dtype=np.float64):
+  """LSE-space merge of two normalised partials over disjoint KV sets.
+
+  ring_attention_kernel.py:1062-1073.  o [..., S, D], lse [..., S].  Start from
+  o_run = 0, lse_run = LSE_INIT.
+  """
+  o_run = np.asarray(o_run, dtype)
+  o_cur = np.asarray(o_cur, dtype)
+  lse_run = np.asarray(lse_run, dtype)
+  lse_cur = np.asarray(lse_cur, dtype)
+  L = np.maximum(lse_run, lse_cur)
+  w1 = np.exp(lse_run - L)
+  w2 = np.exp(lse_cur - L)
+  den = w1 + w2
+  o = (w1[..., None] * o_run + w2[..., None] * o_cur) / den[..., None]
+  return o, L + np.log(den)
+
+
+def merge_mlo(m_run, l_run, o_run, m_cur, l_cur, o_cur):
+  """(m, l, o) merge of un-normalised partials (ring_attention_kernel.py:1120-1126)."""
+  m_next = np.maximum(m_run, m_cur)
+  alpha = np.exp(m_run - m_next)
+  beta = np.exp(m_cur - m_next)
+  return m_next, alpha * l_run + beta * l_cur, alpha[..., None] * o_run + beta[..., None] * o_cur
+
+
+def merge_scan_ring(outs, lses):
+  """The scan-ring merge (attention_flax.py:736-772): lse of the first chunk seeds m,
+  l = exp(lse - m), o = out * l; every later chunk folds in; result o / l."""
+  m = np.asarray(lses[0], np.float64)
+  l = np.exp(np.asarray(lses[0], np.float64) - m)
+  o = np.asarray(outs[0], np.float64) * l[..., None]
+  for out_c, lse_c in zip(outs[1:], lses[1:]):
+    m_old = m
+    m = np.maximum(m_old, lse_c)
+    a = np.exp(m_old - m)
+    l = l * a + np.exp(lse_c - m)
+    o = o * a[..., None] + np.exp(lse_c - m)[..., None] * np.asarray(out_c, np.float64)
+  return o / l[..., None], m + np.log(l)
+
+
+def ring_replay(q, k_chunks, v_chunks, scale: float, dtype=np.float64):
+  """One Q shard against successive KV chunks, merged in LSE space (BASELINE configs[3])."""
+  o_run = np.zeros(q.shape, dtype)
+  lse_run = np.full(q.shape[:-1], LSE_INIT, dtype)
+  for kc, vc in zip(k_chunks, v_chunks):
+    o, lse = attention(q, kc, vc, scale, dtype)
+    o_run, lse_run = merge_lse(o_run, lse_run, o, lse, dtype)
+  return o_run, lse_run
+
+
+# --------------------------------------------------------------------------- A7 fp8 variant
+def quant_e4m3(x):
+  """Per-tensor absmax quantisation: s = absmax/448, x8 = e4m3(x / s).  Returns (x8 as f32, s)."""
+  x = np.asarray(x, np.float32)
+  s = np.float32(max(float(np.abs(x).max()), 1e-12) / E4M3_MAX)
+  return e4m3_round(x / s), s
+
+
+def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64):
+  """Emulation of the fp8 kernel's arithmetic (no reference counterpart).
+
+  Q, K, V quantised per tensor; logits from the quantised operands in f32; online softmax
+  per KV tile with P rounded to e4m3 before the PV product; f32 accumulation; the row sum
+  uses the un-rounded P.  q [H,Sq,D], k/v [H,Skv,D].
+  """
+  q8, sq = quant_e4m3(q)
+  k8, sk = quant_e4m3(k)
+  v8, sv = quant_e4m3(v)
+  H, Sq, D = q8.shape
+  Skv = k8.shape[1]
+  m = np.full((H, Sq), -np.inf, np.float32)
+  l = np.zeros((H, Sq), np.float32)
+  o = np.zeros((H, Sq, D), np.float32)
+  c = np.float32(sq * sk * scale)
+  for t0 in range(0, Skv, kv_tile):
+    s = np.einsum("hqd,hkd->hqk", q8, k8[:, t0:t0 + kv_tile]) * c
+    m_new = np.maximum(m, s.max(axis=-1))
+    a = np.exp(m - m_new)
+    p = np.exp(s - m_new[..., None])
+    l = a * l + p.sum(axis=-1)
+    o = a[..., None] * o + np.einsum("hqk,hkd->hqd", e4m3_round(p), v8[:, t0:t0 + kv_tile])
+    m = m_new
+  return o * sv / l[..., None], m + np.log(l)

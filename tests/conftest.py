@@ -1,0 +1,49 @@
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for _p in (ROOT, os.path.join(ROOT, "tests")):
+  if _p not in sys.path:
+    sys.path.insert(0, _p)
+
+
+def pytest_configure(config):
+  config.addinivalue_line("markers", "gpu: needs a real MI355X (run through gpurun / at round end)")
+
+
+def _has_gpu() -> bool:
+  try:
+    import torch
+
+    return torch.cuda.is_available()
+  except Exception:
+    return False
+
+
+def pytest_collection_modifyitems(config, items):
+  if _has_gpu():
+    return
+  skip = pytest.mark.skip(reason="no GPU visible")
+  for item in items:
+    if "gpu" in item.keywords:
+      item.add_marker(skip)
+
+
+@pytest.fixture(scope="session")
+def lib():
+  """The built C-ABI library; built once here only if nothing is built yet."""
+  from maxdiffusion_amd import _lib, build
+
+  if not os.path.exists(build.LIB_PATH):
+    build.build_library()
+  return _lib.load()
+
+
+@pytest.fixture(scope="session")
+def dev(lib):
+  import torch
+
+  return torch.device("cuda:0")

@@ -1,0 +1,83 @@
+"""Writes the committed golden vectors (inputs + expected outputs) for the hot path.
+
+    python tests/golden/make_golden.py
+
+Every expected output comes from the numpy oracle in float64 (oracle/dit_attention.py), whose
+functions are pinned by tests/test_oracle.py; inputs are bf16 bit patterns.  The reference
+(JAX) cannot be imported in this image, so no vector here was produced by running it.
+"""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+import oracle as O  # noqa: E402
+
+
+def bits(x):
+  return O.to_bf16_bits(x)
+
+
+def main():
+  # Wan-flavour prologue: grid 3x4x4 (the HF parity grid), 4 heads x 128
+  grid, H, D = (3, 4, 4), 4, 128
+  S = 3 * 4 * 4
+  q = O.normal_bf16((1, S, H * D), 0)
+  k = O.normal_bf16((1, S, H * D), 1)
+  wq, wk = O.norm_weight(H * D, 3), O.norm_weight(H * D, 4)
+  cos, sin = O.wan_rope_table(grid, D)
+  np.savez_compressed(
+      os.path.join(HERE, "norm_rope_wan.npz"), q=bits(q), k=bits(k), wq=bits(wq), wk=bits(wk), cos=cos, sin=sin, heads=H,
+      q_out=O.norm_rope_fullrow(q, wq, cos, sin, H).astype(np.float32),
+      k_out=O.norm_rope_fullrow(k, wk, cos, sin, H).astype(np.float32),
+      q_norm_only=O.norm_rope_fullrow(q, wq, None, None, H).astype(np.float32))
+
+  # Flux-flavour prologue: 5 text tokens + 4x6 image tokens, 3 heads x 128, separate text weights
+  ids = O.flux_ids(5, 4, 6)
+  L = ids.shape[0]
+  q = O.normal_bf16((1, L, 3, 128), 0)
+  k = O.normal_bf16((1, L, 3, 128), 1)
+  wq, wk, wqt, wkt = (O.norm_weight(128, s) for s in (3, 4, 5, 6))
+  cos, sin = O.flux_rope_table(ids)
+  np.savez_compressed(
+      os.path.join(HERE, "norm_rope_flux.npz"), q=bits(q), k=bits(k), wq=bits(wq), wk=bits(wk), wq_txt=bits(wqt), wk_txt=bits(wkt),
+      cos=cos, sin=sin, n_txt=5,
+      q_out=O.norm_rope_perhead(q, wq, cos, sin, w_txt=wqt, n_txt=5).astype(np.float32),
+      k_out=O.norm_rope_perhead(k, wk, cos, sin, w_txt=wkt, n_txt=5).astype(np.float32))
+
+  # attention + lse: ragged Sq and Skv (neither a multiple of 32 or 64), 2 heads; plus a sharpened case
+  q = O.normal_bf16((1, 70, 2, 128), 0)
+  k = O.normal_bf16((1, 100, 2, 128), 1)
+  v = O.normal_bf16((1, 100, 2, 128), 2)
+  out, lse = O.attention(q[0].transpose(1, 0, 2), k[0].transpose(1, 0, 2), v[0].transpose(1, 0, 2), 128**-0.5)
+  qs = O.bf16_round(q * 6.0)
+  outs, lses = O.attention(qs[0].transpose(1, 0, 2), k[0].transpose(1, 0, 2), v[0].transpose(1, 0, 2), 128**-0.5)
+  np.savez_compressed(
+      os.path.join(HERE, "attention_small.npz"), q=bits(q), k=bits(k), v=bits(v), scale=128**-0.5,
+      out=out.transpose(1, 0, 2)[None].astype(np.float32), lse=lse[None].astype(np.float32),
+      q_sharp=bits(qs), out_sharp=outs.transpose(1, 0, 2)[None].astype(np.float32), lse_sharp=lses[None].astype(np.float32))
+
+  # merge: three unequal KV chunks of the same attention problem
+  splits = [0, 37, 38, 100]
+  parts_o, parts_l = [], []
+  for a, b in zip(splits[:-1], splits[1:]):
+    o, l = O.attention(q[0].transpose(1, 0, 2), k[0, a:b].transpose(1, 0, 2), v[0, a:b].transpose(1, 0, 2), 128**-0.5)
+    parts_o.append(O.bf16_round(o.transpose(1, 0, 2)[None]))  # partials as the kernel hands them over: bf16
+    parts_l.append(l[None].astype(np.float32))
+  o_run = np.zeros((1, 70, 2, 128))
+  l_run = np.full((1, 2, 70), O.LSE_INIT)
+  for o, l in zip(parts_o, parts_l):
+    o_t, l_run = O.merge_lse(o_run.transpose(0, 2, 1, 3), l_run, o.transpose(0, 2, 1, 3), l)
+    o_run = o_t.transpose(0, 2, 1, 3)
+  np.savez_compressed(
+      os.path.join(HERE, "merge_small.npz"), parts_o=np.stack([bits(o) for o in parts_o]), parts_l=np.stack(parts_l),
+      o_merged=o_run.astype(np.float32), lse_merged=l_run.astype(np.float32))
+  for f in sorted(os.listdir(HERE)):
+    if f.endswith(".npz"):
+      print(f, os.path.getsize(os.path.join(HERE, f)))
+
+
+if __name__ == "__main__":
+  main()

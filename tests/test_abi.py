@@ -1,0 +1,99 @@
+"""The C-ABI library loads on a machine without a GPU, exports every symbol include/mdattn.h
+declares, and rejects malformed requests on the host (no kernel launch, no GPU needed)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mdattn.h")
+
+
+def declared_symbols():
+  text = open(HEADER).read()
+  text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+  return sorted(set(re.findall(r"\b(mdattn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+  assert declared_symbols() == sorted([
+      "mdattn_version", "mdattn_strerror", "mdattn_norm_rope_fullrow", "mdattn_norm_rope_perhead", "mdattn_fwd_bf16",
+      "mdattn_quant_e4m3", "mdattn_fwd_fp8", "mdattn_merge", "mdattn_finalize",
+  ])
+
+
+def test_library_exports_every_declared_symbol(lib):
+  from maxdiffusion_amd import _lib
+
+  for name in declared_symbols():
+    assert hasattr(lib, name), f"libmdattn.so does not export {name}"
+    assert name in _lib.SIGNATURES, f"ctypes binding lacks {name}"
+  assert sorted(_lib.SIGNATURES) == declared_symbols()
+
+
+def test_version_and_strerror(lib):
+  text = open(HEADER).read()
+  want = int(re.search(r"#define MDATTN_VERSION (\d+)", text).group(1))
+  assert lib.mdattn_version() == want
+  for code in (0, -1, -2, -3, -4, -99):
+    assert len(lib.mdattn_strerror(code)) > 0
+  assert lib.mdattn_strerror(0) == b"ok"
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+  from maxdiffusion_amd import _lib
+
+  monkeypatch.setattr(_lib, "_lib", None)
+  monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmdattn.so"))
+  with pytest.raises(RuntimeError, match="no non-HIP fallback"):
+    _lib.load()
+
+
+def _st(b, s, h):
+  from maxdiffusion_amd._lib import Strides
+
+  return ctypes.byref(Strides(b, s, h))
+
+
+def test_bad_arguments_are_rejected_on_the_host(lib):
+  from maxdiffusion_amd import _lib
+
+  P = ctypes.c_void_p
+  fake = P(0x1000)  # aligned, never dereferenced: every call below must fail validation first
+  odd = P(0x1004)
+  st = _st(128 * 8 * 4, 128 * 4, 128)
+  f = lib.mdattn_fwd_bf16
+  assert f(None, None, fake, fake, fake, None, 1, 4, 8, 8, 128, st, st, st, st, 0.1) == _lib.E_BADARG
+  assert f(None, fake, fake, fake, fake, None, 1, 4, 0, 8, 128, st, st, st, st, 0.1) == _lib.E_BADARG
+  assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 128, st, st, st, st, 0.0) == _lib.E_BADARG
+  assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 128, st, st, st, st, float("nan")) == _lib.E_BADARG
+  assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 64, st, st, st, st, 0.1) == _lib.E_UNSUPPORTED
+  assert f(None, odd, fake, fake, fake, None, 1, 4, 8, 8, 128, st, st, st, st, 0.1) == _lib.E_ALIGN
+  assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 128, _st(0, 516, 129), st, st, st, 0.1) == _lib.E_ALIGN
+  assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 128, None, st, st, st, 0.1) == _lib.E_BADARG
+
+  g = lib.mdattn_norm_rope_fullrow
+  assert g(None, None, None, fake, None, fake, None, None, None, 1, 8, 4, 128, 1e-6, 0, 512, st) == _lib.E_BADARG
+  assert g(None, fake, fake, fake, None, fake, fake, None, None, 1, 8, 4, 128, 1e-6, 0, 512, st) == _lib.E_BADARG  # k_in without k_out
+  assert g(None, fake, None, fake, None, fake, None, fake, None, 1, 8, 4, 128, 1e-6, 0, 512, st) == _lib.E_BADARG  # cos without sin
+  assert g(None, fake, None, fake, None, fake, None, None, None, 1, 8, 80, 128, 1e-6, 0, 10240, st) == _lib.E_UNSUPPORTED  # H*D > 8192
+  assert g(None, fake, None, fake, None, fake, None, None, None, 1, 8, 4, 128, 1e-6, 0, 100, st) == _lib.E_BADARG  # row stride < H*D
+  assert g(None, fake, None, odd, None, fake, None, None, None, 1, 8, 4, 128, 1e-6, 0, 512, st) == _lib.E_ALIGN
+
+  p = lib.mdattn_norm_rope_perhead
+  assert p(None, fake, None, fake, None, fake, None, None, None, 0, None, None, 1, 8, 4, 96, 1e-6, st, st) == _lib.E_UNSUPPORTED
+  assert p(None, fake, None, fake, None, fake, None, None, None, 9, None, None, 1, 8, 4, 128, 1e-6, st, st) == _lib.E_BADARG  # n_txt > S
+  assert p(None, fake, None, fake, None, None, None, None, None, 0, None, None, 1, 8, 4, 128, 1e-6, st, st) == _lib.E_BADARG
+
+  m = lib.mdattn_merge
+  assert m(None, fake, fake, fake, None, 0, 1, 4, 8, 128, st, st) == _lib.E_BADARG
+  assert m(None, fake, fake, fake, fake, 0, 1, 4, 8, 100, st, st) == _lib.E_UNSUPPORTED
+  assert m(None, fake, P(0x1002), fake, fake, 0, 1, 4, 8, 128, st, st) == _lib.E_ALIGN
+
+  assert lib.mdattn_finalize(None, fake, fake, 12) == _lib.E_UNSUPPORTED
+  assert lib.mdattn_finalize(None, fake, None, 16) == _lib.E_BADARG
+  assert lib.mdattn_quant_e4m3(None, fake, fake, fake, 24) == _lib.E_UNSUPPORTED
+  assert lib.mdattn_quant_e4m3(None, fake, fake, None, 32) == _lib.E_BADARG
+  with pytest.raises(_lib.MdattnError, match="mdattn error -1"):
+    _lib.check(_lib.E_BADARG, "unit test")

@@ -1,0 +1,128 @@
+"""Host-side mirror of the reference's attention plug-in surface, tested without a GPU with
+fake kernels -- the way the reference tests its own dispatcher (tests/attention_test.py:292-297
+patches kernels with fakes; tests/ltx2/test_attention_ltx2.py:127 patches KERNEL_REGISTRY)."""
+from unittest import mock
+
+import pytest
+import torch
+
+from maxdiffusion_amd import attention_op as A
+
+
+def _call(q, k, v, kernel, heads=2, dim_head=4, mask=None, min_len=0, causal=False):
+  return A._apply_attention(
+      query=q, key=k, value=v, heads=heads, dim_head=dim_head, split_head_dim=True, float32_qk_product=False,
+      attention_kernel=kernel, flash_min_seq_length=min_len, use_memory_efficient_attention=False, scale=dim_head**-0.5,
+      dtype=torch.bfloat16, mesh=None, axis_names_q=(None,) * 4, axis_names_kv=(None,) * 4, flash_block_sizes=None,
+      dpa_layer=None, attention_mask=mask, is_causal=causal)
+
+
+def test_registry_holds_only_the_hip_kernels():
+  assert set(A.HIP_KERNEL_NAMES) <= set(A.KERNEL_REGISTRY)
+  assert "dot_product" not in A.KERNEL_REGISTRY  # no CPU implementation ships in the product
+  for name in A.HIP_KERNEL_NAMES:  # substrings the reference's config layer keys on
+    assert not any(s in name for s in ("ring", "ulysses", "custom", "tokamax"))
+
+
+def test_unknown_kernel_raises_value_error_like_the_reference():
+  q = torch.zeros(1, 8, 8)
+  with pytest.raises(ValueError, match="Unexpected attention kernel"):
+    _call(q, q, q, "no_such_kernel")
+  with pytest.raises(ValueError, match="Unexpected attention kernel"):
+    _call(q, q, q, "dot_product")  # the reference's CPU path is not part of this package
+
+
+def test_dispatch_passes_the_reference_context_keys():
+  seen = {}
+
+  def fake(q, k, v, context):
+    seen.update(context)
+    return q
+
+  q = torch.zeros(1, 8, 8)
+  with mock.patch.dict(A.KERNEL_REGISTRY, {"fake": fake}):
+    out = _call(q, q, q, "fake")
+  assert out is q
+  assert set(seen) == {
+      "heads", "mesh", "axis_names_q", "axis_names_kv", "flash_block_sizes", "dtype", "mask_padding_tokens",
+      "residual_checkpoint_name", "attention_mask", "scale", "use_base2_exp", "use_experimental_scheduler",
+      "ulysses_shards", "ulysses_attention_chunks", "dim_head", "split_head_dim", "float32_qk_product",
+      "use_memory_efficient_attention", "dpa_layer", "is_causal"}
+  assert seen["heads"] == 2 and seen["scale"] == 0.5 and seen["attention_mask"] is None
+
+
+def test_flash_min_length_gate_only_demotes_the_listed_names():
+  calls = []
+  q = torch.zeros(1, 4, 8)
+  with mock.patch.dict(A.KERNEL_REGISTRY, {"flash": lambda *a: calls.append("flash"), "dot_product": lambda *a: calls.append("dot"),
+                                          "hip_flash": lambda *a: calls.append("hip")}):
+    _call(q, q, q, "flash", min_len=8)  # short sequence: the reference falls back to dot_product
+    _call(q, q, q, "flash", min_len=2)
+    _call(q, q, q, "hip_flash", min_len=8)  # not in the gated list: never demoted
+  assert calls == ["dot", "flash", "hip"]
+
+
+def test_input_checks_and_mask_contract():
+  q = torch.zeros(1, 8, 8)
+  # the reference's checks index from the right (attention_flax.py:99-106): axis -2, then axis -3
+  with pytest.raises(AssertionError, match="num_kv_heads must match"):
+    _call(q, torch.zeros(1, 6, 8), torch.zeros(1, 7, 8), "hip_flash")
+  with pytest.raises(AssertionError, match="lengths must match"):
+    _call(torch.zeros(1, 2, 8, 4), torch.zeros(1, 2, 8, 4), torch.zeros(1, 3, 8, 4), "hip_flash")
+  with pytest.raises(AssertionError, match="depths must match"):
+    _call(q, torch.zeros(1, 8, 16), torch.zeros(1, 8, 16), "hip_flash")
+  with pytest.raises(ValueError, match=r"attention_mask must have shape \[batch, kv_length\]"):
+    _call(q, q, q, "hip_flash", mask=torch.ones(1, 1, 8))
+  got = {}
+  with mock.patch.dict(A.KERNEL_REGISTRY, {"fake": lambda q, k, v, c: got.update(c) or q}):
+    _call(q, q, q, "fake", mask=torch.tensor([[1, 0, 1, 1, 0, 0, 1, 1]]))
+  assert got["attention_mask"].dtype == torch.bool  # canonical [B, K] keep mask reaches the kernel
+  with pytest.raises(NotImplementedError, match="attention_mask"):
+    _call(q, q, q, "hip_flash", mask=torch.ones(1, 8, dtype=torch.bool))
+  with pytest.raises(NotImplementedError, match="non-causal"):
+    _call(q, q, q, "hip_flash", causal=True)
+
+
+def test_layout_views_are_zero_copy():
+  x3 = torch.arange(2 * 6 * 8, dtype=torch.float32).reshape(2, 6, 8)
+  v = A._as_bshd(x3, heads=2)
+  assert v.shape == (2, 6, 2, 4) and v.data_ptr() == x3.data_ptr()
+  x4 = torch.arange(2 * 2 * 6 * 4, dtype=torch.float32).reshape(2, 2, 6, 4)  # [B,H,S,D]
+  v4 = A._as_bshd(x4, heads=2)
+  assert v4.shape == (2, 6, 2, 4) and v4.data_ptr() == x4.data_ptr() and v4.stride() == (48, 4, 24, 1)
+  assert torch.equal(v4[1, 3, 1], x4[1, 1, 3])
+  with pytest.raises(ValueError, match="not divisible"):
+    A._as_bshd(torch.zeros(1, 4, 10), heads=4)
+
+
+def test_rotary_table_forms_are_equivalent():
+  import numpy as np
+
+  import oracle as O
+
+  cos, sin = O.wan_rope_table((2, 3, 4), 128)
+  cplx = torch.from_numpy(O.wan_rope_table_complex((2, 3, 4), 128))
+  c1, s1 = A._split_table(cplx, 24, 128)
+  assert torch.equal(c1, torch.from_numpy(cos)) and torch.equal(s1, torch.from_numpy(sin))
+  ids = O.flux_ids(3, 4, 4)
+  fc, fs = O.flux_rope_table(ids)
+  mat = torch.from_numpy(O.flux_rope_table_matrix(ids))
+  c2, s2 = A._split_table(mat, 19, 128)
+  assert torch.equal(c2, torch.from_numpy(fc)) and torch.equal(s2, torch.from_numpy(fs))
+  rep = (torch.from_numpy(np.repeat(fc, 2, axis=1)), torch.from_numpy(np.repeat(fs, 2, axis=1)))  # return_tuple form
+  c3, s3 = A._split_table(rep, 19, 128)
+  assert torch.equal(c3, c2) and torch.equal(s3, s2)
+  assert A._split_table(None, 19, 128) == (None, None)
+
+
+def test_cpu_tensors_are_refused_not_computed():
+  q = torch.zeros(1, 8, 2 * 128, dtype=torch.bfloat16)
+  with pytest.raises(ValueError, match="no CPU path"):
+    _call(q, q, q, "hip_flash", heads=2, dim_head=128)
+
+
+def test_attention_op_mirrors_constructor_and_call():
+  op = A.AttentionOp(mesh=None, attention_kernel="fake", scale=0.5, heads=2, dim_head=4, dtype=torch.bfloat16)
+  q = torch.zeros(1, 8, 8)
+  with mock.patch.dict(A.KERNEL_REGISTRY, {"fake": lambda q, k, v, c: (c["scale"], c["heads"])}):
+    assert op.apply_attention(q, q, q) == (0.5, 2)

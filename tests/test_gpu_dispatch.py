@@ -1,0 +1,81 @@
+"""`hip_flash` behind the reference-shaped dispatcher: rank-3 and rank-4 inputs, cross-attention,
+compared with a restated `dot_product` registered by the test (the reference's own integration
+test compares flash against dot_product the same way, tests/attention_test.py:90-147)."""
+from unittest import mock
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from helpers import err_stats, rel_l2, to_dev_bf16, to_np
+from maxdiffusion_amd import attention_op as A
+
+pytestmark = pytest.mark.gpu
+
+
+def _dot_product_oracle(q, k, v, context):
+  """Test-only registry entry: the bf16 dtype flow of _apply_attention_dot on the CPU."""
+  h = context["heads"]
+  to_hsd = lambda t: np.ascontiguousarray(to_np(A._as_bshd(t, h))[0].transpose(1, 0, 2))
+  out = O.attention_dot_product_bf16(to_hsd(q), to_hsd(k), to_hsd(v), context["scale"])
+  return torch.from_numpy(out.transpose(1, 0, 2).reshape(1, out.shape[1], -1)).to(q.device).to(q.dtype)
+
+
+def _op(kernel, heads):
+  return A.AttentionOp(mesh=None, attention_kernel=kernel, scale=128**-0.5, heads=heads, dim_head=128, dtype=torch.bfloat16,
+                       float32_qk_product=False, split_head_dim=False)
+
+
+def test_hip_flash_matches_dot_product_rank3_rank4_and_cross(dev):
+  H, S, T = 10, 1024, 77
+  q, k, v = (O.normal_bf16((1, S, H * 128), s) for s in (0, 1, 2))
+  kt, vt = O.normal_bf16((1, T, H * 128), 5), O.normal_bf16((1, T, H * 128), 6)
+  qd, kd, vd, ktd, vtd = (to_dev_bf16(x, dev) for x in (q, k, v, kt, vt))
+  with mock.patch.dict(A.KERNEL_REGISTRY, {"dot_product": _dot_product_oracle}):
+    for name, args in (("self rank-3", (qd, kd, vd)), ("cross rank-3", (qd, ktd, vtd))):
+      got = _op("hip_flash", H).apply_attention(*args)
+      want = _op("dot_product", H).apply_attention(*args)
+      assert got.shape == (1, S, H * 128) and got.dtype == torch.bfloat16
+      mx, mean = err_stats(to_np(got), to_np(want))
+      print(f"{name}: max-abs {mx:.3e} mean-abs {mean:.3e}")
+      assert mx <= 2e-2 and mean <= 2e-3 and rel_l2(to_np(got), to_np(want)) <= 3e-2
+      if name.startswith("self"):  # the reference's own criterion for self-attention (attention_test.py:147)
+        diff_norm = float((got.float() - want.float()).norm())
+        assert diff_norm < 1.0, diff_norm
+    # rank-4 [B,H,S,D] inputs, the layout Wan self-attention hands over after rope (attention_flax.py:2673-2684)
+    to4 = lambda t: t.view(1, -1, H, 128).permute(0, 2, 1, 3).contiguous()
+    got4 = _op("hip_flash", H).apply_attention(to4(qd), to4(kd), to4(vd))
+    got3 = _op("hip_flash", H).apply_attention(qd, kd, vd)
+    assert got4.shape == (1, S, H * 128) and torch.equal(got4, got3)
+
+
+def test_f32_inputs_are_accepted_and_returned_in_f32(dev):
+  # LTX2 passes f32 q/k (attention_ltx2.py:415-432); the result must come back in q's dtype
+  H, S = 2, 128
+  q, k, v = (to_dev_bf16(O.normal_bf16((1, S, H * 128), s), dev).float() for s in (0, 1, 2))
+  got = _op("hip_flash", H).apply_attention(q, k, v)
+  assert got.dtype == torch.float32
+  want = _op("hip_flash", H).apply_attention(q.bfloat16(), k.bfloat16(), v.bfloat16())
+  assert torch.equal(got, want.float())
+
+
+def test_fused_prologue_feeds_attention_without_transposes(dev):
+  # Wan block order: norm_q/norm_k over H*D -> rope -> attention (attention_flax.py:2655-2684), then the
+  # cross-attention with norm only (:2671); compared with the un-fused oracle chain.
+  w = O.WORKLOADS["wan1.3b"]
+  H, S = w.heads, 3 * 10 * 13
+  cos, sin = O.wan_rope_table((3, 10, 13), 128)
+  q, k, v = (O.normal_bf16((1, S, H * 128), s) for s in (0, 1, 2))
+  wq, wk = O.norm_weight(H * 128, 3), O.norm_weight(H * 128, 4)
+  table = torch.from_numpy(O.wan_rope_table_complex((3, 10, 13), 128)).to(dev)  # complex64 [1,1,S,64], as the model passes it
+  qn, kn = A.hip_norm_rope(to_dev_bf16(q, dev), to_dev_bf16(k, dev), to_dev_bf16(wq, dev), to_dev_bf16(wk, dev), table, H, out_layout="bhsd")
+  out = _op("hip_flash", H).apply_attention(qn.permute(0, 2, 1, 3), kn.permute(0, 2, 1, 3), to_dev_bf16(v, dev).view(1, S, H, 128).permute(0, 2, 1, 3))
+  qe, ke = O.norm_rope_fullrow(q, wq, cos, sin, H), O.norm_rope_fullrow(k, wk, cos, sin, H)
+  ro, _ = O.attention(qe[0].transpose(1, 0, 2), ke[0].transpose(1, 0, 2), v.reshape(S, H, 128).transpose(1, 0, 2), w.scale)
+  got = to_np(out).reshape(S, H, 128).transpose(1, 0, 2)
+  mx, mean = err_stats(got, ro)
+  assert mx <= 2e-2 and mean <= 2e-3 and rel_l2(got, ro) <= 1.5e-2
+  qc, none = A.hip_norm_rope(to_dev_bf16(q, dev), None, to_dev_bf16(wq, dev), None, None, H)  # cross-attention: norm only
+  assert none is None
+  assert err_stats(to_np(qc), O.norm_rope_fullrow(q, wq, None, None, H))[0] <= 1.6e-2

@@ -1,0 +1,96 @@
+"""Chunk merge + ring replay on the device against the oracle (BASELINE configs[3])."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from helpers import bits_to_dev, err_stats, golden, hsd, rel_l2, to_dev_bf16, to_np, torch_attention_f32
+from maxdiffusion_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def test_golden_merge(dev):
+  g = golden("merge_small.npz")
+  o_run, l_run = ops.new_merge_state(1, 70, 2, 128, dev)
+  for ob, lb in zip(g["parts_o"], g["parts_l"]):
+    ops.merge_partial(o_run, l_run, bits_to_dev(ob, dev), torch.from_numpy(lb).to(dev))
+  assert err_stats(to_np(o_run), g["o_merged"])[0] < 1e-6
+  assert err_stats(to_np(l_run), g["lse_merged"])[0] < 1e-5
+  fin = ops.finalize(o_run)
+  assert fin.dtype == torch.bfloat16
+  assert torch.equal(fin, o_run.to(torch.bfloat16))  # round-to-nearest-even cast
+
+
+def test_merge_f32_partials_layouts_and_neutral_element(dev):
+  rng = np.random.default_rng(0)
+  B, S, H, D = 2, 33, 3, 128
+  o1, o2 = rng.standard_normal((B, S, H, D)).astype(np.float32), rng.standard_normal((B, S, H, D)).astype(np.float32)
+  l1, l2 = (rng.standard_normal((B, H, S)) * 4).astype(np.float32), (rng.standard_normal((B, H, S)) * 4).astype(np.float32)
+  want_o, want_l = O.merge_lse(o1.transpose(0, 2, 1, 3), l1, o2.transpose(0, 2, 1, 3), l2)
+  for layout in ("bshd", "bhsd"):
+    o_run, l_run = ops.new_merge_state(B, S, H, D, dev, layout=layout)
+    ops.merge_partial(o_run, l_run, torch.from_numpy(o1).to(dev), torch.from_numpy(l1).to(dev))  # into the neutral element
+    assert err_stats(to_np(o_run), o1)[0] < 1e-6 and err_stats(to_np(l_run), l1)[0] < 1e-6
+    cur = torch.from_numpy(o2).to(dev).permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)  # a [B,H,S,D] partial
+    ops.merge_partial(o_run, l_run, cur, torch.from_numpy(l2).to(dev))
+    assert err_stats(to_np(o_run), want_o.transpose(0, 2, 1, 3))[0] < 2e-6
+    assert err_stats(to_np(l_run), want_l)[0] < 2e-6
+  # an empty partial (lse = -inf) leaves the state untouched; two empty states stay empty with out = 0
+  o_run, l_run = ops.new_merge_state(1, 8, 1, 128, dev)
+  o_run.fill_(1.5); l_run.fill_(0.25)
+  ops.merge_partial(o_run, l_run, torch.zeros_like(o_run), torch.full_like(l_run, float("-inf")))
+  assert float((o_run - 1.5).abs().max()) == 0 and float((l_run - 0.25).abs().max()) == 0
+  l_run.fill_(float("-inf"))
+  ops.merge_partial(o_run, l_run, torch.ones_like(o_run), torch.full_like(l_run, float("-inf")))
+  assert float(o_run.abs().max()) == 0 and bool(torch.isneginf(l_run).all())
+
+
+def test_ring_replay_small_unequal_chunks(dev):
+  # tests/ring_fixed_m_test.py:156-189 (2 x 2048 shards) and its ragged-tail case :173-180, re-expressed on one GPU
+  H = 5
+  q = O.normal_bf16((1, 300, H, 128), 0)
+  sizes = [2048, 2048, 1, 63, 777]
+  ks = [O.normal_bf16((1, n, H, 128), 10 + i) for i, n in enumerate(sizes)]
+  vs = [O.normal_bf16((1, n, H, 128), 20 + i) for i, n in enumerate(sizes)]
+  o_run, l_run = ops.new_merge_state(1, 300, H, 128, dev)
+  qd = to_dev_bf16(q, dev)
+  for kc, vc in zip(ks, vs):
+    o, l = ops.flash_attention(qd, to_dev_bf16(kc, dev), to_dev_bf16(vc, dev), return_lse=True)
+    ops.merge_partial(o_run, l_run, o, l)
+  ro, rl = O.attention(hsd(q), hsd(np.concatenate(ks, 1)), hsd(np.concatenate(vs, 1)), 128**-0.5)
+  out = to_np(ops.finalize(o_run))
+  mx, mean = err_stats(hsd(out), ro)
+  print(f"ring small: max-abs {mx:.3e} mean-abs {mean:.3e}")
+  assert mx < 2e-2 and mean < 2e-3 and rel_l2(hsd(out), ro) < 1.5e-2
+  assert err_stats(to_np(l_run)[0], rl)[0] < 1e-3
+
+
+def test_wan14b_ring_shard_replay_full_size(dev):
+  """Config 3: a 9 450-token Q chunk x 40 heads against 8 successive 9 450-token KV chunks; the merged
+  result must equal full 75 600-token attention for that Q chunk."""
+  w = O.WORKLOADS["wan14b-ring"]
+  C, n = w.seq, w.ring_chunks
+  gen = torch.Generator(device=dev).manual_seed(3)
+  mk = lambda s: torch.randn((1, s, w.heads, 128), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+  q, k, v = mk(C), mk(C * n), mk(C * n)
+  o_run, l_run = ops.new_merge_state(1, C, w.heads, 128, dev)
+  for i in range(n):
+    o, l = ops.flash_attention(q, k[:, i * C:(i + 1) * C], v[:, i * C:(i + 1) * C], scale=w.scale, return_lse=True)
+    ops.merge_partial(o_run, l_run, o, l)
+  merged = ops.finalize(o_run)
+  full, full_l = ops.flash_attention(q, k, v, scale=w.scale, return_lse=True)  # one pass over all 75 600 keys
+  assert float((merged.float() - full.float()).abs().max()) < 2e-3
+  assert float((l_run - full_l).abs().max()) < 1e-4
+  for h0 in range(0, w.heads, 8):  # and both against the torch f32 reference on the whole chunk
+    ro, rl = torch_attention_f32(q[:, :, h0:h0 + 8], k[:, :, h0:h0 + 8], v[:, :, h0:h0 + 8], w.scale, q_block=1024)
+    d = (merged[:, :, h0:h0 + 8].float() - ro).abs()
+    assert float(d.max()) <= 2e-2 and float(d.mean()) <= 2e-3
+    assert float((merged[:, :, h0:h0 + 8].float() - ro).norm() / ro.norm()) <= 1.5e-2
+    assert float((l_run[:, h0:h0 + 8] - rl).abs().max()) <= 1e-3
+  rows = O.sample_rows(C, n_random=24)
+  idx = torch.from_numpy(rows).to(dev)
+  for h in (0, 21, 39):  # CPU oracle on sampled rows
+    co, cl = O.attention_rows(to_np(q[0, idx, h]), to_np(k[0, :, h]), to_np(v[0, :, h]), w.scale)
+    assert err_stats(to_np(merged[0, idx, h]), co)[0] <= 2e-2 and rel_l2(to_np(merged[0, idx, h]), co) <= 1.5e-2
+    assert err_stats(to_np(l_run[0, h, idx]), cl)[0] <= 1e-3
