@@ -1,0 +1,163 @@
+"""Benchmark of the DiT attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload wan14b|wan14b-ring|wan1.3b|flux-dev]
+
+One step = one pass of the path over one synthetic batch already resident in HBM: fused q/k
+RMSNorm + RoPE, then the bf16 self-attention forward (with LSE).  Prints ONE JSON line:
+`value` is attention TFLOP/s over the whole step (4*B*H*Sq*Skv*D FLOP / step time); `roofline`
+is the attention kernel alone, timed with events on the launch stream; `roofline_norm_rope` is the
+prologue kernel against HBM peak; `cpu_baseline` is the oracle's restatement of the reference's
+`dot_product` path timed on the host cores over a bounded slice of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
+
+
+def cpu_baseline(workload, budget_rows: int):
+  """The oracle's bf16-flow `dot_product` (attention_flax.py:1487-1567 restated in numpy), one head,
+  one block of query rows against every key of the workload, on the host cores."""
+  import numpy as np
+
+  import oracle as O
+
+  rows = min(budget_rows, workload.seq)
+  q = O.normal_bf16((1, rows, 128), 0)
+  k = O.normal_bf16((1, workload.kv_seq, 128), 1)
+  v = O.normal_bf16((1, workload.kv_seq, 128), 2)
+  O.attention_dot_product_bf16(q[:, :64], k[:, :1024], v[:, :1024], workload.scale)  # first call untimed
+  t0 = time.perf_counter()
+  O.attention_dot_product_bf16(q, k, v, workload.scale)
+  dt = time.perf_counter() - t0
+  flops = O.attention_flops(1, 1, rows, workload.kv_seq, 128)
+  cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or os.cpu_count()
+  return {
+      "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+      "sample": f"1 head x {rows} query rows x {workload.kv_seq} keys (of {workload.heads} heads x {workload.seq} rows), "
+                f"numpy restatement of dot_product with bf16 score/prob rounding, {dt:.2f} s; not JAX (absent from the image)",
+  }
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=10)
+  ap.add_argument("--warmup", type=int, default=3)
+  ap.add_argument("--workload", default="wan14b")
+  ap.add_argument("--cpu-rows", type=int, default=2048, help="query rows of the CPU-baseline slice (0: skip)")
+  args = ap.parse_args()
+  if args.gpus != 1:
+    print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+    sys.exit(2)
+
+  import torch
+
+  import oracle as O
+  from maxdiffusion_amd import _lib, ops
+  from maxdiffusion_amd.build import LIB_PATH, build_library
+
+  if not os.path.exists(LIB_PATH):
+    build_library()
+  _lib.load()
+  if not torch.cuda.is_available():
+    raise RuntimeError("bench.py needs a GPU: the hot path has no CPU implementation")
+  dev = torch.device("cuda:0")
+  w = O.WORKLOADS[args.workload]
+  H, D, S, Skv = w.heads, w.head_dim, w.seq, w.kv_seq
+  ring = max(w.ring_chunks, 1)
+
+  gen = torch.Generator(device=dev).manual_seed(0)
+  randn = lambda *shape: torch.randn(shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+  tb = lambda x: torch.from_numpy(O.to_bf16_bits(x).view("int16")).view(torch.bfloat16).to(dev)
+  # pre-norm projections q, k [1,S,H*D] and v, N(0,1) in bf16; norm weights 1 + 0.1 N(0,1)
+  q_in, k_in = randn(1, S, H * D), randn(1, S, H * D)
+  v = randn(1, Skv * ring, H, D)
+  k_extra = randn(1, Skv * (ring - 1), H, D) if ring > 1 else None
+  if w.norm == "fullrow":
+    wq, wk = tb(O.norm_weight(H * D, 3)), tb(O.norm_weight(H * D, 4))
+    # a ring shard owns the first S tokens of the full latent grid
+    cos, sin = (torch.from_numpy(t[:S].copy()).to(dev) for t in O.wan_rope_table(w.grid, D))
+    prologue = lambda: ops.norm_rope_fullrow(q_in, k_in, wq, wk, cos, sin, H)
+  else:
+    wq, wk = tb(O.norm_weight(D, 3)), tb(O.norm_weight(D, 4))
+    cos, sin = (torch.from_numpy(t).to(dev) for t in O.flux_rope_table(O.flux_ids(*w.grid)))
+    q4, k4 = q_in.view(1, S, H, D), k_in.view(1, S, H, D)
+    prologue = lambda: ops.norm_rope_perhead(q4, k4, wq, wk, cos, sin)
+
+  ev = lambda: torch.cuda.Event(enable_timing=True)
+  t_pro, t_att = [], []
+
+  def step(record: bool):
+    e0, e1, e2 = ev(), ev(), ev()
+    e0.record()
+    qn, kn = prologue()
+    e1.record()
+    if ring == 1:
+      ops.flash_attention(qn, kn, v, scale=w.scale, return_lse=True)
+    else:  # one ring shard: this Q chunk against `ring` successive KV chunks, merged in LSE space
+      o_run, l_run = ops.new_merge_state(1, S, H, D, dev)
+      for i in range(ring):
+        kc = kn if i == 0 else k_extra[:, (i - 1) * Skv:i * Skv]
+        o, l = ops.flash_attention(qn, kc, v[:, i * Skv:(i + 1) * Skv], scale=w.scale, return_lse=True)
+        ops.merge_partial(o_run, l_run, o, l)
+      ops.finalize(o_run)
+    e2.record()
+    if record:
+      torch.cuda.synchronize()
+      t_pro.append(e0.elapsed_time(e1))
+      t_att.append(e1.elapsed_time(e2))
+
+  for _ in range(args.warmup):
+    step(False)
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(args.steps):
+    step(True)
+  torch.cuda.synchronize()
+  ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+  flops = O.attention_flops(1, H, S, Skv * ring, D)
+  att_ms = sum(t_att) / len(t_att)
+  pro_ms = sum(t_pro) / len(t_pro)
+  nr_bytes = O.normrope_bytes(1, S, H, D, with_table=True)
+  achieved = flops / (att_ms * 1e-3) / 1e12
+  out = {
+      "metric": "self-attn TFLOP/s at Wan-14B 75.6k tokens (bf16); norm-RoPE GB/s" if args.workload == "wan14b"
+      else f"self-attn TFLOP/s ({args.workload}); norm-RoPE GB/s",
+      "value": flops / (ms_per_step * 1e-3) / 1e12,
+      "unit": "TFLOP/s",
+      "n_gpus": 1,
+      "steps": args.steps,
+      "warmup": args.warmup,
+      "ms_per_step": ms_per_step,
+      "higher_is_better": True,
+      "scaling": "weak",
+      "vs_baseline": None,
+      "dtype": "bf16",
+      "data": "synthetic",
+      "config": {"workload": f"{args.workload}: B=1 H={H} D={D} Sq={S} Skv={Skv * ring} norm={w.norm} rope={w.rope}"
+                             + (f" ring_chunks={ring} (merge per chunk)" if ring > 1 else ""),
+                 "step": "fused q/k RMSNorm+RoPE -> bf16 flash-attention forward with LSE"},
+      "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                   "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "attn_fwd_bf16_kernel",
+                   "kernel_ms": att_ms, "flop_per_launch": flops / ring},
+      "roofline_norm_rope": {"bound": "hbm", "achieved": nr_bytes / (pro_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                             "frac": nr_bytes / (pro_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "traffic": None,
+                             "kernel": f"norm_rope_{w.norm}_kernel", "kernel_ms": pro_ms, "bytes_per_launch": nr_bytes},
+  }
+  if args.cpu_rows > 0:
+    out["cpu_baseline"] = cpu_baseline(w, args.cpu_rows)
+  print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+  main()

@@ -16,12 +16,15 @@ INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "libmdattn.so")
 FFI_LIB_PATH = os.path.join(PKG_DIR, "libmdattn_ffi.so")
 
-SOURCES = ["mdattn_api.hip", "norm_rope.hip", "attn_fwd_bf16.hip", "attn_fwd_fp8.hip", "merge_quant.hip"]
+SOURCES = ["mdattn_api.hip", "norm_rope.hip", "attn_fwd_bf16.hip", "attn_fwd_bf16_pipe.hip", "attn_fwd_fp8.hip", "merge_quant.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32 out of scalar float code.
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results that the vector ALU reads next (attention logits) stay in architectural VGPRs
+    # instead of bouncing through AGPRs with v_accvgpr_read/write
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
 ]
 

@@ -18,24 +18,12 @@
 //                share it through that XCD's L2.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "mdattn_common.h"
 
 namespace mdattn {
 
-struct AttnArgs {
-  const __bf16* q;
-  const __bf16* k;
-  const __bf16* v;
-  __bf16* out;
-  float* lse;
-  int H, Sq, Skv;
-  int nqt, total, chunk;
-  int64_t q_sb, q_ss, q_sh;
-  int64_t k_sb, k_ss, k_sh;
-  int64_t v_sb, v_ss, v_sh;
-  int64_t o_sb, o_ss, o_sh;
-  float c;  // scale * log2(e)
-};
 
 constexpr int kBN = 64;          // keys per tile
 constexpr int kD = 128;          // head dim
@@ -43,6 +31,7 @@ constexpr int kKStr = kD + 8;    // K row stride in LDS (272 B: 16 rows x 16 B h
 constexpr int kVStr = kD + 32;   // V row stride in LDS (320 B: 4 rows x 64 B hit 64 distinct banks)
 constexpr int kStage = kBN * kKStr + kBN * kVStr;  // elements per stage
 constexpr int kLdsBytes = 2 * kStage * 2;
+constexpr float kLazy = 8.0f;      // log2 units a row max may lag behind before accumulators are rescaled
 
 typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
@@ -55,7 +44,8 @@ __device__ __forceinline__ bf16x8 read_vt(const __bf16* p0, const __bf16* p1) {
 }
 
 template <int QB, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(QB == 1 ? 2 : 1, QB == 1 ? 2 : 1)))
+void attn_fwd_bf16_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
   constexpr int NT = NW * 64;
@@ -78,7 +68,18 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   const int nt = (a.Skv + kBN - 1) / kBN;
   const float c = a.c;
 
-  // ---- stage tile 0 while the Q fragments load
+  // ---- Q fragments (B operand of K.Q^T), kept in registers for the whole kernel
+  bf16x8 qf[QB][8];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    int row = q0 + qb * 32 + l32;
+    row = row < a.Sq ? row : a.Sq - 1;
+    const __bf16* p = qp + (int64_t)row * a.q_ss + hh * 8;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) qf[qb][s] = *reinterpret_cast<const bf16x8*>(p + s * 16);
+  }
+
+  // ---- stage tile 0
   u32x4 kr[LPT], vr[LPT];
 #define MDATTN_GLOAD(IT)                                                                       \
   _Pragma("unroll") for (int i = 0; i < LPT; ++i) {                                            \
@@ -100,17 +101,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
       *reinterpret_cast<u32x4*>(Vs_ + row * kVStr + cc * 8) = vr[i];                           \
     }                                                                                          \
   }
-  MDATTN_GLOAD(0)
-
-  bf16x8 qf[QB][8];
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    int row = q0 + qb * 32 + l32;
-    row = row < a.Sq ? row : a.Sq - 1;
-    const __bf16* p = qp + (int64_t)row * a.q_ss + hh * 8;
-#pragma unroll
-    for (int s = 0; s < 8; ++s) qf[qb][s] = *reinterpret_cast<const bf16x8*>(p + s * 16);
-  }
+  MDATTN_GLOAD(0)  // issued after the Q loads: waiting for tile 0 then also completes them
 
   f32x16 O[QB][4];
   float m[QB], l[QB];
@@ -124,6 +115,9 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
       for (int i = 0; i < 16; ++i) O[qb][db][i] = 0.f;
   }
 
+  // every global load issued so far (Q fragments, tile 0) completes here: the loop starts with no
+  // vector-memory operation pending, so its own prefetches are never waited on early
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   MDATTN_LSTORE(0)
   __syncthreads();
 
@@ -131,7 +125,10 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   const int k_off = l32 * kKStr + hh * 8;
   const int v_off = (4 * hh + ((lane & 15) >> 2)) * kVStr + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
 
-  for (int it = 0; it < nt; ++it) {
+  // One KV tile.  MASK is set only for the last tile of a ragged key axis, so the main loop carries
+  // no per-element compare/select.
+  auto tile = [&](int it, auto mask_tag) {
+    constexpr bool MASK = decltype(mask_tag)::value;
     const int stage = it & 1;
     const bool more = it + 1 < nt;
     if (more) { MDATTN_GLOAD(it + 1) }
@@ -139,7 +136,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
     const __bf16* Ks = smem + stage * kStage;
     const __bf16* Vs = Ks + kBN * kKStr;
 
-    // ---- S^T = K Q^T
+    // ---- S^T = K Q^T; accumulators alternate so that consecutive MFMAs are independent
     f32x16 S[QB][2];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb)
@@ -147,19 +144,32 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
       for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) S[qb][jb][i] = 0.f;
+    // all K fragments are requested before the first MFMA so that LDS latency is paid once per tile
+    bf16x8 kf[2][8];
 #pragma unroll
-    for (int jb = 0; jb < 2; ++jb) {
+    for (int s = 0; s < 8; ++s)
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + jb * 32 * kKStr + k_off + s * 16);
+      for (int jb = 0; jb < 2; ++jb) kf[jb][s] = *reinterpret_cast<const bf16x8*>(Ks + jb * 32 * kKStr + k_off + s * 16);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+#pragma unroll
+      for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb)
-          S[qb][jb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][s], S[qb][jb], 0, 0, 0);
+          S[qb][jb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jb][s], qf[qb][s], S[qb][jb], 0, 0, 0);
+    // V^T fragments for the PV product are requested now and land while the softmax runs
+    bf16x8 vf[4][4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+        const __bf16* p0 = Vs + v_off + ks * 16 * kVStr + db * 32;
+        vf[ks][db] = read_vt(p0, p0 + 8 * kVStr);
       }
-    }
+    __builtin_amdgcn_sched_barrier(0);
 
-    // ---- ragged tail of the key axis: only the last tile can hold invalid keys
-    if (!more && (a.Skv & (kBN - 1)) != 0) {
+    if (MASK) {
       const int kv_base = it * kBN + 4 * hh;
 #pragma unroll
       for (int jb = 0; jb < 2; ++jb)
@@ -183,10 +193,20 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, S[qb][jb][i]);
       mloc = xhalf_max(mloc);
-      const float mnew = fmaxf(m[qb], mloc);
-      const float alpha = __builtin_amdgcn_exp2f((m[qb] - mnew) * c);
-      const float mc = mnew * c;
-      m[qb] = mnew;
+      // Lazy rescale: the running max only moves when some row of this wave would otherwise see
+      // exp2 arguments above kLazy (P <= 2^kLazy stays exact enough in bf16/f32); with a stale max
+      // the accumulators need no multiply.  The branch is wave-uniform.
+      if (__builtin_amdgcn_ballot_w64((mloc - m[qb]) * c > kLazy) != 0) {
+        const float mnew = fmaxf(m[qb], mloc);
+        const float alpha = __builtin_amdgcn_exp2f((m[qb] - mnew) * c);
+        m[qb] = mnew;
+        l[qb] *= alpha;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) O[qb][db][i] *= alpha;
+      }
+      const float mc = m[qb] * c;
       float lsum = 0.f;
 #pragma unroll
       for (int jb = 0; jb < 2; ++jb) {
@@ -201,29 +221,28 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
           P[qb][2 * jb + j] = __builtin_bit_cast(bf16x8, pack8(p));
         }
       }
-      l[qb] = l[qb] * alpha + lsum;
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) O[qb][db][i] *= alpha;
+      l[qb] += lsum;
     }
 
     // ---- O^T += V^T P^T
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
+    for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        const __bf16* p0 = Vs + v_off + ks * 16 * kVStr + db * 32;
-        const bf16x8 vf = read_vt(p0, p0 + 8 * kVStr);
+      for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb)
-          O[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P[qb][ks], O[qb][db], 0, 0, 0);
-      }
-    }
+          O[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[ks][db], P[qb][ks], O[qb][db], 0, 0, 0);
 
     if (more) MDATTN_LSTORE(stage ^ 1)
     __syncthreads();
-  }
+  };
+
+  if (a.prio == 1 && NW == 8 && wave < 4) __builtin_amdgcn_s_setprio(2);
+  if (a.prio == 2 && NW == 4 && ((blockIdx.x >> 3) & 1)) __builtin_amdgcn_s_setprio(2);
+  const int nfull = a.Skv / kBN;  // tiles with 64 valid keys
+  for (int it = 0; it < nfull; ++it) tile(it, std::false_type{});
+  if (nfull < nt) tile(nfull, std::true_type{});
 
   // ---- epilogue: normalise, convert, store; lse = m*scale + ln(l)
   __bf16* op = a.out + b * a.o_sb + h * a.o_sh;
@@ -289,20 +308,25 @@ extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const
   a.v_sb = v_strides->batch; a.v_ss = v_strides->seq; a.v_sh = v_strides->head;
   a.o_sb = o_strides->batch; a.o_ss = o_strides->seq; a.o_sh = o_strides->head;
   a.c = scale * kLog2e;
+  a.prio = getenv("MDATTN_PRIO") ? atoi(getenv("MDATTN_PRIO")) : 0;
   hipStream_t st = (hipStream_t)stream;
 
-  // Tile choice: 256 query rows per workgroup (4 waves x 64 rows) halves the LDS traffic per MFMA;
-  // 128-row workgroups fill the chip when there are few (head, q-tile) pairs.
+  // Tile choice.  8 waves x 32 query rows (two waves per SIMD: one wave's softmax overlaps the
+  // other's MFMAs) measures fastest at every size tried; 4 waves x 32 rows gives more workgroups
+  // when there are few (head, q-tile) pairs.  MDATTN_FWD_VARIANT overrides for experiments.
   int variant = 0;
   if (const char* e = getenv("MDATTN_FWD_VARIANT")) variant = atoi(e);
   if (variant == 0) {
     const int64_t wg256 = (int64_t)B * H * ((Sq + 255) / 256);
-    variant = wg256 >= 2 * 256 ? 1 : 2;
+    variant = wg256 >= 256 ? 3 : 2;
   }
   switch (variant) {
     case 1: return launch_fwd<2, 4>(st, a, B);
     case 2: return launch_fwd<1, 4>(st, a, B);
     case 3: return launch_fwd<1, 8>(st, a, B);
+    case 4: return launch_fwd_pipe(st, a, B, 64);
+    case 5: return launch_fwd_pipe(st, a, B, 32);
+    case 6: return launch_fwd_pipe(st, a, B, 0);
     default: return MDATTN_E_BADARG;
   }
 }

@@ -77,6 +77,25 @@ __device__ __forceinline__ void st_nt(uint4* p, const uint4& u) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
 
+// Arguments of the attention-forward kernels (element strides; head_dim contiguous).
+struct AttnArgs {
+  const __bf16* q;
+  const __bf16* k;
+  const __bf16* v;
+  __bf16* out;
+  float* lse;
+  int H, Sq, Skv;
+  int nqt, total, chunk;
+  int64_t q_sb, q_ss, q_sh;
+  int64_t k_sb, k_ss, k_sh;
+  int64_t v_sb, v_ss, v_sh;
+  int64_t o_sb, o_ss, o_sh;
+  float c;  // scale * log2(e)
+  int prio;
+};
+
+int launch_fwd_pipe(hipStream_t st, AttnArgs a, int B, int rows_per_wave);  // attn_fwd_bf16_pipe.hip
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool strides_ok(const mdattn_strides* s, int64_t mult) {
   return s && s->batch % mult == 0 && s->seq % mult == 0 && s->head % mult == 0 && s->seq > 0 && s->head > 0 && s->batch >= 0;
