@@ -91,10 +91,9 @@ struct AttnArgs {
   int64_t v_sb, v_ss, v_sh;
   int64_t o_sb, o_ss, o_sh;
   float c;  // scale * log2(e)
-  int prio;
 };
 
-int launch_fwd_pipe(hipStream_t st, AttnArgs a, int B, int rows_per_wave);  // attn_fwd_bf16_pipe.hip
+
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool strides_ok(const mdattn_strides* s, int64_t mult) {
