@@ -31,12 +31,14 @@ def cpu_baseline(workload, budget_rows: int):
   import oracle as O
 
   rows = min(budget_rows, workload.seq)
+  block = 2048  # query rows per call: bounds the [rows, keys] score matrix to ~0.6 GB in f32
   q = O.normal_bf16((1, rows, 128), 0)
   k = O.normal_bf16((1, workload.kv_seq, 128), 1)
   v = O.normal_bf16((1, workload.kv_seq, 128), 2)
   O.attention_dot_product_bf16(q[:, :64], k[:, :1024], v[:, :1024], workload.scale)  # first call untimed
   t0 = time.perf_counter()
-  O.attention_dot_product_bf16(q, k, v, workload.scale)
+  for r0 in range(0, rows, block):
+    O.attention_dot_product_bf16(q[:, r0:r0 + block], k, v, workload.scale)
   dt = time.perf_counter() - t0
   flops = O.attention_flops(1, 1, rows, workload.kv_seq, 128)
   cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or os.cpu_count()
@@ -53,7 +55,10 @@ def main():
   ap.add_argument("--steps", type=int, default=10)
   ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--workload", default="wan14b")
-  ap.add_argument("--cpu-rows", type=int, default=2048, help="query rows of the CPU-baseline slice (0: skip)")
+  ap.add_argument("--cpu-rows", type=int, default=16384, help="query rows of the CPU-baseline slice (0: skip)")
+  ap.add_argument("--traffic-probe", action="store_true",
+                  help="also launch one 1 GiB device copy: the plain copy kernel of known size that scales rocprofv3's "
+                       "FETCH_SIZE / WRITE_SIZE counters")
   args = ap.parse_args()
   if args.gpus != 1:
     print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -116,6 +121,12 @@ def main():
       t_pro.append(e0.elapsed_time(e1))
       t_att.append(e1.elapsed_time(e2))
 
+  if args.traffic_probe:
+    src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+    dst = torch.empty_like(src)
+    dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+    torch.cuda.synchronize()
+    del src, dst
   for _ in range(args.warmup):
     step(False)
   torch.cuda.synchronize()
@@ -130,8 +141,12 @@ def main():
   pro_ms = sum(t_pro) / len(t_pro)
   nr_bytes = O.normrope_bytes(1, S, H, D, with_table=True)
   achieved = flops / (att_ms * 1e-3) / 1e12
+  traffic = {}
+  tpath = os.path.join(ROOT, "profiles", "traffic.json")
+  if os.path.exists(tpath):  # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command
+    traffic = json.load(open(tpath)).get(args.workload, {})
   out = {
-      "metric": "self-attn TFLOP/s at Wan-14B 75.6k tokens (bf16); norm-RoPE GB/s" if args.workload == "wan14b"
+      "metric": "self-attn TFLOP/s (% bf16 MFMA peak) at Wan-14B 75.6k tokens; norm-RoPE GB/s" if args.workload == "wan14b"
       else f"self-attn TFLOP/s ({args.workload}); norm-RoPE GB/s",
       "value": flops / (ms_per_step * 1e-3) / 1e12,
       "unit": "TFLOP/s",
@@ -148,10 +163,10 @@ def main():
                              + (f" ring_chunks={ring} (merge per chunk)" if ring > 1 else ""),
                  "step": "fused q/k RMSNorm+RoPE -> bf16 flash-attention forward with LSE"},
       "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                   "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "attn_fwd_bf16_kernel",
+                   "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic.get("attn_fwd_bf16_kernel"), "kernel": "attn_fwd_bf16_kernel",
                    "kernel_ms": att_ms, "flop_per_launch": flops / ring},
       "roofline_norm_rope": {"bound": "hbm", "achieved": nr_bytes / (pro_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                             "frac": nr_bytes / (pro_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "traffic": None,
+                             "frac": nr_bytes / (pro_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "traffic": traffic.get(f"norm_rope_{w.norm}_kernel"),
                              "kernel": f"norm_rope_{w.norm}_kernel", "kernel_ms": pro_ms, "bytes_per_launch": nr_bytes},
   }
   if args.cpu_rows > 0:
