@@ -1,12 +1,308 @@
-// fp8-e4m3 attention forward (placeholder until the MFMA kernel lands).
+// Non-causal flash-attention forward for gfx950 (MI355X) on fp8-e4m3 (OCP) operands, head_dim 128.
+//
+// Same decomposition as the bf16 kernel, on v_mfma_f32_32x32x64_f8f6f4 (K = 64 per instruction, twice
+// the bf16 rate):
+//   workgroup  = NW waves x 32 query rows; keys walked in tiles of 64, double-buffered in LDS with the
+//                next tile's global loads in flight in registers.
+//   S^T = K.Q^T  two 32-key blocks per tile, two MFMAs each (d = 0..63, 64..127).  A = K rows from LDS
+//                (row stride 144 B), B = the wave's Q fragment, resident in registers.  A and B use the
+//                same k-slot order, so a lane simply holds 32 contiguous bytes of its row.
+//   softmax      in f32 on the 32 logits a lane holds for its query row; q_scale*k_scale*scale*log2(e)
+//                is folded into the exp2 argument.  P is kept 2^4 above the usual normalisation
+//                (reference point = running max - 4) so that e4m3's normal range [2^-6, 448] covers
+//                probabilities down to 2^-10 of the row max; the reference point only moves when a
+//                new maximum would push P beyond 2^8 (lazy rescale).  The row sum uses the f32 P.
+//   O^T += V^T.P^T  one MFMA per 32-wide slab of d with all 64 keys of the tile as K.  P goes from the
+//                accumulator layout to the B operand by the e4m3 convert alone (operand byte s = value
+//                s%16 of block s/16).  V^T comes from the row-major V tile through ds_read_b64_tr_b8:
+//                within 16 lanes, lane i receives as byte e the element i%8 of the 8-byte chunk whose
+//                address lane 2e + i/8 supplies, so each lane points at one key row and one 8-byte
+//                column chunk, and every lane ends up with 8 keys of its own d.  The V tile has no row
+//                padding (128 B rows); its 8-byte chunks are XOR-swizzled by row bits 1 and 3, which
+//                makes the 8 rows x 32 B a half-wave reads hit 64 distinct banks.
+//   epilogue     O * v_scale / l, bf16; lse = ln2 * (reference + log2 l).
+#include <stdlib.h>
+
+#include <type_traits>
+
 #include "mdattn_common.h"
+
+namespace mdattn {
+namespace {
+
+constexpr int kBN8 = 64;                                  // keys per tile
+constexpr int kD8 = 128;                                  // head dim = bytes per row
+constexpr int kKS8 = kD8 + 16;                            // K row stride in LDS, bytes
+constexpr int kVS8 = kD8;                                 // V row stride in LDS, bytes (swizzled, not padded)
+constexpr int kStage8 = kBN8 * kKS8 + kBN8 * kVS8;        // bytes per LDS stage
+constexpr float kPOff = 4.0f;                             // P = exp2(logit - max + kPOff) at a fresh maximum
+constexpr float kPLazy = 4.0f;                            // extra headroom before the reference point moves
+
+typedef __attribute__((ext_vector_type(2))) int i32x2;
+typedef i32x2 __attribute__((address_space(3))) * lds_i32x2_ptr;
+
+struct Fp8Args {
+  const uint8_t* q;
+  const uint8_t* k;
+  const uint8_t* v;
+  __bf16* out;
+  float* lse;
+  const float* q_scale;
+  const float* k_scale;
+  const float* v_scale;
+  int H, Sq, Skv;
+  int nqt, total, chunk;
+  int64_t q_sb, q_ss, q_sh;
+  int64_t k_sb, k_ss, k_sh;
+  int64_t v_sb, v_ss, v_sh;
+  int64_t o_sb, o_ss, o_sh;
+  float c;  // scale * log2(e)
+};
+
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void attn_fwd_fp8_kernel(Fp8Args a) {
+  extern __shared__ __attribute__((aligned(16))) char smem8[];
+  constexpr int NT = NW * 64;
+  constexpr int LPT = (kBN8 * 8) / NT;  // 16-byte chunks per lane per tile and tensor
+  constexpr int BM = NW * 32;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hh = lane >> 5;
+
+  const int wg = blockIdx.x;
+  const int w = (wg & 7) * a.chunk + (wg >> 3);
+  if (w >= a.total) return;
+  const int bh = w / a.nqt, qt = w - bh * a.nqt;
+  const int b = bh / a.H, h = bh - b * a.H;
+
+  const uint8_t* qp = a.q + b * a.q_sb + h * a.q_sh;
+  const uint8_t* kp = a.k + b * a.k_sb + h * a.k_sh;
+  const uint8_t* vp = a.v + b * a.v_sb + h * a.v_sh;
+  const int q0 = qt * BM + wave * 32;
+  const int nt = (a.Skv + kBN8 - 1) / kBN8;
+  const float c = a.c * a.q_scale[0] * a.k_scale[0];
+
+  // ---- Q fragments: lane (row l32, half hh) holds bytes 64*j + 32*hh .. +31 of its row
+  i32x8 qf[2];
+  {
+    int row = q0 + l32;
+    row = row < a.Sq ? row : a.Sq - 1;
+    const uint8_t* p = qp + (int64_t)row * a.q_ss + hh * 32;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const u32x4 lo = *reinterpret_cast<const u32x4*>(p + j * 64);
+      const u32x4 hi = *reinterpret_cast<const u32x4*>(p + j * 64 + 16);
+      qf[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    }
+  }
+
+  // ---- global -> register -> LDS staging.  Rows past the end re-read the last valid row: they only
+  // ever meet masked logits (P = 0), and every e4m3 code the quantiser emits is finite.
+  u32x4 kr[LPT], vr[LPT];
+  auto gload = [&](int kt) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int id = tid + i * NT;
+      const int row = id >> 3, cc = id & 7;
+      int kk = kt * kBN8 + row;
+      kk = kk < a.Skv ? kk : a.Skv - 1;
+      kr[i] = *reinterpret_cast<const u32x4*>(kp + (int64_t)kk * a.k_ss + cc * 16);
+      vr[i] = *reinterpret_cast<const u32x4*>(vp + (int64_t)kk * a.v_ss + cc * 16);
+    }
+  };
+  auto lstore = [&](int slot) __attribute__((always_inline)) {
+    char* Ks = smem8 + slot * kStage8;
+    char* Vs = Ks + kBN8 * kKS8;
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int id = tid + i * NT;
+      const int row = id >> 3, cc = id & 7;
+      const int swz = 2 * (((row >> 1) & 1) + 2 * ((row >> 3) & 1));  // in 16-byte chunks
+      *reinterpret_cast<u32x4*>(Ks + row * kKS8 + cc * 16) = kr[i];
+      *reinterpret_cast<u32x4*>(Vs + row * kVS8 + ((cc ^ swz) * 16)) = vr[i];
+    }
+  };
+
+  f32x16 O[4];
+#pragma unroll
+  for (int sl = 0; sl < 4; ++sl)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) O[sl][i] = 0.f;
+  float ref = -1e30f, l = 0.f;  // reference point of P (log2 units), per-lane partial row sum
+
+  // lane-constant LDS offsets (bytes)
+  const int k_off = l32 * kKS8 + hh * 32;
+  int v_off[4];
+  {
+    const int e = (lane & 15) >> 1;
+    const int rowl = 8 * (e >> 2) + 4 * hh + (e & 3);
+    const int fl = ((e >> 1) & 1) + 2 * ((e >> 2) & 1);
+    const int cl = 2 * ((lane >> 4) & 1) + (lane & 1);
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) v_off[sl] = kBN8 * kKS8 + rowl * kVS8 + 32 * (sl ^ fl) + 8 * cl;
+  }
+
+  auto tile = [&](int t, auto masked) __attribute__((always_inline)) {
+    const char* Ks = smem8 + (t & 1) * kStage8;
+    // ---- S^T = K.Q^T for the two 32-key blocks
+    f32x16 S[2];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      i32x8 kf[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const char* p = Ks + k_off + blk * 32 * kKS8 + j * 64;
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(p);
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(p + 16);
+        kf[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+      }
+      f32x16 z;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) z[i] = 0.f;
+      z = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[0], qf[0], z, 0, 0, 0, 0, 0, 0);
+      S[blk] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], z, 0, 0, 0, 0, 0, 0);
+    }
+    if constexpr (decltype(masked)::value) {
+      const int kbase = t * kBN8 + 4 * hh;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (kbase + 32 * blk + 8 * (i >> 2) + (i & 3) >= a.Skv) S[blk][i] = -INFINITY;
+    }
+    // ---- row max over the tile; move the reference point only when P would leave [0, 2^8]
+    float mx = S[0][0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, S[0][i]);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, S[1][i]);
+    mx = xhalf_max(mx) * c;
+    const bool need = mx > ref + (kPOff + kPLazy);
+    if (__builtin_amdgcn_ballot_w64(need) != 0) {
+      const float nref = need ? mx - kPOff : ref;
+      const float alpha = __builtin_amdgcn_exp2f(ref - nref);
+      ref = nref;
+      l *= alpha;
+#pragma unroll
+      for (int sl = 0; sl < 4; ++sl)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) O[sl][i] *= alpha;
+    }
+    // ---- P = exp2(c*S - ref), f32 row sum, e4m3 pack in B-operand order
+    i32x8 pk;
+    float ls = 0.f;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float p[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          p[x] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[blk][4 * g + x], c, -ref));
+          ls += p[x];
+        }
+        int u = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
+        u = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], u, true);
+        pk[4 * blk + g] = u;
+      }
+    l += ls;
+    // ---- O^T += V^T.P^T
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      const char* vsrc = Ks + v_off[sl];
+      const i32x2 r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_ptr)(vsrc));
+      const i32x2 r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_ptr)(vsrc + 16 * kVS8));
+      const i32x2 r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_ptr)(vsrc + 32 * kVS8));
+      const i32x2 r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_ptr)(vsrc + 48 * kVS8));
+      const i32x8 vf = {r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
+      O[sl] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pk, O[sl], 0, 0, 0, 0, 0, 0);
+    }
+  };
+
+  gload(0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  lstore(0);
+  gload(1);
+  __syncthreads();
+  for (int t = 0; t < nt - 1; ++t) {
+    tile(t, std::false_type{});
+    // slot (t+1)&1 was last read in iteration t-1, which every wave left through the barrier below
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    lstore((t + 1) & 1);
+    gload(t + 2);
+    __syncthreads();
+  }
+  tile(nt - 1, std::true_type{});
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the look-ahead loads before the registers die
+
+  // ---- epilogue
+  __bf16* op = a.out + b * a.o_sb + h * a.o_sh;
+  const float lt = xhalf_sum(l);
+  const float inv = a.v_scale[0] / lt;
+  const int row = q0 + l32;
+  if (row < a.Sq) {
+    __bf16* orow = op + (int64_t)row * a.o_ss + 4 * hh;
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        uint2 u;
+        u.x = pack2(O[sl][4 * g] * inv, O[sl][4 * g + 1] * inv);
+        u.y = pack2(O[sl][4 * g + 2] * inv, O[sl][4 * g + 3] * inv);
+        *reinterpret_cast<uint2*>(orow + sl * 32 + 8 * g) = u;
+      }
+    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (ref + __log2f(lt)) * kLn2;
+  }
+}
+
+template <int NW>
+int launch_fwd8(hipStream_t st, Fp8Args a, int B) {
+  constexpr int BM = NW * 32;
+  constexpr int lds_bytes = 2 * kStage8;
+  a.nqt = (a.Sq + BM - 1) / BM;
+  const int64_t total = (int64_t)B * a.H * a.nqt;
+  if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
+  a.total = (int)total;
+  a.chunk = (a.total + 7) / 8;
+  hipLaunchKernelGGL(attn_fwd_fp8_kernel<NW>, dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  return launch_status();
+}
+
+}  // namespace
+}  // namespace mdattn
+
+using namespace mdattn;
 
 extern "C" int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, const void* v8, void* out, float* lse,
                               int B, int H, int Sq, int Skv, int D,
                               const mdattn_strides* q_strides, const mdattn_strides* k_strides,
                               const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
                               const float* q_scale, const float* k_scale, const float* v_scale) {
-  (void)stream; (void)q8; (void)k8; (void)v8; (void)out; (void)lse; (void)B; (void)H; (void)Sq; (void)Skv; (void)D;
-  (void)q_strides; (void)k_strides; (void)v_strides; (void)o_strides; (void)scale; (void)q_scale; (void)k_scale; (void)v_scale;
-  return MDATTN_E_UNSUPPORTED;
+  if (!q8 || !k8 || !v8 || !out || !q_scale || !k_scale || !v_scale) return MDATTN_E_BADARG;
+  if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return MDATTN_E_BADARG;
+  if (!q_strides || !k_strides || !v_strides || !o_strides) return MDATTN_E_BADARG;
+  if (!(scale > 0.f) || !(scale < 1e30f)) return MDATTN_E_BADARG;
+  if (D != kD8) return MDATTN_E_UNSUPPORTED;
+  if (!aligned16(q8) || !aligned16(k8) || !aligned16(v8) || !aligned16(out) || (reinterpret_cast<uintptr_t>(lse) & 3u) ||
+      (reinterpret_cast<uintptr_t>(q_scale) & 3u) || (reinterpret_cast<uintptr_t>(k_scale) & 3u) ||
+      (reinterpret_cast<uintptr_t>(v_scale) & 3u))
+    return MDATTN_E_ALIGN;
+  // fp8 rows are read in 16-byte pieces, bf16 output rows written in 8-byte pieces
+  if (!strides_ok(q_strides, 16) || !strides_ok(k_strides, 16) || !strides_ok(v_strides, 16) || !strides_ok(o_strides, 8))
+    return MDATTN_E_ALIGN;
+  if (q_strides->seq < D || k_strides->seq < D || v_strides->seq < D || o_strides->seq < D) return MDATTN_E_BADARG;
+
+  Fp8Args a;
+  a.q = (const uint8_t*)q8; a.k = (const uint8_t*)k8; a.v = (const uint8_t*)v8; a.out = (__bf16*)out; a.lse = lse;
+  a.q_scale = q_scale; a.k_scale = k_scale; a.v_scale = v_scale;
+  a.H = H; a.Sq = Sq; a.Skv = Skv;
+  a.q_sb = q_strides->batch; a.q_ss = q_strides->seq; a.q_sh = q_strides->head;
+  a.k_sb = k_strides->batch; a.k_ss = k_strides->seq; a.k_sh = k_strides->head;
+  a.v_sb = v_strides->batch; a.v_ss = v_strides->seq; a.v_sh = v_strides->head;
+  a.o_sb = o_strides->batch; a.o_ss = o_strides->seq; a.o_sh = o_strides->head;
+  a.c = scale * kLog2e;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t wg256 = (int64_t)B * H * ((Sq + 255) / 256);
+  return wg256 >= 256 ? launch_fwd8<8>(st, a, B) : launch_fwd8<4>(st, a, B);
 }

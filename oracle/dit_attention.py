@@ -367,28 +367,34 @@ def quant_e4m3(x):
   return e4m3_round(x / s), s
 
 
-def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64):
+def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: float = 4.0, p_lazy: float = 4.0):
   """Emulation of the fp8 kernel's arithmetic (no reference counterpart).
 
-  Q, K, V quantised per tensor; logits from the quantised operands in f32; online softmax
-  per KV tile with P rounded to e4m3 before the PV product; f32 accumulation; the row sum
-  uses the un-rounded P.  q [H,Sq,D], k/v [H,Skv,D].
+  Q, K, V quantised per tensor; logits from the quantised operands in f32; online softmax per
+  KV tile in base 2 with P rounded to e4m3 before the PV product; f32 accumulation; the row
+  sum uses the un-rounded P.  P = exp2(logit - ref) where the reference point `ref` is set to
+  (row max - p_offset) whenever the running row max exceeds ref + p_offset + p_lazy: P then
+  stays within [0, 2^(p_offset+p_lazy)] = [0, 256], inside e4m3's range, and probabilities
+  down to 2^-(6+p_offset) of the row max stay in e4m3's normal range.  The result does not
+  depend on `ref` except through the e4m3 rounding.  q [H,Sq,D], k/v [H,Skv,D].
   """
   q8, sq = quant_e4m3(q)
   k8, sk = quant_e4m3(k)
   v8, sv = quant_e4m3(v)
   H, Sq, D = q8.shape
   Skv = k8.shape[1]
-  m = np.full((H, Sq), -np.inf, np.float32)
+  ref = np.full((H, Sq), -1e30, np.float32)
   l = np.zeros((H, Sq), np.float32)
   o = np.zeros((H, Sq, D), np.float32)
-  c = np.float32(sq * sk * scale)
+  c = np.float32(np.float32(scale) * np.float32(np.log2(np.e)) * sq * sk)
   for t0 in range(0, Skv, kv_tile):
-    s = np.einsum("hqd,hkd->hqk", q8, k8[:, t0:t0 + kv_tile]) * c
-    m_new = np.maximum(m, s.max(axis=-1))
-    a = np.exp(m - m_new)
-    p = np.exp(s - m_new[..., None])
+    s = np.einsum("hqd,hkd->hqk", q8, k8[:, t0:t0 + kv_tile])
+    mx = s.max(axis=-1) * c
+    need = mx > ref + np.float32(p_offset + p_lazy)
+    nref = np.where(need, mx - np.float32(p_offset), ref).astype(np.float32)
+    a = np.exp2(ref - nref)
+    ref = nref
+    p = np.exp2(s * c - ref[..., None]).astype(np.float32)
     l = a * l + p.sum(axis=-1)
     o = a[..., None] * o + np.einsum("hqk,hkd->hqd", e4m3_round(p), v8[:, t0:t0 + kv_tile])
-    m = m_new
-  return o * sv / l[..., None], m + np.log(l)
+  return o * sv / l[..., None], (ref + np.log2(l)) * np.float32(np.log(2.0))
