@@ -1,6 +1,6 @@
 """Benchmark of the DiT attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload wan14b|wan14b-ring|wan1.3b|flux-dev]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload wan14b|wan14b-ring|wan14b-fp8|wan1.3b|flux-dev]
 
 One step = one pass of the path over one synthetic batch already resident in HBM: fused q/k
 RMSNorm + RoPE, then the bf16 self-attention forward (with LSE).  Prints ONE JSON line:
@@ -20,6 +20,7 @@ if ROOT not in sys.path:
   sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA
 PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 
 
@@ -99,14 +100,19 @@ def main():
     prologue = lambda: ops.norm_rope_perhead(q4, k4, wq, wk, cos, sin)
 
   ev = lambda: torch.cuda.Event(enable_timing=True)
-  t_pro, t_att = [], []
+  t_pro, t_att, t_quant = [], [], []
+  fp8 = args.workload.endswith("-fp8")
 
   def step(record: bool):
-    e0, e1, e2 = ev(), ev(), ev()
+    e0, e1, e2, eq = ev(), ev(), ev(), ev()
     e0.record()
     qn, kn = prologue()
     e1.record()
-    if ring == 1:
+    if fp8:  # per-tensor absmax e4m3 quantisation of q, k, v, then the fp8 kernel
+      (q8, sq), (k8, sk), (v8, sv) = (ops.quant_e4m3(x) for x in (qn, kn, v))
+      eq.record()
+      ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=w.scale, return_lse=True)
+    elif ring == 1:
       ops.flash_attention(qn, kn, v, scale=w.scale, return_lse=True)
     else:  # one ring shard: this Q chunk against `ring` successive KV chunks, merged in LSE space
       o_run, l_run = ops.new_merge_state(1, S, H, D, dev)
@@ -119,7 +125,9 @@ def main():
     if record:
       torch.cuda.synchronize()
       t_pro.append(e0.elapsed_time(e1))
-      t_att.append(e1.elapsed_time(e2))
+      t_att.append((eq if fp8 else e1).elapsed_time(e2))
+      if fp8:
+        t_quant.append(e1.elapsed_time(eq))
 
   if args.traffic_probe:
     src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
@@ -145,6 +153,8 @@ def main():
   tpath = os.path.join(ROOT, "profiles", "traffic.json")
   if os.path.exists(tpath):  # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command
     traffic = json.load(open(tpath)).get(args.workload, {})
+  peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
+  kname = "attn_fwd_fp8_kernel" if fp8 else "attn_fwd_bf16_kernel"
   out = {
       "metric": "self-attn TFLOP/s (% bf16 MFMA peak) at Wan-14B 75.6k tokens; norm-RoPE GB/s" if args.workload == "wan14b"
       else f"self-attn TFLOP/s ({args.workload}); norm-RoPE GB/s",
@@ -157,18 +167,21 @@ def main():
       "higher_is_better": True,
       "scaling": "weak",
       "vs_baseline": None,
-      "dtype": "bf16",
+      "dtype": "fp8-e4m3" if fp8 else "bf16",
       "data": "synthetic",
       "config": {"workload": f"{args.workload}: B=1 H={H} D={D} Sq={S} Skv={Skv * ring} norm={w.norm} rope={w.rope}"
                              + (f" ring_chunks={ring} (merge per chunk)" if ring > 1 else ""),
-                 "step": "fused q/k RMSNorm+RoPE -> bf16 flash-attention forward with LSE"},
-      "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                   "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic.get("attn_fwd_bf16_kernel"), "kernel": "attn_fwd_bf16_kernel",
+                 "step": "fused q/k RMSNorm+RoPE -> " + ("per-tensor e4m3 quantisation of q, k, v -> fp8 flash-attention forward with LSE"
+                                                             if fp8 else "bf16 flash-attention forward with LSE")},
+      "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+                   "frac": achieved / peak, "traffic": traffic.get(kname), "kernel": kname,
                    "kernel_ms": att_ms, "flop_per_launch": flops / ring},
       "roofline_norm_rope": {"bound": "hbm", "achieved": nr_bytes / (pro_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                              "frac": nr_bytes / (pro_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "traffic": traffic.get(f"norm_rope_{w.norm}_kernel"),
                              "kernel": f"norm_rope_{w.norm}_kernel", "kernel_ms": pro_ms, "bytes_per_launch": nr_bytes},
   }
+  if fp8:
+    out["quant_ms"] = sum(t_quant) / len(t_quant)
   if args.cpu_rows > 0:
     out["cpu_baseline"] = cpu_baseline(w, args.cpu_rows)
   print(json.dumps(out), flush=True)

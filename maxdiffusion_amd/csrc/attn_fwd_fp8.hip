@@ -59,8 +59,10 @@ struct Fp8Args {
   float c;  // scale * log2(e)
 };
 
+// Register budget: three waves per SIMD (<= 168 VGPRs).  The kernel is bound by the vector ALU (softmax)
+// and by latencies a single wave cannot hide, so the third wave per SIMD is worth more than registers.
 template <int NW>
-__global__ __launch_bounds__(NW * 64) void attn_fwd_fp8_kernel(Fp8Args a) {
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_fwd_fp8_kernel(Fp8Args a) {
   extern __shared__ __attribute__((aligned(16))) char smem8[];
   constexpr int NT = NW * 64;
   constexpr int LPT = (kBN8 * 8) / NT;  // 16-byte chunks per lane per tile and tensor
@@ -97,30 +99,47 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_fp8_kernel(Fp8Args a) {
     }
   }
 
-  // ---- global -> register -> LDS staging.  Rows past the end re-read the last valid row: they only
-  // ever meet masked logits (P = 0), and every e4m3 code the quantiser emits is finite.
+  // ---- global -> register -> LDS staging.  A tile's address is a uniform base (advanced on the scalar
+  // unit) plus a per-lane byte offset that never changes, so the main loop spends no vector
+  // instruction on addressing.  Rows past the end of a ragged last tile re-read the last valid row:
+  // they only ever meet masked logits (P = 0), and every e4m3 code the quantiser emits is finite.
   u32x4 kr[LPT], vr[LPT];
-  auto gload = [&](int kt) __attribute__((always_inline)) {
+  constexpr int RPP = NT / 8;  // rows covered by one pass of the workgroup (a multiple of 32: same swizzle)
+  const int srow = tid >> 3, scc = tid & 7;
+  const int sswz = 2 * (((srow >> 1) & 1) + 2 * ((srow >> 3) & 1));  // in 16-byte chunks
+  const unsigned kofs = (unsigned)(srow * (int)a.k_ss + scc * 16);
+  const unsigned vofs = (unsigned)(srow * (int)a.v_ss + scc * 16);
+  const unsigned lofs_k = (unsigned)(srow * kKS8 + scc * 16);
+  const unsigned lofs_v = (unsigned)(kBN8 * kKS8 + srow * kVS8 + ((scc ^ sswz) * 16));
+  const int64_t k_tile_bytes = a.k_ss * kBN8, v_tile_bytes = a.v_ss * kBN8;
+  const bool ragged = (a.Skv & (kBN8 - 1)) != 0;
+  auto gload = [&](int it) __attribute__((always_inline)) {
+    if (it >= nt) return;
+    const uint8_t* kt = kp + it * k_tile_bytes;
+    const uint8_t* vt = vp + it * v_tile_bytes;
+    if (ragged && it == nt - 1) {
 #pragma unroll
-    for (int i = 0; i < LPT; ++i) {
-      const int id = tid + i * NT;
-      const int row = id >> 3, cc = id & 7;
-      int kk = kt * kBN8 + row;
-      kk = kk < a.Skv ? kk : a.Skv - 1;
-      kr[i] = *reinterpret_cast<const u32x4*>(kp + (int64_t)kk * a.k_ss + cc * 16);
-      vr[i] = *reinterpret_cast<const u32x4*>(vp + (int64_t)kk * a.v_ss + cc * 16);
+      for (int i = 0; i < LPT; ++i) {
+        int row = srow + i * RPP;
+        const int last = a.Skv - 1 - it * kBN8;
+        row = row < last ? row : last;
+        kr[i] = *reinterpret_cast<const u32x4*>(kt + (int64_t)row * a.k_ss + scc * 16);
+        vr[i] = *reinterpret_cast<const u32x4*>(vt + (int64_t)row * a.v_ss + scc * 16);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < LPT; ++i) {
+        kr[i] = *reinterpret_cast<const u32x4*>(kt + i * RPP * a.k_ss + kofs);
+        vr[i] = *reinterpret_cast<const u32x4*>(vt + i * RPP * a.v_ss + vofs);
+      }
     }
   };
   auto lstore = [&](int slot) __attribute__((always_inline)) {
-    char* Ks = smem8 + slot * kStage8;
-    char* Vs = Ks + kBN8 * kKS8;
+    char* base = smem8 + slot * kStage8;
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
-      const int id = tid + i * NT;
-      const int row = id >> 3, cc = id & 7;
-      const int swz = 2 * (((row >> 1) & 1) + 2 * ((row >> 3) & 1));  // in 16-byte chunks
-      *reinterpret_cast<u32x4*>(Ks + row * kKS8 + cc * 16) = kr[i];
-      *reinterpret_cast<u32x4*>(Vs + row * kVS8 + ((cc ^ swz) * 16)) = vr[i];
+      *reinterpret_cast<u32x4*>(base + lofs_k + i * RPP * kKS8) = kr[i];
+      *reinterpret_cast<u32x4*>(base + lofs_v + i * RPP * kVS8) = vr[i];
     }
   };
 
@@ -179,9 +198,10 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_fp8_kernel(Fp8Args a) {
     for (int i = 0; i < 16; ++i) mx = fmaxf(mx, S[1][i]);
     mx = xhalf_max(mx) * c;
     const bool need = mx > ref + (kPOff + kPLazy);
-    if (__builtin_amdgcn_ballot_w64(need) != 0) {
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(need) != 0, 0)) {
       const float nref = need ? mx - kPOff : ref;
-      const float alpha = __builtin_amdgcn_exp2f(ref - nref);
+      float alpha = __builtin_amdgcn_exp2f(ref - nref);
+      asm volatile("" : "+v"(alpha));  // keeps the rescale inside this rarely taken branch
       ref = nref;
       l *= alpha;
 #pragma unroll
@@ -292,6 +312,8 @@ extern "C" int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, cons
   if (!strides_ok(q_strides, 16) || !strides_ok(k_strides, 16) || !strides_ok(v_strides, 16) || !strides_ok(o_strides, 8))
     return MDATTN_E_ALIGN;
   if (q_strides->seq < D || k_strides->seq < D || v_strides->seq < D || o_strides->seq < D) return MDATTN_E_BADARG;
+  // per-lane byte offsets inside one 64-row tile are kept in 32 bits
+  if (k_strides->seq >= (1 << 24) || v_strides->seq >= (1 << 24)) return MDATTN_E_UNSUPPORTED;
 
   Fp8Args a;
   a.q = (const uint8_t*)q8; a.k = (const uint8_t*)k8; a.v = (const uint8_t*)v8; a.out = (__bf16*)out; a.lse = lse;
@@ -303,6 +325,13 @@ extern "C" int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, cons
   a.o_sb = o_strides->batch; a.o_ss = o_strides->seq; a.o_sh = o_strides->head;
   a.c = scale * kLog2e;
   hipStream_t st = (hipStream_t)stream;
-  const int64_t wg256 = (int64_t)B * H * ((Sq + 255) / 256);
-  return wg256 >= 256 ? launch_fwd8<8>(st, a, B) : launch_fwd8<4>(st, a, B);
+  // Four waves per workgroup (three workgroups per CU) measured faster than eight at every shape tried;
+  // MDATTN_FP8_VARIANT (1: 8 waves, 2: 4 waves per workgroup) overrides the choice for experiments.
+  int variant = 2;
+  if (const char* e = getenv("MDATTN_FP8_VARIANT")) variant = atoi(e);
+  switch (variant) {
+    case 1: return launch_fwd8<8>(st, a, B);
+    case 2: return launch_fwd8<4>(st, a, B);
+    default: return MDATTN_E_BADARG;
+  }
 }
