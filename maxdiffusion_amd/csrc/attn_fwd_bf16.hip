@@ -2,10 +2,10 @@
 //
 // Work decomposition
 //   workgroup  = NW waves, each wave owns 32 query rows  (BM = NW*32 rows); two waves per SIMD
-//   K/V tiles  = 64 keys x 128, staged through a 3-deep LDS ring.  Ring slot t%3 holds K(t) together
-//                with V(t-1): both are consumed in the same "period" (two 32-key iterations).  One
-//                barrier per period; the global loads of slot t+3 are in flight in registers while
-//                period t runs.
+//   K/V tiles  = 64 keys x 128, in a 4-deep LDS ring filled by direct global->LDS loads (no staging
+//                registers, no LDS store instructions).  Ring slot t%4 holds K(t) together with V(t-1):
+//                both are consumed in the same "period" (two 32-key iterations).  One barrier per
+//                period; the loads of slots t+2 and t+3 are in flight while period t runs.
 //   S^T = K.Q^T with v_mfma_f32_32x32x16_bf16: A = K rows from LDS (ds_read_b128), B = Q fragment
 //                held in registers for the whole kernel.  In the 32x32 accumulator layout every lane
 //                then holds 16 keys of ONE query row, so the row max / row sum are in-lane
@@ -39,9 +39,19 @@ namespace mdattn {
 
 constexpr int kBN = 64;          // keys per tile
 constexpr int kD = 128;          // head dim
-constexpr int kKStr = kD + 8;    // K row stride in LDS (272 B: 16 rows x 16 B hit 64 distinct banks)
-constexpr int kVStr = kD + 32;   // V row stride in LDS (320 B: 4 rows x 64 B hit 64 distinct banks)
-constexpr int kStage = kBN * kKStr + kBN * kVStr;  // elements per ring stage
+// LDS tile layouts (elements).  Tiles are filled by direct global->LDS loads.  One wave instruction
+// writes 1 KB = one group of 4 rows, row-major; the lane -> global address map is free, so inside a row
+// the 16-byte chunks are stored permuted (XOR with the row's position in its group), which replaces
+// row padding:
+//   K: chunk c of row r sits at chunk position c ^ (r & 3); groups are padded by 64 B.  The 16 lanes a
+//      ds_read_b128 serves at once (16 rows, one logical chunk) hit 16 distinct 16-byte bank slots.
+//   V: 64-byte segment s of row r sits at segment position s ^ (r & 3).  The 4 rows x 64 B a half-wave
+//      reads through ds_read_b64_tr_b16 cover all 64 banks once.
+// Every 16 lanes of a load fetch one whole 256-byte row from global memory.
+constexpr int kGK = 4 * kD + 32;  // K group stride (1088 B)
+constexpr int kGV = 4 * kD;       // V group stride (1024 B)
+constexpr int kKTile = (kBN / 4) * kGK;
+constexpr int kStage = kKTile + (kBN / 4) * kGV;  // elements per ring stage
 constexpr float kLazy = 8.0f;    // log2 units a row max may lag behind before accumulators are rescaled
 
 typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
@@ -54,12 +64,25 @@ __device__ __forceinline__ bf16x8 read_vt(const __bf16* p0, const __bf16* p1) {
   return __builtin_bit_cast(bf16x8, r);
 }
 
+// Direct global -> LDS load of 16 bytes per lane: lane i's bytes land at lds_addr + 16*i (the LDS base
+// travels in M0).  Written as inline assembly so that the loads stay asynchronous: the compiler cannot
+// tell which LDS bytes such a load writes and would otherwise wait for it before the next LDS read.
+// The kernel tracks them itself with s_waitcnt vmcnt.
+__device__ __forceinline__ void lds_dma16(const void* base, unsigned byte_off, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(byte_off), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void lds_dma16(const void* addr, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(addr) : "memory", "m0");
+}
+__device__ __forceinline__ unsigned lds_addr_of(const void* p) {
+  return (unsigned)(uintptr_t)(const void __attribute__((address_space(3)))*)p;
+}
+
 template <int NW>
 __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
   constexpr int NT = NW * 64;
-  constexpr int LPT = (kBN * 16) / NT;  // 16-byte chunks per lane per tile and tensor
   constexpr int BM = NW * 32;
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -89,42 +112,44 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
     for (int s = 0; s < 8; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(p + s * 16);
   }
 
-  // ---- global -> register -> LDS staging of one ring slot: K(kt) and V(kt-1).  Rows outside the
-  // sequence re-read the nearest valid row: they only ever meet masked logits / zero probabilities,
-  // but must be finite.
-  u32x4 kr[LPT], vr[LPT];
-  auto gload = [&](int kt) __attribute__((always_inline)) {
+  // ---- direct global -> LDS loads of one ring slot: K(kt) and V(kt-1).  Wave w fills the row groups
+  // w, w+NW, ...  Rows outside the sequence re-read the nearest valid row: they only ever meet masked
+  // logits / zero probabilities, but must be finite.  Tiles that lie fully inside the sequence use a
+  // uniform base plus a lane offset that never changes.
+  const int grow = lane >> 4;                                  // row of the group this lane fills
+  const int kcol = ((lane & 15) ^ grow) * 8;                   // K: logical chunk stored at this lane's position
+  const int vcol = ((lane & 15) ^ (grow << 2)) * 8;            // V: same, segments permuted instead of chunks
+  const unsigned kofs = (unsigned)(grow * (int)a.k_ss + kcol) * 2u;    // bytes
+  const unsigned vofs = (unsigned)(grow * (int)a.v_ss + vcol) * 2u;
+  const unsigned smem_addr = lds_addr_of(smem);
+  auto dma = [&](int slot, int kt) __attribute__((always_inline)) {
+    const unsigned Ks = smem_addr + (unsigned)(slot * kStage) * 2u;
+    const unsigned Vs = Ks + kKTile * 2u;
+    if (kt >= 1 && kt * kBN + kBN <= a.Skv) {
+      const __bf16* kt0 = kp + (int64_t)(kt * kBN + 4 * wave) * a.k_ss;
+      const __bf16* vt0 = vp + (int64_t)((kt - 1) * kBN + 4 * wave) * a.v_ss;
 #pragma unroll
-    for (int i = 0; i < LPT; ++i) {
-      const int id = tid + i * NT;
-      const int row = id >> 4, cc = id & 15;
-      int kk = kt * kBN + row;
-      kk = kk < a.Skv ? kk : a.Skv - 1;
-      int kvv = (kt - 1) * kBN + row;
-      kvv = kvv < a.Skv ? kvv : a.Skv - 1;
-      kvv = kvv > 0 ? kvv : 0;
-      kr[i] = *reinterpret_cast<const u32x4*>(kp + (int64_t)kk * a.k_ss + cc * 8);
-      vr[i] = *reinterpret_cast<const u32x4*>(vp + (int64_t)kvv * a.v_ss + cc * 8);
+      for (int i = 0; i < 16 / NW; ++i) {
+        lds_dma16(kt0 + (int64_t)(4 * NW * i) * a.k_ss, kofs, Ks + (unsigned)((wave + NW * i) * kGK) * 2u);
+        lds_dma16(vt0 + (int64_t)(4 * NW * i) * a.v_ss, vofs, Vs + (unsigned)((wave + NW * i) * kGV) * 2u);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16 / NW; ++i) {
+        const int g = wave + NW * i;
+        int kk = kt * kBN + 4 * g + grow;
+        kk = kk < a.Skv ? kk : a.Skv - 1;
+        int kvv = (kt - 1) * kBN + 4 * g + grow;
+        kvv = kvv < a.Skv ? kvv : a.Skv - 1;
+        kvv = kvv > 0 ? kvv : 0;
+        lds_dma16(kp + (int64_t)kk * a.k_ss + kcol, Ks + (unsigned)(g * kGK) * 2u);
+        lds_dma16(vp + (int64_t)kvv * a.v_ss + vcol, Vs + (unsigned)(g * kGV) * 2u);
+      }
     }
   };
-  auto lstore = [&](int slot) __attribute__((always_inline)) {
-    __bf16* Ks = smem + slot * kStage;
-    __bf16* Vs = Ks + kBN * kKStr;
-#pragma unroll
-    for (int i = 0; i < LPT; ++i) {
-      const int id = tid + i * NT;
-      const int row = id >> 4, cc = id & 15;
-      *reinterpret_cast<u32x4*>(Ks + row * kKStr + cc * 8) = kr[i];
-      *reinterpret_cast<u32x4*>(Vs + row * kVStr + cc * 8) = vr[i];
-    }
-  };
-  gload(0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): Q fragments and slot 0 have landed
-  lstore(0);
-  gload(1);
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  lstore(1);
-  gload(2);  // stays in flight; stored at the top of period 0
+  dma(0, 0);
+  dma(1, 1);
+  dma(2, 2);
 
   f32x16 O[4];
 #pragma unroll
@@ -134,8 +159,17 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   float m = -1e30f, l = 0.f;
 
   // lane-constant LDS offsets
-  const int k_off = l32 * kKStr + hh * 8;
-  const int v_off = kBN * kKStr + (4 * hh + ((lane & 15) >> 2)) * kVStr + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+  // K fragment j (logical chunk 2j + hh) of row l32 sits at chunk position (2j + hh) ^ (l32 & 3): pair j ^ x1,
+  // half hh ^ x0.  Even and odd j get a base each, so that the rest of the offset is a compile-time constant.
+  const int kx0 = l32 & 1, kx1 = (l32 >> 1) & 1;
+  const int k_base = (l32 >> 2) * kGK + (l32 & 3) * kD + (hh ^ kx0) * 8;
+  const int k_off_e = k_base + 16 * kx1, k_off_o = k_base - 16 * kx1;
+  // V fragment jv: segment s = jv & 3 of row group 4*(jv >> 2) + hh, row xr of the group; one base per segment
+  const int vxr = (lane & 15) >> 2;
+  int v_off[4];
+#pragma unroll
+  for (int sg = 0; sg < 4; ++sg)
+    v_off[sg] = kKTile + hh * kGV + vxr * kD + (sg ^ vxr) * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
 
   f32x16 Sa, Sb;        // logits of odd / even blocks
   bf16x8 Pa[2], Pb[2];  // probabilities of odd / even blocks (PV B-operand layout, 16 keys each)
@@ -149,7 +183,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   // KC/KN: K rows of block BLK+1 / BLK+2; VC/VN: V rows of block BLK-1 / BLK.
   // Slot n of the stream: n even -> PV MFMA n/2, n odd -> QK MFMA n/2, each followed by the LDS
   // request for the MFMA of the same kind three ahead, then a chunk of the softmax of block BLK.
-#define MDATTN_ITER(SC, SN, PC, PP, KC, KN, VC, VN, BLK)                                                     \
+#define MDATTN_ITER(SC, SN, PC, PP, KC, KN, VC, VN, BLK) /* KC.. : base pointers [even j, odd j]; VC.. : [segment] */                                                     \
   {                                                                                                           \
     float alpha = 1.f, mc = 0.f, lsum = 0.f, p[8];                                                            \
     bool need = false;                                                                                        \
@@ -163,8 +197,8 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
       const int j = n >> 1, jn = j + 3;                                                                       \
       if ((n & 1) == 0) {                                                                                     \
         O[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[j & 3], PP[j >> 2], O[j & 3], 0, 0, 0);        \
-        const __bf16* vsrc = (jn < 8 ? (VC) : (VN)) + ((jn & 7) >> 2) * 16 * kVStr + (jn & 3) * 32;           \
-        vfr[jn & 3] = read_vt(vsrc, vsrc + 8 * kVStr);                                                        \
+        const __bf16* vsrc = (jn < 8 ? (VC) : (VN))[jn & 3] + ((jn & 7) >> 2) * 4 * kGV;                      \
+        vfr[jn & 3] = read_vt(vsrc, vsrc + 2 * kGV);                                                          \
       } else {                                                                                                \
         if (j == 0) {                                                                                         \
           f32x16 z;                                                                                           \
@@ -173,7 +207,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
         } else {                                                                                              \
           SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[j & 3], qf[j], SN, 0, 0, 0);                       \
         }                                                                                                     \
-        kfr[jn & 3] = *reinterpret_cast<const bf16x8*>((jn < 8 ? (KC) : (KN)) + (jn & 7) * 16);               \
+        kfr[jn & 3] = *reinterpret_cast<const bf16x8*>((jn < 8 ? (KC) : (KN))[jn & 1] + (jn & 7) * 16);       \
       }                                                                                                       \
       if (n == 1) {                                                                                           \
         /* row max + lazy-rescale decision: a row's max moves only when it would otherwise see an exp2    */  \
@@ -211,33 +245,40 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
     }                                                                                                         \
   }
 
-  // ring bookkeeping: period t uses slot t%3 (K(t), V(t-1)) and looks ahead into slot (t+1)%3
-  int s_cur = 0, s_nxt = 1, s_fill = 2;
+  // ring bookkeeping: period t uses slot t%4 (K(t), V(t-1)) and looks ahead into slot (t+1)%4
+  int s_cur = 0, s_nxt = 1, s_nn = 2, s_fill = 3;
   // fragments the first iteration's first three QK / PV MFMAs expect in the windows
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): Q fragments and this wave's share of slots 0..2
   __syncthreads();
 #pragma unroll
   for (int s = 0; s < 3; ++s) {
-    kfr[s] = *reinterpret_cast<const bf16x8*>(smem + k_off + s * 16);
-    const __bf16* vsrc = smem + v_off + s * 32;
-    vfr[s] = read_vt(vsrc, vsrc + 8 * kVStr);
+    kfr[s] = *reinterpret_cast<const bf16x8*>(smem + ((s & 1) ? k_off_o : k_off_e) + s * 16);
+    const __bf16* vsrc = smem + v_off[s];
+    vfr[s] = read_vt(vsrc, vsrc + 2 * kGV);
   }
   for (int t = 0; t <= nt; ++t) {
-    // slot s_fill was last read in period t-1; K(t+2), V(t+1) were requested one period ago
+    // every wave's loads into slot s_nxt (issued two periods ago) have landed once all waves pass the
+    // barrier: only the loads of the previous period (2 * 16 / NW per wave) may still be in flight.
+    // Slot s_fill was last read in period t-1 and now receives K(t+3), V(t+2).
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (32 / NW));
     __syncthreads();
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    lstore(s_fill);
-    gload(t + 3);
-    const __bf16* Kcur = smem + s_cur * kStage + k_off;
-    const __bf16* Knxt = smem + s_nxt * kStage + k_off;
-    const __bf16* Vcur = smem + s_cur * kStage + v_off;
-    const __bf16* Vnxt = smem + s_nxt * kStage + v_off;
+    dma(s_fill, t + 3);
+    const __bf16* cur = smem + s_cur * kStage;
+    const __bf16* nxt = smem + s_nxt * kStage;
+    const __bf16* Kc0[2] = {cur + k_off_e, cur + k_off_o};
+    const __bf16* Kc1[2] = {Kc0[0] + 8 * kGK, Kc0[1] + 8 * kGK};
+    const __bf16* Kn0[2] = {nxt + k_off_e, nxt + k_off_o};
+    const __bf16* Vc0[4] = {cur + v_off[0], cur + v_off[1], cur + v_off[2], cur + v_off[3]};
+    const __bf16* Vc1[4] = {Vc0[0] + 8 * kGV, Vc0[1] + 8 * kGV, Vc0[2] + 8 * kGV, Vc0[3] + 8 * kGV};
+    const __bf16* Vn0[4] = {nxt + v_off[0], nxt + v_off[1], nxt + v_off[2], nxt + v_off[3]};
     // iteration 2t-1: softmax(2t-1), PV(2t-2), QK(2t)
-    MDATTN_ITER(Sa, Sb, Pa, Pb, Kcur, Kcur + 32 * kKStr, Vcur, Vcur + 32 * kVStr, 2 * t - 1)
+    MDATTN_ITER(Sa, Sb, Pa, Pb, Kc0, Kc1, Vc0, Vc1, 2 * t - 1)
     // iteration 2t: softmax(2t), PV(2t-1), QK(2t+1)
-    MDATTN_ITER(Sb, Sa, Pb, Pa, Kcur + 32 * kKStr, Knxt, Vcur + 32 * kVStr, Vnxt, 2 * t)
+    MDATTN_ITER(Sb, Sa, Pb, Pa, Kc1, Kn0, Vc1, Vn0, 2 * t)
     const int tmp = s_cur;
     s_cur = s_nxt;
-    s_nxt = s_fill;
+    s_nxt = s_nn;
+    s_nn = s_fill;
     s_fill = tmp;
   }
 #undef MDATTN_ITER
@@ -265,7 +306,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
 template <int NW>
 static int launch_fwd(hipStream_t st, AttnArgs a, int B) {
   constexpr int BM = NW * 32;
-  constexpr int lds_bytes = 3 * kStage * 2;
+  constexpr int lds_bytes = 4 * kStage * 2;
   a.nqt = (a.Sq + BM - 1) / BM;
   const int64_t total = (int64_t)B * a.H * a.nqt;
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
