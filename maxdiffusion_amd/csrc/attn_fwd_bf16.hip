@@ -64,20 +64,6 @@ __device__ __forceinline__ bf16x8 read_vt(const __bf16* p0, const __bf16* p1) {
   return __builtin_bit_cast(bf16x8, r);
 }
 
-// Direct global -> LDS load of 16 bytes per lane: lane i's bytes land at lds_addr + 16*i (the LDS base
-// travels in M0).  Written as inline assembly so that the loads stay asynchronous: the compiler cannot
-// tell which LDS bytes such a load writes and would otherwise wait for it before the next LDS read.
-// The kernel tracks them itself with s_waitcnt vmcnt.
-__device__ __forceinline__ void lds_dma16(const void* base, unsigned byte_off, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(byte_off), "s"(base) : "memory", "m0");
-}
-__device__ __forceinline__ void lds_dma16(const void* addr, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(addr) : "memory", "m0");
-}
-__device__ __forceinline__ unsigned lds_addr_of(const void* p) {
-  return (unsigned)(uintptr_t)(const void __attribute__((address_space(3)))*)p;
-}
-
 template <int NW>
 __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];

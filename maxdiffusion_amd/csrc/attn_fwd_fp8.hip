@@ -32,9 +32,10 @@ namespace {
 
 constexpr int kBN8 = 64;                                  // keys per tile
 constexpr int kD8 = 128;                                  // head dim = bytes per row
-constexpr int kKS8 = kD8 + 16;                            // K row stride in LDS, bytes
-constexpr int kVS8 = kD8;                                 // V row stride in LDS, bytes (swizzled, not padded)
+constexpr int kKS8 = kD8;                                 // K row stride in LDS, bytes (chunks permuted, not padded)
+constexpr int kVS8 = kD8;                                 // V row stride in LDS, bytes (chunks permuted, not padded)
 constexpr int kStage8 = kBN8 * kKS8 + kBN8 * kVS8;        // bytes per LDS stage
+constexpr int kSlots8 = 3;                                // LDS ring depth
 constexpr float kPOff = 4.0f;                             // P = exp2(logit - max + kPOff) at a fresh maximum
 constexpr float kPLazy = 4.0f;                            // extra headroom before the reference point moves
 
@@ -65,7 +66,6 @@ template <int NW>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_fwd_fp8_kernel(Fp8Args a) {
   extern __shared__ __attribute__((aligned(16))) char smem8[];
   constexpr int NT = NW * 64;
-  constexpr int LPT = (kBN8 * 8) / NT;  // 16-byte chunks per lane per tile and tensor
   constexpr int BM = NW * 32;
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -99,47 +99,39 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
     }
   }
 
-  // ---- global -> register -> LDS staging.  A tile's address is a uniform base (advanced on the scalar
-  // unit) plus a per-lane byte offset that never changes, so the main loop spends no vector
-  // instruction on addressing.  Rows past the end of a ragged last tile re-read the last valid row:
-  // they only ever meet masked logits (P = 0), and every e4m3 code the quantiser emits is finite.
-  u32x4 kr[LPT], vr[LPT];
-  constexpr int RPP = NT / 8;  // rows covered by one pass of the workgroup (a multiple of 32: same swizzle)
-  const int srow = tid >> 3, scc = tid & 7;
-  const int sswz = 2 * (((srow >> 1) & 1) + 2 * ((srow >> 3) & 1));  // in 16-byte chunks
-  const unsigned kofs = (unsigned)(srow * (int)a.k_ss + scc * 16);
-  const unsigned vofs = (unsigned)(srow * (int)a.v_ss + scc * 16);
-  const unsigned lofs_k = (unsigned)(srow * kKS8 + scc * 16);
-  const unsigned lofs_v = (unsigned)(kBN8 * kKS8 + srow * kVS8 + ((scc ^ sswz) * 16));
-  const int64_t k_tile_bytes = a.k_ss * kBN8, v_tile_bytes = a.v_ss * kBN8;
-  const bool ragged = (a.Skv & (kBN8 - 1)) != 0;
-  auto gload = [&](int it) __attribute__((always_inline)) {
-    if (it >= nt) return;
-    const uint8_t* kt = kp + it * k_tile_bytes;
-    const uint8_t* vt = vp + it * v_tile_bytes;
-    if (ragged && it == nt - 1) {
+  // ---- direct global -> LDS loads of one K/V tile (no staging registers, no LDS store instructions).
+  // One wave instruction writes 1 KB = 8 rows, row-major; inside a row the 16-byte chunks are stored
+  // permuted, which replaces padding: K chunk c of row r sits at position c ^ ((r >> 1) & 7), V chunk c at
+  // c ^ 2*(((r >> 1) & 1) + 2*((r >> 3) & 1)).  Every 8 lanes fetch one whole 128-byte row.  Wave w fills
+  // the row groups w, w+NW, ...  Rows past the end re-read the last valid row: they only ever meet
+  // masked logits (P = 0), and every e4m3 code the quantiser emits is finite.
+  constexpr int GPW = 8 / NW;                                  // 8-row groups per wave, tile and tensor
+  const int grow = lane >> 3;                                  // row of the group this lane fills
+  const int kx_fill = (4 * (wave & 1) + (grow >> 1)) & 7;      // (row >> 1) & 7 of that row (groups w, w+NW: same parity)
+  const int vx_fill = 2 * (((grow >> 1) & 1) + 2 * (wave & 1));
+  const unsigned kofs = (unsigned)(grow * (int)a.k_ss + (((lane & 7) ^ kx_fill) * 16));
+  const unsigned vofs = (unsigned)(grow * (int)a.v_ss + (((lane & 7) ^ vx_fill) * 16));
+  const unsigned smem_addr = lds_addr_of(smem8);
+  auto dma = [&](int slot, int kt) __attribute__((always_inline)) {
+    const unsigned Ks = smem_addr + (unsigned)(slot * kStage8);
+    const unsigned Vs = Ks + kBN8 * kKS8;
+    if (kt * kBN8 + kBN8 <= a.Skv) {
+      const uint8_t* kt0 = kp + (int64_t)(kt * kBN8 + 8 * wave) * a.k_ss;
+      const uint8_t* vt0 = vp + (int64_t)(kt * kBN8 + 8 * wave) * a.v_ss;
 #pragma unroll
-      for (int i = 0; i < LPT; ++i) {
-        int row = srow + i * RPP;
-        const int last = a.Skv - 1 - it * kBN8;
-        row = row < last ? row : last;
-        kr[i] = *reinterpret_cast<const u32x4*>(kt + (int64_t)row * a.k_ss + scc * 16);
-        vr[i] = *reinterpret_cast<const u32x4*>(vt + (int64_t)row * a.v_ss + scc * 16);
+      for (int i = 0; i < GPW; ++i) {
+        lds_dma16(kt0 + (int64_t)(8 * NW * i) * a.k_ss, kofs, Ks + (unsigned)((wave + NW * i) * 8 * kKS8));
+        lds_dma16(vt0 + (int64_t)(8 * NW * i) * a.v_ss, vofs, Vs + (unsigned)((wave + NW * i) * 8 * kVS8));
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < LPT; ++i) {
-        kr[i] = *reinterpret_cast<const u32x4*>(kt + i * RPP * a.k_ss + kofs);
-        vr[i] = *reinterpret_cast<const u32x4*>(vt + i * RPP * a.v_ss + vofs);
+      for (int i = 0; i < GPW; ++i) {
+        const int g = wave + NW * i;
+        int kk = kt * kBN8 + 8 * g + grow;
+        kk = kk < a.Skv ? kk : a.Skv - 1;
+        lds_dma16(kp + (int64_t)kk * a.k_ss + (((lane & 7) ^ kx_fill) * 16), Ks + (unsigned)(g * 8 * kKS8));
+        lds_dma16(vp + (int64_t)kk * a.v_ss + (((lane & 7) ^ vx_fill) * 16), Vs + (unsigned)(g * 8 * kVS8));
       }
-    }
-  };
-  auto lstore = [&](int slot) __attribute__((always_inline)) {
-    char* base = smem8 + slot * kStage8;
-#pragma unroll
-    for (int i = 0; i < LPT; ++i) {
-      *reinterpret_cast<u32x4*>(base + lofs_k + i * RPP * kKS8) = kr[i];
-      *reinterpret_cast<u32x4*>(base + lofs_v + i * RPP * kVS8) = vr[i];
     }
   };
 
@@ -151,7 +143,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   float ref = -1e30f, l = 0.f;  // reference point of P (log2 units), per-lane partial row sum
 
   // lane-constant LDS offsets (bytes)
-  const int k_off = l32 * kKS8 + hh * 32;
+  // K fragment (d half j, 16-byte half i) of row l32 is logical chunk 4j + 2hh + i
+  int k_off[2][2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) k_off[j][i] = l32 * kKS8 + (((4 * j + 2 * hh + i) ^ ((l32 >> 1) & 7)) * 16);
   int v_off[4];
   {
     const int e = (lane & 15) >> 1;
@@ -162,8 +159,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
     for (int sl = 0; sl < 4; ++sl) v_off[sl] = kBN8 * kKS8 + rowl * kVS8 + 32 * (sl ^ fl) + 8 * cl;
   }
 
-  auto tile = [&](int t, auto masked) __attribute__((always_inline)) {
-    const char* Ks = smem8 + (t & 1) * kStage8;
+  auto tile = [&](int t, int slot, auto masked) __attribute__((always_inline)) {
+    const char* Ks = smem8 + slot * kStage8;
     // ---- S^T = K.Q^T for the two 32-key blocks
     f32x16 S[2];
 #pragma unroll
@@ -171,9 +168,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       i32x8 kf[2];
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const char* p = Ks + k_off + blk * 32 * kKS8 + j * 64;
-        const u32x4 lo = *reinterpret_cast<const u32x4*>(p);
-        const u32x4 hi = *reinterpret_cast<const u32x4*>(p + 16);
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(Ks + k_off[j][0] + blk * 32 * kKS8);
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(Ks + k_off[j][1] + blk * 32 * kKS8);
         kf[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
       }
       f32x16 z;
@@ -240,21 +236,22 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
     }
   };
 
-  gload(0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-  lstore(0);
-  gload(1);
-  __syncthreads();
+  // Ring of kSlots8 tiles: the loads of tile t+2 are issued at the top of iteration t, so at the top of
+  // iteration t only the 2*GPW loads of tile t+1 may still be in flight once tile t is needed.
+  dma(0, 0);
+  dma(1, 1);
+  int slot = 0, fill = 2;
   for (int t = 0; t < nt - 1; ++t) {
-    tile(t, std::false_type{});
-    // slot (t+1)&1 was last read in iteration t-1, which every wave left through the barrier below
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    lstore((t + 1) & 1);
-    gload(t + 2);
-    __syncthreads();
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * GPW));  // vmcnt: this wave's share of tile t has landed
+    __syncthreads();                                  // ... and everyone's; slot `fill` (tile t-1) is free
+    dma(fill, t + 2);
+    tile(t, slot, std::false_type{});
+    slot = slot == kSlots8 - 1 ? 0 : slot + 1;
+    fill = fill == kSlots8 - 1 ? 0 : fill + 1;
   }
-  tile(nt - 1, std::true_type{});
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the look-ahead loads before the registers die
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+  tile(nt - 1, slot, std::true_type{});
 
   // ---- epilogue
   __bf16* op = a.out + b * a.o_sb + h * a.o_sh;
@@ -279,7 +276,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
 template <int NW>
 int launch_fwd8(hipStream_t st, Fp8Args a, int B) {
   constexpr int BM = NW * 32;
-  constexpr int lds_bytes = 2 * kStage8;
+  constexpr int lds_bytes = kSlots8 * kStage8;
   a.nqt = (a.Sq + BM - 1) / BM;
   const int64_t total = (int64_t)B * a.H * a.nqt;
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;

@@ -77,6 +77,21 @@ __device__ __forceinline__ void st_nt(uint4* p, const uint4& u) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
 
+// Direct global -> LDS load of 16 bytes per lane: lane i's bytes land at lds_addr + 16*i (the LDS base
+// travels in M0).  Written as inline assembly so that the loads stay asynchronous: the compiler cannot
+// tell which LDS bytes such a load writes and would otherwise wait for it before the next LDS read.
+// M0 is never live across statements in compiled code (the compiler sets it right before each use).
+// The kernels track these loads themselves with s_waitcnt vmcnt.
+__device__ __forceinline__ void lds_dma16(const void* base, unsigned byte_off, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(byte_off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void lds_dma16(const void* addr, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(addr) : "memory");
+}
+__device__ __forceinline__ unsigned lds_addr_of(const void* p) {
+  return (unsigned)(uintptr_t)(const void __attribute__((address_space(3)))*)p;
+}
+
 // Arguments of the attention-forward kernels (element strides; head_dim contiguous).
 struct AttnArgs {
   const __bf16* q;
