@@ -33,6 +33,8 @@
 //                share it through that XCD's L2.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "mdattn_common.h"
 
 namespace mdattn {
@@ -289,6 +291,198 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Second schedule: no software pipelining inside a wave.  Four waves per workgroup, 32-key tiles in a
+// 3-slot ring (50 KB of LDS) and at most 168 VGPRs, so that three workgroups share a CU and three waves
+// share each SIMD: while one wave runs its softmax on the vector ALU the other two keep the matrix
+// pipe busy.  Same tile layouts, same fragment reads, same arithmetic as the pipelined kernel.
+constexpr int kTS = 32;                               // keys per tile
+constexpr int kKTileS = (kTS / 4) * kGK;              // elements
+constexpr int kStageS = kKTileS + (kTS / 4) * kGV;    // elements per ring slot
+constexpr int kSlotsS = 3;
+
+template <int NW>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_fwd_bf16_flat_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
+  constexpr int BM = NW * 32;
+  constexpr int GPW = (kTS / 4) / NW;  // 4-row groups per wave, tile and tensor
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hh = lane >> 5;
+
+  const int wg = blockIdx.x;
+  const int w = (wg & 7) * a.chunk + (wg >> 3);
+  if (w >= a.total) return;
+  const int bh = w / a.nqt, qt = w - bh * a.nqt;
+  const int b = bh / a.H, h = bh - b * a.H;
+
+  const __bf16* qp = a.q + b * a.q_sb + h * a.q_sh;
+  const __bf16* kp = a.k + b * a.k_sb + h * a.k_sh;
+  const __bf16* vp = a.v + b * a.v_sb + h * a.v_sh;
+  const int q0 = qt * BM + wave * 32;
+  const int nt = (a.Skv + kTS - 1) / kTS;
+  const float c = a.c;
+
+  bf16x8 qf[8];
+  {
+    int row = q0 + l32;
+    row = row < a.Sq ? row : a.Sq - 1;
+    const __bf16* p = qp + (int64_t)row * a.q_ss + hh * 8;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(p + s * 16);
+  }
+
+  const int grow = lane >> 4;
+  const int kcol = ((lane & 15) ^ grow) * 8;
+  const int vcol = ((lane & 15) ^ (grow << 2)) * 8;
+  const unsigned kofs = (unsigned)(grow * (int)a.k_ss + kcol) * 2u;
+  const unsigned vofs = (unsigned)(grow * (int)a.v_ss + vcol) * 2u;
+  const unsigned smem_addr = lds_addr_of(smem);
+  auto dma = [&](int slot, int kt) __attribute__((always_inline)) {
+    const unsigned Ks = smem_addr + (unsigned)(slot * kStageS) * 2u;
+    const unsigned Vs = Ks + kKTileS * 2u;
+    if (kt * kTS + kTS <= a.Skv) {
+      const __bf16* kt0 = kp + (int64_t)(kt * kTS + 4 * wave) * a.k_ss;
+      const __bf16* vt0 = vp + (int64_t)(kt * kTS + 4 * wave) * a.v_ss;
+#pragma unroll
+      for (int i = 0; i < GPW; ++i) {
+        lds_dma16(kt0 + (int64_t)(4 * NW * i) * a.k_ss, kofs, Ks + (unsigned)((wave + NW * i) * kGK) * 2u);
+        lds_dma16(vt0 + (int64_t)(4 * NW * i) * a.v_ss, vofs, Vs + (unsigned)((wave + NW * i) * kGV) * 2u);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < GPW; ++i) {
+        const int g = wave + NW * i;
+        int kk = kt * kTS + 4 * g + grow;
+        kk = kk < a.Skv ? kk : a.Skv - 1;
+        lds_dma16(kp + (int64_t)kk * a.k_ss + kcol, Ks + (unsigned)(g * kGK) * 2u);
+        lds_dma16(vp + (int64_t)kk * a.v_ss + vcol, Vs + (unsigned)(g * kGV) * 2u);
+      }
+    }
+  };
+
+  f32x16 O[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) O[db][i] = 0.f;
+  float m = -1e30f, l = 0.f;
+
+  const int kx0 = l32 & 1, kx1 = (l32 >> 1) & 1;
+  const int k_base = (l32 >> 2) * kGK + (l32 & 3) * kD + (hh ^ kx0) * 8;
+  const int k_off_e = k_base + 16 * kx1, k_off_o = k_base - 16 * kx1;
+  const int vxr = (lane & 15) >> 2;
+  int v_off[4];
+#pragma unroll
+  for (int sg = 0; sg < 4; ++sg)
+    v_off[sg] = kKTileS + hh * kGV + vxr * kD + (sg ^ vxr) * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+
+  auto tile = [&](int t, int slot, auto masked) __attribute__((always_inline)) {
+    const __bf16* base = smem + slot * kStageS;
+    // ---- S^T = K.Q^T: one chain of 8 MFMAs; the other waves of the SIMD fill the gaps between them
+    f32x16 S;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) S[i] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + ((j & 1) ? k_off_o : k_off_e) + j * 16);
+      S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[j], S, 0, 0, 0);
+    }
+    if constexpr (decltype(masked)::value) {
+      const int kv_base = t * kTS + 4 * hh;
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (kv_base + 8 * (i >> 2) + (i & 3) >= a.Skv) S[i] = -INFINITY;
+    }
+    // ---- online softmax with lazy rescale
+    float mloc = S[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, S[i]);
+    mloc = xhalf_max(mloc);
+    const bool moved = (mloc - m) * c > kLazy;
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(moved) != 0, 0)) {
+      const float mnew = moved ? mloc : m;
+      float alpha = __builtin_amdgcn_exp2f((m - mnew) * c);
+      asm volatile("" : "+v"(alpha));  // keeps the rescale inside this rarely taken branch
+      m = mnew;
+      l *= alpha;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) O[db][i] *= alpha;
+    }
+    const float mc = m * c;
+    bf16x8 P[2];
+    float lsum = 0.f;
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb) {
+      float p[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[8 * hb + e], c, -mc));
+        lsum += p[e];
+      }
+      P[hb] = __builtin_bit_cast(bf16x8, pack8(p));
+    }
+    l += lsum;
+    // ---- O^T += V^T.P^T
+#pragma unroll
+    for (int jv = 0; jv < 8; ++jv) {
+      const __bf16* vsrc = base + v_off[jv & 3] + (jv >> 2) * 4 * kGV;
+      const bf16x8 vf = read_vt(vsrc, vsrc + 2 * kGV);
+      O[jv & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P[jv >> 2], O[jv & 3], 0, 0, 0);
+    }
+  };
+
+  dma(0, 0);
+  dma(1, 1);
+  int slot = 0, fill = 2;
+  for (int t = 0; t < nt - 1; ++t) {
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * GPW));  // vmcnt: this wave's share of tile t has landed
+    __syncthreads();                                  // ... and everyone's; slot `fill` (tile t-1) is free
+    dma(fill, t + 2);
+    tile(t, slot, std::false_type{});
+    slot = slot == kSlotsS - 1 ? 0 : slot + 1;
+    fill = fill == kSlotsS - 1 ? 0 : fill + 1;
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+  tile(nt - 1, slot, std::true_type{});
+
+  __bf16* op = a.out + b * a.o_sb + h * a.o_sh;
+  const float lt = xhalf_sum(l);
+  const float inv = 1.0f / lt;
+  const int row = q0 + l32;
+  if (row < a.Sq) {
+    __bf16* orow = op + (int64_t)row * a.o_ss + 4 * hh;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        uint2 u;
+        u.x = pack2(O[db][4 * g] * inv, O[db][4 * g + 1] * inv);
+        u.y = pack2(O[db][4 * g + 2] * inv, O[db][4 * g + 3] * inv);
+        *reinterpret_cast<uint2*>(orow + db * 32 + 8 * g) = u;
+      }
+    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (m * c + __log2f(lt)) * kLn2;
+  }
+}
+
+template <int NW>
+static int launch_flat(hipStream_t st, AttnArgs a, int B) {
+  constexpr int BM = NW * 32;
+  constexpr int lds_bytes = kSlotsS * kStageS * 2;
+  a.nqt = (a.Sq + BM - 1) / BM;
+  const int64_t total = (int64_t)B * a.H * a.nqt;
+  if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
+  a.total = (int)total;
+  a.chunk = (a.total + 7) / 8;
+  hipLaunchKernelGGL(attn_fwd_bf16_flat_kernel<NW>, dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  return launch_status();
+}
+
 template <int NW>
 static int launch_fwd(hipStream_t st, AttnArgs a, int B) {
   constexpr int BM = NW * 32;
@@ -333,18 +527,20 @@ extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const
   a.c = scale * kLog2e;
   hipStream_t st = (hipStream_t)stream;
 
-  // 8 waves x 32 query rows (two waves per SIMD) is the fast shape; 4 waves x 32 rows gives more
-  // workgroups when there are few (head, q-tile) pairs.  MDATTN_FWD_VARIANT (1: 8 waves, 2: 4 waves)
-  // overrides the choice for experiments.
+  // Two schedules.  The software-pipelined kernel (8 waves x 32 query rows, two waves per SIMD) is a little
+  // faster once every CU has many workgroups to go through; the flat kernel (4 waves x 32 rows, three
+  // workgroups per CU) wins on smaller grids.  MDATTN_FWD_VARIANT (1: pipelined 8 waves, 2: pipelined
+  // 4 waves, 3: flat) overrides the choice for experiments and tests.
   int variant = 0;
   if (const char* e = getenv("MDATTN_FWD_VARIANT")) variant = atoi(e);
   if (variant == 0) {
     const int64_t wg256 = (int64_t)B * H * ((Sq + 255) / 256);
-    variant = wg256 >= 256 ? 1 : 2;
+    variant = wg256 >= 4096 ? 1 : 3;
   }
   switch (variant) {
     case 1: return launch_fwd<8>(st, a, B);
     case 2: return launch_fwd<4>(st, a, B);
+    case 3: return launch_flat<4>(st, a, B);
     default: return MDATTN_E_BADARG;
   }
 }

@@ -57,7 +57,7 @@ def test_golden_small_and_sharp(dev):
   _check(to_np(out), to_np(lse), g["out_sharp"], g["lse_sharp"], "golden sharp (q x6)")
 
 
-@pytest.mark.parametrize("var", [1, 2])
+@pytest.mark.parametrize("var", [1, 2, 3])
 @pytest.mark.parametrize("sq,skv", [(1, 1), (31, 65), (257, 63), (300, 333), (1000, 77), (64, 4097), (513, 512)])
 def test_ragged_shapes_every_tile_variant(dev, variant, var, sq, skv):
   variant(var)
