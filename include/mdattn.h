@@ -106,6 +106,30 @@ int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const void* v, v
  *   scale_out f32[2] device: [0] = absmax/448 (x ~= x_fp8 * scale_out[0]), [1] = absmax (scratch of the reduction)
  * n % 16 == 0.
  */
+/*
+ * The same forward with an additive per-key bias: logits = scale*q.k + key_bias[b, key] (natural-log units;
+ * -inf excludes a key).  Replaces: the key padding mask of `_apply_attention` (models/attention_flax.py:1926-1939:
+ * a [B,Skv] keep-mask becomes an additive bias; rows whose keys are all masked return 0, :1552-1554) and the
+ * segment-id masking of the flash wrappers (:390-438).
+ *   key_bias     f32 [B, bias_stride]; bias_stride a multiple of 32 and >= Skv rounded up to 32 (entries at and
+ *                past Skv are ignored); 16-byte aligned
+ * Rows without any kept key give out = 0 and lse = -inf.
+ */
+int mdattn_fwd_bf16_bias(void* stream, const void* q, const void* k, const void* v, void* out, float* lse,
+                         int B, int H, int Sq, int Skv, int D,
+                         const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                         const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
+                         const float* key_bias, int64_t bias_stride);
+
+/*
+ * Keep-mask -> additive bias for mdattn_fwd_bf16_bias: bias[b, j] = keep[b, j] ? 0 : masked_value for j < Skv,
+ * masked_value for the padding up to bias_stride.  Replaces: the mask canonicalisation of
+ * models/attention_flax.py:1931-1939 (which uses -10000; the flash kernels exclude masked keys, i.e. -inf).
+ *   keep         u8 [B, Skv] contiguous (non-zero = keep);  bias  f32 [B, bias_stride]
+ */
+int mdattn_key_mask_bias(void* stream, const void* keep, float* bias, int B, int Skv, int64_t bias_stride,
+                         float masked_value);
+
 int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, float* scale_out, int64_t n);
 
 /*

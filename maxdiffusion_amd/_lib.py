@@ -36,6 +36,8 @@ SIGNATURES = {
     "mdattn_norm_rope_fullrow": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _L, _L, _S], _I),
     "mdattn_norm_rope_perhead": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _F, _S, _S], _I),
     "mdattn_fwd_bf16": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),
+    "mdattn_fwd_bf16_bias": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F, _P, _L], _I),
+    "mdattn_key_mask_bias": ([_P, _P, _P, _I, _I, _L, _F], _I),
     "mdattn_quant_e4m3": ([_P, _P, _P, _P, _L], _I),
     "mdattn_fwd_fp8": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F, _P, _P, _P], _I),
     "mdattn_merge": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S], _I),

@@ -68,11 +68,11 @@ def _as_bshd(x: torch.Tensor, heads: int) -> torch.Tensor:
   raise ValueError(f"attention inputs must have rank 3 or 4, got {x.dim()}")
 
 
-def _reject_unsupported(context) -> None:
+def _reject_unsupported(context, masks_ok: bool) -> None:
   # The custom kernels of the reference raise NotImplementedError for masks they cannot honour
-  # (attention_flax.py:850-854, :1300-1304); this kernel is non-causal, FullMask only.
-  if context.get("attention_mask") is not None:
-    raise NotImplementedError("hip_flash does not take an attention_mask (non-causal, unmasked DiT attention only)")
+  # (attention_flax.py:850-854, :1300-1304); these kernels are non-causal.
+  if context.get("attention_mask") is not None and not masks_ok:
+    raise NotImplementedError("hip_flash_fp8 does not take an attention_mask")
   if context.get("is_causal"):
     raise NotImplementedError("hip_flash is non-causal")
 
@@ -85,13 +85,17 @@ def hip_flash_kernel(q, k, v, context):
   to the kernel and is folded into the exp2 argument; `flash_block_sizes`, `mesh` and the axis names
   are accepted and ignored (one GPU, tiles fixed by the kernel).
   """
-  _reject_unsupported(context)
+  _reject_unsupported(context, masks_ok=True)
   heads = context["heads"]
   qv, kv, vv = _as_bshd(q, heads), _as_bshd(k, heads), _as_bshd(v, heads)
   cast = q.dtype != torch.bfloat16
   if cast:  # LTX2 hands f32 q/k (attention_ltx2.py:415-432); the MFMA operands are bf16
     qv, kv, vv = qv.to(torch.bfloat16), kv.to(torch.bfloat16), vv.to(torch.bfloat16)
-  out = ops.flash_attention(qv, kv, vv, scale=context["scale"])
+  # [B,Skv] keep-mask (attention_flax.py:1926-1939): masked keys are excluded, as the flash wrappers do with
+  # segment ids (:390-438); rows without a kept key return 0 (:1552-1554)
+  mask = context.get("attention_mask")
+  bias = ops.key_mask_bias(mask) if mask is not None else None
+  out = ops.flash_attention(qv, kv, vv, scale=context["scale"], key_bias=bias)
   b, s, h, d = out.shape
   out = out.reshape(b, s, h * d)
   return out.to(q.dtype) if cast else out
@@ -100,7 +104,7 @@ def hip_flash_kernel(q, k, v, context):
 @register_kernel("hip_flash_fp8")
 def hip_flash_fp8_kernel(q, k, v, context):
   """fp8-e4m3 variant: per-tensor absmax quantisation of q, k, v on the device, then the fp8 kernel."""
-  _reject_unsupported(context)
+  _reject_unsupported(context, masks_ok=False)
   heads = context["heads"]
   qv, kv, vv = (_as_bshd(t, heads).to(torch.bfloat16).contiguous() for t in (q, k, v))
   q8, sq = ops.quant_e4m3(qv)

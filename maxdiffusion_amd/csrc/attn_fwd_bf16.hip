@@ -301,7 +301,7 @@ constexpr int kKTileS = (kTS / 4) * kGK;              // elements
 constexpr int kStageS = kKTileS + (kTS / 4) * kGV;    // elements per ring slot
 constexpr int kSlotsS = 3;
 
-template <int NW>
+template <int NW, bool BIAS>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_fwd_bf16_flat_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
@@ -324,6 +324,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   const int q0 = qt * BM + wave * 32;
   const int nt = (a.Skv + kTS - 1) / kTS;
   const float c = a.c;
+  // with a bias the logits are brought to log2 units (scale folded, bias added) right after the MFMAs
+  const float cs = BIAS ? 1.0f : c;
+  const float* bias_row = BIAS ? a.bias + b * a.bias_sb + 4 * hh : nullptr;
 
   bf16x8 qf[8];
   {
@@ -390,6 +393,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       const bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + ((j & 1) ? k_off_o : k_off_e) + j * 16);
       S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[j], S, 0, 0, 0);
     }
+    if constexpr (BIAS) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_row + t * kTS + 8 * g);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) S[4 * g + e] = __builtin_fmaf(S[4 * g + e], c, bv[e] * kLog2e);
+      }
+    }
     if constexpr (decltype(masked)::value) {
       const int kv_base = t * kTS + 4 * hh;
 #pragma unroll
@@ -401,10 +412,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
 #pragma unroll
     for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, S[i]);
     mloc = xhalf_max(mloc);
-    const bool moved = (mloc - m) * c > kLazy;
+    const bool moved = (mloc - m) * cs > kLazy;
     if (__builtin_expect(__builtin_amdgcn_ballot_w64(moved) != 0, 0)) {
       const float mnew = moved ? mloc : m;
-      float alpha = __builtin_amdgcn_exp2f((m - mnew) * c);
+      float alpha = __builtin_amdgcn_exp2f((m - mnew) * cs);
       asm volatile("" : "+v"(alpha));  // keeps the rescale inside this rarely taken branch
       m = mnew;
       l *= alpha;
@@ -413,7 +424,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[db][i] *= alpha;
     }
-    const float mc = m * c;
+    const float mc = m * cs;
     bf16x8 P[2];
     float lsum = 0.f;
 #pragma unroll
@@ -421,7 +432,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       float p[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[8 * hb + e], c, -mc));
+        p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[8 * hb + e], cs, -mc));
         lsum += p[e];
       }
       P[hb] = __builtin_bit_cast(bf16x8, pack8(p));
@@ -453,7 +464,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
 
   __bf16* op = a.out + b * a.o_sb + h * a.o_sh;
   const float lt = xhalf_sum(l);
-  const float inv = 1.0f / lt;
+  const float inv = lt > 0.f ? 1.0f / lt : 0.f;  // rows whose keys are all excluded return 0
   const int row = q0 + l32;
   if (row < a.Sq) {
     __bf16* orow = op + (int64_t)row * a.o_ss + 4 * hh;
@@ -466,11 +477,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
         u.y = pack2(O[db][4 * g + 2] * inv, O[db][4 * g + 3] * inv);
         *reinterpret_cast<uint2*>(orow + db * 32 + 8 * g) = u;
       }
-    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (m * c + __log2f(lt)) * kLn2;
+    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (m * cs + __log2f(lt)) * kLn2;
   }
 }
 
-template <int NW>
+template <int NW, bool BIAS>
 static int launch_flat(hipStream_t st, AttnArgs a, int B) {
   constexpr int BM = NW * 32;
   constexpr int lds_bytes = kSlotsS * kStageS * 2;
@@ -479,7 +490,7 @@ static int launch_flat(hipStream_t st, AttnArgs a, int B) {
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
-  hipLaunchKernelGGL(attn_fwd_bf16_flat_kernel<NW>, dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  hipLaunchKernelGGL((attn_fwd_bf16_flat_kernel<NW, BIAS>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   return launch_status();
 }
 
@@ -503,10 +514,10 @@ static int launch_fwd(hipStream_t st, AttnArgs a, int B) {
 
 using namespace mdattn;
 
-extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* out, float* lse,
-                               int B, int H, int Sq, int Skv, int D,
-                               const mdattn_strides* q_strides, const mdattn_strides* k_strides,
-                               const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
+static int fill_args(AttnArgs& a, const void* q, const void* k, const void* v, void* out, float* lse,
+                     int B, int H, int Sq, int Skv, int D,
+                     const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                     const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
   if (!q || !k || !v || !out || B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return MDATTN_E_BADARG;
   if (!q_strides || !k_strides || !v_strides || !o_strides) return MDATTN_E_BADARG;
   if (!(scale > 0.f) || !(scale < 1e30f)) return MDATTN_E_BADARG;
@@ -516,8 +527,8 @@ extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const
   if (!strides_ok(q_strides, 8) || !strides_ok(k_strides, 8) || !strides_ok(v_strides, 8) || !strides_ok(o_strides, 8))
     return MDATTN_E_ALIGN;
   if (q_strides->seq < D || k_strides->seq < D || v_strides->seq < D || o_strides->seq < D) return MDATTN_E_BADARG;
-
-  AttnArgs a;
+  // per-lane byte offsets inside one tile are kept in 32 bits
+  if (k_strides->seq >= (1 << 23) || v_strides->seq >= (1 << 23)) return MDATTN_E_UNSUPPORTED;
   a.q = (const __bf16*)q; a.k = (const __bf16*)k; a.v = (const __bf16*)v; a.out = (__bf16*)out; a.lse = lse;
   a.H = H; a.Sq = Sq; a.Skv = Skv;
   a.q_sb = q_strides->batch; a.q_ss = q_strides->seq; a.q_sh = q_strides->head;
@@ -525,6 +536,17 @@ extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const
   a.v_sb = v_strides->batch; a.v_ss = v_strides->seq; a.v_sh = v_strides->head;
   a.o_sb = o_strides->batch; a.o_ss = o_strides->seq; a.o_sh = o_strides->head;
   a.c = scale * kLog2e;
+  a.bias = nullptr; a.bias_sb = 0;
+  return MDATTN_OK;
+}
+
+extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* out, float* lse,
+                               int B, int H, int Sq, int Skv, int D,
+                               const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                               const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
+  AttnArgs a;
+  const int rc = fill_args(a, q, k, v, out, lse, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides, scale);
+  if (rc != MDATTN_OK) return rc;
   hipStream_t st = (hipStream_t)stream;
 
   // Two schedules.  The software-pipelined kernel (8 waves x 32 query rows, two waves per SIMD) is a little
@@ -540,7 +562,22 @@ extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const
   switch (variant) {
     case 1: return launch_fwd<8>(st, a, B);
     case 2: return launch_fwd<4>(st, a, B);
-    case 3: return launch_flat<4>(st, a, B);
+    case 3: return launch_flat<4, false>(st, a, B);
     default: return MDATTN_E_BADARG;
   }
+}
+
+extern "C" int mdattn_fwd_bf16_bias(void* stream, const void* q, const void* k, const void* v, void* out, float* lse,
+                                    int B, int H, int Sq, int Skv, int D,
+                                    const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                                    const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
+                                    const float* key_bias, int64_t bias_stride) {
+  AttnArgs a;
+  const int rc = fill_args(a, q, k, v, out, lse, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides, scale);
+  if (rc != MDATTN_OK) return rc;
+  if (!key_bias || bias_stride < ((Skv + kTS - 1) / kTS) * kTS || bias_stride % kTS != 0) return MDATTN_E_BADARG;
+  if (!aligned16(key_bias)) return MDATTN_E_ALIGN;
+  a.bias = key_bias;
+  a.bias_sb = bias_stride;
+  return launch_flat<4, true>((hipStream_t)stream, a, B);
 }

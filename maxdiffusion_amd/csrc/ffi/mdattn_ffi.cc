@@ -55,6 +55,26 @@ ffi::Error FwdBf16Impl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, f
                  "mdattn_fwd_bf16");
 }
 
+// key_bias: f32 [B, P] with P a multiple of 32 and >= Skv rounded up to 32 (0 keeps a key, -inf excludes it)
+ffi::Error FwdBf16BiasImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v, ffi::AnyBuffer key_bias,
+                           ffi::Result<ffi::AnyBuffer> out, ffi::Result<ffi::AnyBuffer> lse, float scale, int64_t layout) {
+  if (q.element_type() != ffi::BF16 || k.element_type() != ffi::BF16 || v.element_type() != ffi::BF16 ||
+      out->element_type() != ffi::BF16 || lse->element_type() != ffi::F32 || key_bias.element_type() != ffi::F32)
+    return ffi::Error::InvalidArgument("mdattn_fwd_bf16_bias: q, k, v, out must be bf16, key_bias and lse f32");
+  int64_t B, Sq, H, D, Bk, Skv, Hk, Dk, Bo, So, Ho, Do;
+  mdattn_strides sq, sk, sv, so;
+  if (!Describe(q.dimensions(), layout, &B, &Sq, &H, &D, &sq) || !Describe(k.dimensions(), layout, &Bk, &Skv, &Hk, &Dk, &sk) ||
+      !Describe(v.dimensions(), layout, &Bk, &Skv, &Hk, &Dk, &sv) || !Describe(out->dimensions(), 0, &Bo, &So, &Ho, &Do, &so))
+    return ffi::Error::InvalidArgument("mdattn_fwd_bf16_bias: rank-4 buffers expected");
+  auto bd = key_bias.dimensions();
+  if (Bk != B || Hk != H || Dk != D || Bo != B || So != Sq || Ho != H || Do != D || bd.size() != 2 || bd[0] != B)
+    return ffi::Error::InvalidArgument("mdattn_fwd_bf16_bias: inconsistent shapes");
+  return ToError(mdattn_fwd_bf16_bias(stream, q.untyped_data(), k.untyped_data(), v.untyped_data(), out->untyped_data(),
+                                      static_cast<float*>(lse->untyped_data()), (int)B, (int)H, (int)Sq, (int)Skv, (int)D,
+                                      &sq, &sk, &sv, &so, scale, static_cast<const float*>(key_bias.untyped_data()), bd[1]),
+                 "mdattn_fwd_bf16_bias");
+}
+
 ffi::Error NormRopeFullrowImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer wq, ffi::AnyBuffer wk,
                                ffi::AnyBuffer cos, ffi::AnyBuffer sin, ffi::Result<ffi::AnyBuffer> q_out,
                                ffi::Result<ffi::AnyBuffer> k_out, float eps, int64_t heads, int64_t rope) {
@@ -104,6 +124,13 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnFwdBf16, FwdBf16Impl,
                               ffi::Ffi::Bind()
                                   .Ctx<ffi::PlatformStream<hipStream_t>>()
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
+                                  .Attr<float>("scale").Attr<int64_t>("layout"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnFwdBf16Bias, FwdBf16BiasImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
                                   .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
                                   .Attr<float>("scale").Attr<int64_t>("layout"));
 

@@ -106,6 +106,8 @@ struct AttnArgs {
   int64_t v_sb, v_ss, v_sh;
   int64_t o_sb, o_ss, o_sh;
   float c;  // scale * log2(e)
+  const float* bias;   // optional additive per-key bias [B, bias_sb] (natural-log units), flat kernel only
+  int64_t bias_sb;
 };
 
 

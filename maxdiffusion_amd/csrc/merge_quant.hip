@@ -164,3 +164,23 @@ extern "C" int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, 
   hipLaunchKernelGGL(quant_kernel, dim3(g2), dim3(256), 0, st, (const uint4*)x_bf16, (uint4*)x_fp8, n16, scale_out);
   return launch_status();
 }
+
+// ------------------------------------------------------------------------------------------- key mask -> bias
+namespace mdattn {
+__global__ __launch_bounds__(256) void key_mask_bias_kernel(const uint8_t* __restrict__ keep, float* __restrict__ bias,
+                                                            int Skv, int64_t bias_stride, float masked_value) {
+  const int b = blockIdx.y;
+  for (int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x; j < bias_stride; j += (int64_t)gridDim.x * 256)
+    bias[b * bias_stride + j] = (j < Skv && keep[(int64_t)b * Skv + j]) ? 0.f : masked_value;
+}
+}  // namespace mdattn
+
+extern "C" int mdattn_key_mask_bias(void* stream, const void* keep, float* bias, int B, int Skv, int64_t bias_stride,
+                                    float masked_value) {
+  if (!keep || !bias || B <= 0 || Skv <= 0 || bias_stride < Skv) return MDATTN_E_BADARG;
+  if (B > 65535) return MDATTN_E_UNSUPPORTED;
+  const unsigned gx = (unsigned)((bias_stride + 255) / 256 < 1024 ? (bias_stride + 255) / 256 : 1024);
+  hipLaunchKernelGGL(mdattn::key_mask_bias_kernel, dim3(gx, B), dim3(256), 0, (hipStream_t)stream,
+                     (const uint8_t*)keep, bias, Skv, bias_stride, masked_value);
+  return mdattn::launch_status();
+}

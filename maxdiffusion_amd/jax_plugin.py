@@ -18,6 +18,7 @@ from .build import FFI_LIB_PATH, build_ffi_library
 
 FFI_TARGETS = {
     "mdattn_fwd_bf16": "MdattnFwdBf16",
+    "mdattn_fwd_bf16_bias": "MdattnFwdBf16Bias",
     "mdattn_norm_rope_fullrow": "MdattnNormRopeFullrow",
     "mdattn_norm_rope_perhead": "MdattnNormRopePerhead",
     "mdattn_merge": "MdattnMerge",
@@ -45,8 +46,10 @@ def register_ffi_targets():
     jax.ffi.register_ffi_target(target, jax.ffi.pycapsule(getattr(lib, symbol)), platform="ROCM")
 
 
-def hip_flash_attention(q, k, v, scale: float, layout: int):
-  """q [B,Sq,H,D] (layout 0) or [B,H,Sq,D] (layout 1) bf16 -> (out [B,Sq,H,D] bf16, lse [B,H,Sq] f32)."""
+def hip_flash_attention(q, k, v, scale: float, layout: int, keep_mask=None):
+  """q [B,Sq,H,D] (layout 0) or [B,H,Sq,D] (layout 1) bf16 -> (out [B,Sq,H,D] bf16, lse [B,H,Sq] f32).
+
+  keep_mask: optional [B,Skv] bool; masked keys are excluded (the bias is built with jnp: a [B,Skv] select)."""
   jax, jnp = _require_jax()
   if layout == 0:
     b, sq, h, d = q.shape
@@ -59,6 +62,17 @@ def hip_flash_attention(q, k, v, scale: float, layout: int):
   )
   import numpy as np
 
+  if keep_mask is not None:
+    skv = k.shape[1] if layout == 0 else k.shape[2]
+    pad = (-skv) % 32
+    bias = jnp.where(keep_mask, 0.0, -jnp.inf).astype(jnp.float32)
+    bias = jnp.pad(bias, ((0, 0), (0, pad)), constant_values=-jnp.inf)
+    call = jax.ffi.ffi_call(
+        "mdattn_fwd_bf16_bias",
+        (jax.ShapeDtypeStruct((b, sq, h, d), jnp.bfloat16), jax.ShapeDtypeStruct((b, h, sq), jnp.float32)),
+        vmap_method="sequential",
+    )
+    return call(q, k, v, bias, scale=np.float32(scale), layout=np.int64(layout))
   return call(q, k, v, scale=np.float32(scale), layout=np.int64(layout))
 
 
@@ -80,8 +94,6 @@ def hip_norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6)
 def hip_flash_kernel(q, k, v, context):
   """The KERNEL_REGISTRY entry: fn(q, k, v, context) -> [B, Sq, H*D] in q's dtype."""
   _, jnp = _require_jax()
-  if context.get("attention_mask") is not None:
-    raise NotImplementedError("hip_flash does not take an attention_mask (non-causal, unmasked DiT attention only)")
   if context.get("is_causal"):
     raise NotImplementedError("hip_flash is non-causal")
   heads = context["heads"]
@@ -95,7 +107,8 @@ def hip_flash_kernel(q, k, v, context):
   else:
     q4, k4, v4, layout = q, k, v, 1
   dt = q.dtype
-  out, _ = hip_flash_attention(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"], layout)
+  out, _ = hip_flash_attention(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"], layout,
+                               keep_mask=context.get("attention_mask"))
   b, sq, h, d = out.shape
   return out.reshape(b, sq, h * d).astype(dt)
 

@@ -16,7 +16,7 @@ from . import _lib
 from ._lib import Strides
 
 __all__ = [
-    "norm_rope_fullrow", "norm_rope_perhead", "flash_attention", "flash_attention_fp8", "quant_e4m3",
+    "norm_rope_fullrow", "norm_rope_perhead", "flash_attention", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
     "merge_partial", "finalize", "new_merge_state", "LSE_INIT",
 ]
 
@@ -105,10 +105,26 @@ def norm_rope_perhead(q, k, wq, wk, cos, sin, eps: float = 1e-6, wq_txt=None, wk
   return q_out, k_out
 
 
-def flash_attention(q, k, v, scale: float | None = None, return_lse: bool = False, out_layout: str = "bshd", out=None):
-  """softmax(scale * q k^T) v, non-causal.  q [B,Sq,H,D], k/v [B,Skv,H,D] logical views, bf16.
+def key_mask_bias(keep: torch.Tensor, masked_value: float = -math.inf) -> torch.Tensor:
+  """[B,Skv] keep-mask (bool / uint8) -> additive key bias f32 [B, Skv rounded up to 32] for `flash_attention`."""
+  _check_dev(keep)
+  if keep.dim() != 2:
+    raise ValueError(f"keep mask must have shape [batch, kv_length], got {tuple(keep.shape)}")
+  keep8 = keep.to(torch.uint8).contiguous() if keep.dtype != torch.uint8 else keep.contiguous()
+  b, skv = keep8.shape
+  stride = (skv + 31) // 32 * 32
+  bias = torch.empty((b, stride), dtype=torch.float32, device=keep.device)
+  rc = _lib.load().mdattn_key_mask_bias(_stream(), _ptr(keep8), _ptr(bias), b, skv, stride, float(masked_value))
+  _lib.check(rc, "mdattn_key_mask_bias")
+  return bias
 
-  Returns out (logical [B,Sq,H,D] in `out_layout`) and, if asked, lse f32 [B,H,Sq] (natural log).
+
+def flash_attention(q, k, v, scale: float | None = None, return_lse: bool = False, out_layout: str = "bshd", out=None,
+                    key_bias: torch.Tensor | None = None):
+  """softmax(scale * q k^T [+ key_bias]) v, non-causal.  q [B,Sq,H,D], k/v [B,Skv,H,D] logical views, bf16.
+
+  `key_bias` f32 [B, >= Skv rounded up to 32] (see `key_mask_bias`) is added to the scaled logits of each key;
+  -inf excludes a key.  Returns out (logical [B,Sq,H,D] in `out_layout`) and, if asked, lse f32 [B,H,Sq] (natural log).
   """
   _check_dev(q, k, v)
   if not (q.dtype == k.dtype == v.dtype == torch.bfloat16):
@@ -123,10 +139,20 @@ def flash_attention(q, k, v, scale: float | None = None, return_lse: bool = Fals
     out = _alloc_like_layout(b, sq, h, d, out_layout, torch.bfloat16, q.device)
   lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device) if return_lse else None
   sq_, sk_, sv_, so_ = _strides(q), _strides(k), _strides(v), _strides(out)
-  rc = _lib.load().mdattn_fwd_bf16(
-      _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), b, h, sq, skv, d,
-      ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale))
-  _lib.check(rc, "mdattn_fwd_bf16")
+  if key_bias is None:
+    rc = _lib.load().mdattn_fwd_bf16(
+        _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), b, h, sq, skv, d,
+        ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale))
+    _lib.check(rc, "mdattn_fwd_bf16")
+  else:
+    _check_dev(key_bias)
+    if key_bias.dtype != torch.float32 or key_bias.dim() != 2 or key_bias.shape[0] != b or key_bias.stride(1) != 1:
+      raise ValueError("key_bias must be an f32 [batch, padded kv_length] tensor with a contiguous last axis")
+    rc = _lib.load().mdattn_fwd_bf16_bias(
+        _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), b, h, sq, skv, d,
+        ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale),
+        _ptr(key_bias), key_bias.stride(0))
+    _lib.check(rc, "mdattn_fwd_bf16_bias")
   return (out, lse) if return_lse else out
 
 
