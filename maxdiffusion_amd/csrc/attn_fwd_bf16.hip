@@ -170,7 +170,9 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   // One iteration.  SC holds the logits of block BLK; SN receives those of block BLK+1.
   // KC/KN: K rows of block BLK+1 / BLK+2; VC/VN: V rows of block BLK-1 / BLK.
   // Slot n of the stream: n even -> PV MFMA n/2, n odd -> QK MFMA n/2, each followed by the LDS
-  // request for the MFMA of the same kind three ahead, then a chunk of the softmax of block BLK.
+  // request for the MFMA of the same kind three ahead, then a chunk of the softmax of block BLK.  The
+  // softmax starts at slot 5 (row max) and 7 (exp2 chunks): the last QK MFMA of block BLK was issued at
+  // slot 15 of the previous iteration, and reading its result earlier stalls the wave's whole stream.
 #define MDATTN_ITER(SC, SN, PC, PP, KC, KN, VC, VN, BLK) /* KC.. : base pointers [even j, odd j]; VC.. : [segment] */                                                     \
   {                                                                                                           \
     float alpha = 1.f, mc = 0.f, lsum = 0.f, p[8];                                                            \
@@ -197,7 +199,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
         }                                                                                                     \
         kfr[jn & 3] = *reinterpret_cast<const bf16x8*>((jn < 8 ? (KC) : (KN))[jn & 1] + (jn & 7) * 16);       \
       }                                                                                                       \
-      if (n == 1) {                                                                                           \
+      if (n == 5) {                                                                                           \
         /* row max + lazy-rescale decision: a row's max moves only when it would otherwise see an exp2    */  \
         /* argument above kLazy (per-lane select: the stream stays one basic block); the accumulator      */  \
         /* multiply waits until every PV MFMA of the previous block has been issued (iteration end)       */  \
@@ -212,8 +214,8 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
         mc = m * c;                                                                                           \
         asm volatile("" : "+v"(alpha), "+v"(mc));                                                             \
       }                                                                                                       \
-      if (n >= 3 && n <= 10) {                                                                                \
-        const int e = (n - 3) * 2;                                                                            \
+      if (n >= 7 && n <= 14) {                                                                                \
+        const int e = (n - 7) * 2;                                                                            \
         p[e & 7] = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[e], c, -mc));                                     \
         p[(e & 7) + 1] = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[e + 1], c, -mc));                           \
         lsum += p[e & 7] + p[(e & 7) + 1];                                                                    \
