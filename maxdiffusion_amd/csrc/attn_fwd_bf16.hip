@@ -24,7 +24,9 @@
 //                iteration b every wave issues, interleaved in one instruction stream,
 //                    matrix pipe : O^T += V^T(b-1).P^T(b-1)  (8 MFMAs)  and  S^T(b+1) = K(b+1).Q^T  (8 MFMAs)
 //                    vector ALU  : P(b) = exp2(c*S(b) - c*m), row sums, bf16 convert
-//                    LDS         : the K / V^T fragments of the MFMAs three issues ahead
+//                    LDS         : the K / V^T fragment of the next MFMA of the same kind (a longer look-ahead
+//                                  measured slower: the read would overwrite a register an MFMA issued just
+//                                  before may still be reading)
 //                PV and QK MFMAs alternate, so no MFMA depends on the one issued just before it.  The
 //                loop body is the same for every iteration: the iterations before the first and after
 //                the last real block run on fully masked logits (P = 0) instead of being peeled.
@@ -170,7 +172,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   // One iteration.  SC holds the logits of block BLK; SN receives those of block BLK+1.
   // KC/KN: K rows of block BLK+1 / BLK+2; VC/VN: V rows of block BLK-1 / BLK.
   // Slot n of the stream: n even -> PV MFMA n/2, n odd -> QK MFMA n/2, each followed by the LDS
-  // request for the MFMA of the same kind three ahead, then a chunk of the softmax of block BLK.  The
+  // request for the next MFMA of the same kind, then a chunk of the softmax of block BLK.  The
   // softmax starts at slot 5 (row max) and 7 (exp2 chunks): the last QK MFMA of block BLK was issued at
   // slot 15 of the previous iteration, and reading its result earlier stalls the wave's whole stream.
 #define MDATTN_ITER(SC, SN, PC, PP, KC, KN, VC, VN, BLK) /* KC.. : base pointers [even j, odd j]; VC.. : [segment] */                                                     \
@@ -184,7 +186,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
         if (kv_base + 8 * (i >> 2) + (i & 3) >= a.Skv) SC[i] = -INFINITY;                                     \
     }                                                                                                         \
     _Pragma("unroll") for (int n = 0; n < 16; ++n) {                                                          \
-      const int j = n >> 1, jn = j + 3;                                                                       \
+      const int j = n >> 1, jn = j + 1;                                                                       \
       if ((n & 1) == 0) {                                                                                     \
         O[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[j & 3], PP[j >> 2], O[j & 3], 0, 0, 0);        \
         const __bf16* vsrc = (jn < 8 ? (VC) : (VN))[jn & 3] + ((jn & 7) >> 2) * 4 * kGV;                      \
@@ -237,11 +239,11 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
 
   // ring bookkeeping: period t uses slot t%4 (K(t), V(t-1)) and looks ahead into slot (t+1)%4
   int s_cur = 0, s_nxt = 1, s_nn = 2, s_fill = 3;
-  // fragments the first iteration's first three QK / PV MFMAs expect in the windows
+  // fragments the first iteration's first QK / PV MFMA expect in the windows
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): Q fragments and this wave's share of slots 0..2
   __syncthreads();
 #pragma unroll
-  for (int s = 0; s < 3; ++s) {
+  for (int s = 0; s < 1; ++s) {
     kfr[s] = *reinterpret_cast<const bf16x8*>(smem + ((s & 1) ? k_off_o : k_off_e) + s * 16);
     const __bf16* vsrc = smem + v_off[s];
     vfr[s] = read_vt(vsrc, vsrc + 2 * kGV);
