@@ -100,13 +100,6 @@ int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const void* v, v
                     const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale);
 
 /*
- * Per-tensor absmax quantisation bf16 -> OCP float8 e4m3fn (BASELINE configs[4]; no reference
- * counterpart: the reference's fp8 is qwix quantisation of dense layers, pipelines/wan/wan_pipeline.py:581-626).
- *   x_bf16 [n] contiguous, x_fp8 [n] bytes,
- *   scale_out f32[2] device: [0] = absmax/448 (x ~= x_fp8 * scale_out[0]), [1] = absmax (scratch of the reduction)
- * n % 16 == 0.
- */
-/*
  * The same forward with an additive per-key bias: logits = scale*q.k + key_bias[b, key] (natural-log units;
  * -inf excludes a key).  Replaces: the key padding mask of `_apply_attention` (models/attention_flax.py:1926-1939:
  * a [B,Skv] keep-mask becomes an additive bias; rows whose keys are all masked return 0, :1552-1554) and the
@@ -130,6 +123,13 @@ int mdattn_fwd_bf16_bias(void* stream, const void* q, const void* k, const void*
 int mdattn_key_mask_bias(void* stream, const void* keep, float* bias, int B, int Skv, int64_t bias_stride,
                          float masked_value);
 
+/*
+ * Per-tensor absmax quantisation bf16 -> OCP float8 e4m3fn (BASELINE configs[4]; no reference
+ * counterpart: the reference's fp8 is qwix quantisation of dense layers, pipelines/wan/wan_pipeline.py:581-626).
+ *   x_bf16 [n] contiguous, x_fp8 [n] bytes,
+ *   scale_out f32[2] device: [0] = absmax/448 (x ~= x_fp8 * scale_out[0]), [1] = absmax (scratch of the reduction)
+ * n % 16 == 0.
+ */
 int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, float* scale_out, int64_t n);
 
 /*
