@@ -553,15 +553,16 @@ extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const
   if (rc != MDATTN_OK) return rc;
   hipStream_t st = (hipStream_t)stream;
 
-  // Two schedules.  The software-pipelined kernel (8 waves x 32 query rows, two waves per SIMD) is a little
-  // faster once every CU has many workgroups to go through; the flat kernel (4 waves x 32 rows, three
-  // workgroups per CU) wins on smaller grids.  MDATTN_FWD_VARIANT (1: pipelined 8 waves, 2: pipelined
-  // 4 waves, 3: flat) overrides the choice for experiments and tests.
+  // Two schedules.  The software-pipelined kernel (8 waves x 32 query rows, two waves per SIMD) is the faster one
+  // on long key sequences; its prologue and epilogue (three tiles of look-ahead, one virtual block at each end)
+  // weigh on short ones, where the flat kernel (4 waves x 32 rows, three workgroups per CU) wins: measured
+  // cross-over between 2048 and 4608 keys.  The flat kernel also yields twice the workgroups on tiny grids.
+  // MDATTN_FWD_VARIANT (1: pipelined 8 waves, 2: pipelined 4 waves, 3: flat) overrides the choice.
   int variant = 0;
   if (const char* e = getenv("MDATTN_FWD_VARIANT")) variant = atoi(e);
   if (variant == 0) {
     const int64_t wg256 = (int64_t)B * H * ((Sq + 255) / 256);
-    variant = wg256 >= 4096 ? 1 : 3;
+    variant = (Skv <= 3072 || wg256 < 128) ? 3 : 1;
   }
   switch (variant) {
     case 1: return launch_fwd<8>(st, a, B);
