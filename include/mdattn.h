@@ -83,6 +83,22 @@ int mdattn_norm_rope_perhead(void* stream, const void* q_in, const void* k_in, v
                              const mdattn_strides* in_strides, const mdattn_strides* out_strides);
 
 /*
+ * Full-row RMSNorm + rotary embedding of ONE tensor with position tables that differ per batch element and per
+ * head.  Replaces, for q and for k separately: `norm_q` / `norm_k` (f32 statistics and f32 weight) followed by
+ * `apply_rotary_emb` or `apply_split_rotary_emb` in LTX2Attention.__call__ (models/ltx2/attention_ltx2.py:556-585,
+ * :33-60, :62-102); tables as LTX2RotaryPosEmbed returns them (:292-324).
+ *   x_in         [B,S,H*D] bf16 (x_is_f32 = 0) or f32 (1), strides in elements
+ *   x_out        bf16 [B,S,H,D] by out_strides
+ *   w            f32 [H*D]
+ *   rope_mode    0: norm only (cross-attention keys);  1: interleaved, cos/sin f32 [B,S,H*D];
+ *                2: split, cos/sin f32 [B,H,S,D/2]
+ * Requires D % 16 == 0 and H*D <= 8192.
+ */
+int mdattn_norm_rope_rows(void* stream, const void* x_in, int x_is_f32, void* x_out, const float* w,
+                          const float* cos, const float* sin, int rope_mode, int B, int S, int H, int D, float eps,
+                          int64_t in_stride_batch, int64_t in_stride_seq, const mdattn_strides* out_strides);
+
+/*
  * Non-causal softmax attention forward, bf16 MFMA, online softmax in f32, optional LSE.
  * Replaces: the kernel a KERNEL_REGISTRY entry dispatches to (models/attention_flax.py:1589-1597,
  * :1965-1966), i.e. what _tpu_flash_attention (:563-809) / kernels/custom_splash_attention.py:69-320

@@ -21,7 +21,7 @@ from . import ops
 
 __all__ = [
     "KERNEL_REGISTRY", "register_kernel", "AttentionOp", "hip_flash_kernel", "hip_flash_fp8_kernel",
-    "hip_norm_rope", "HIP_KERNEL_NAMES",
+    "hip_norm_rope", "hip_norm_rope_ltx2", "HIP_KERNEL_NAMES",
 ]
 
 KERNEL_REGISTRY = {}
@@ -113,6 +113,33 @@ def hip_flash_fp8_kernel(q, k, v, context):
   out = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=context["scale"])
   b, s, h, d = out.shape
   return out.reshape(b, s, h * d).to(q.dtype)
+
+
+
+def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotary_emb=None, k_rotary_emb=None,
+                       rope_type: str = "interleaved", is_self_attention: bool = True, eps: float = 1e-6):
+  """Fused prologue of LTX2Attention.__call__ (models/ltx2/attention_ltx2.py:556-585).
+
+  query/key [B,S,H*D] (bf16 or f32) are normalised over the full inner dim with the f32 scales; the query is rotated
+  by `rotary_emb`, the key by `k_rotary_emb` if given, else by `rotary_emb` when this is self-attention, else not
+  at all.  Tables are (cos, sin) as LTX2RotaryPosEmbed returns them: [B,S,H*D] (interleaved) or [B,H,S,D/2] (split).
+  Returns (q, k) bf16 [B,S,H,D], ready for `hip_flash`.  `key` None (cached K/V): only the query is processed."""
+  if rope_type not in ("interleaved", "split"):
+    raise ValueError(f"{rope_type=} not supported. Choose between 'interleaved' and 'split'.")  # :145-146
+  q_tab = rotary_emb
+  k_tab = k_rotary_emb if k_rotary_emb is not None else (rotary_emb if is_self_attention else None)
+  if rotary_emb is None:
+    q_tab = k_tab = None
+
+  def run(x, scale, tab):
+    if tab is None:
+      return ops.norm_rope_rows(x, scale, heads=heads, mode="none", eps=eps)
+    cos, sin = (t.to(torch.float32).contiguous() for t in tab)
+    return ops.norm_rope_rows(x, scale, cos, sin, heads=heads, mode=rope_type, eps=eps)
+
+  q = run(query, norm_q_scale, q_tab)
+  k = run(key, norm_k_scale, k_tab) if key is not None else None
+  return q, k
 
 
 def _apply_attention(

@@ -189,6 +189,120 @@ __global__ __launch_bounds__(256) void norm_rope_perhead_kernel(NormRopeHeadArgs
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// One tensor at a time, with position tables that differ per batch element and per head (LTX-2):
+// full-row RMSNorm with an f32 weight, then either the interleaved rotation with full-size tables
+// [B,S,H*D] (out = x*cos + rot(x)*sin, rot pairs neighbours as (-x1, x0)) or the split rotation with
+// tables [B,H,S,D/2] (element i of a head pairs with element i + D/2).  A lane works on "units" of two
+// 8-element chunks of one head, c and c + D/16, which holds both partners of either pairing.
+struct NormRopeRowsArgs {
+  const void* x_in;
+  uint4* x_out;
+  const float* w;
+  const float* cos;
+  const float* sin;
+  int S, H, D, N, mode;  // mode 0: no rotation, 1: interleaved, 2: split
+  float eps, inv_n;
+  int64_t in_sb, in_ss;
+  int64_t out_sb, out_ss, out_sh;
+};
+
+template <int MAXU, bool F32IN>
+__global__ __launch_bounds__(256) void norm_rope_rows_kernel(NormRopeRowsArgs a) {
+  const int tid = threadIdx.x;
+  const int s = blockIdx.x, b = blockIdx.y;
+  const int cph = a.D >> 4;            // chunk pairs (units) per head
+  const int nunits = a.H * cph;
+  __shared__ float red[16];
+
+  float x[MAXU][16];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < MAXU; ++i) {
+    const int u = tid + i * 256;
+    if (u < nunits) {
+      const int h = u / cph, c = u - h * cph;
+      const int64_t e0 = b * a.in_sb + s * a.in_ss + h * a.D + c * 8;  // first chunk; partner at + D/2
+      if (F32IN) {
+        const float4* p0 = reinterpret_cast<const float4*>(static_cast<const float*>(a.x_in) + e0);
+        const float4* p1 = reinterpret_cast<const float4*>(static_cast<const float*>(a.x_in) + e0 + (a.D >> 1));
+        const float4 v0 = ld_nt(p0), v1 = ld_nt(p0 + 1), v2 = ld_nt(p1), v3 = ld_nt(p1 + 1);
+        const float t[16] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w, v2.x, v2.y, v2.z, v2.w, v3.x, v3.y, v3.z, v3.w};
+#pragma unroll
+        for (int j = 0; j < 16; ++j) x[i][j] = t[j];
+      } else {
+        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const __bf16*>(a.x_in) + e0);
+        unpack8(ld_nt(p), x[i]);
+        unpack8(ld_nt(p + (a.D >> 4)), x[i] + 8);
+      }
+#pragma unroll
+      for (int j = 0; j < 16; ++j) ss = __builtin_fmaf(x[i][j], x[i][j], ss);
+    }
+  }
+  ss = row16_sum(ss);
+  if ((tid & 15) == 0) red[tid >> 4] = ss;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) tot += red[j];
+  const float xx = tot * a.inv_n + a.eps;
+  const float y0 = __builtin_amdgcn_rsqf(xx);
+  const float inv = y0 * (1.5f - 0.5f * xx * y0 * y0);
+
+#pragma unroll
+  for (int i = 0; i < MAXU; ++i) {
+    const int u = tid + i * 256;
+    if (u < nunits) {
+      const int h = u / cph, c = u - h * cph;
+      const int half = a.D >> 1;
+      const float4* wp0 = reinterpret_cast<const float4*>(a.w + h * a.D + c * 8);
+      const float4* wp1 = reinterpret_cast<const float4*>(a.w + h * a.D + c * 8 + half);
+      const float4 w0 = wp0[0], w1 = wp0[1], w2 = wp1[0], w3 = wp1[1];
+      const float w[16] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w, w2.x, w2.y, w2.z, w2.w, w3.x, w3.y, w3.z, w3.w};
+      float y[16], o[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) y[j] = x[i][j] * inv * w[j];
+      if (a.mode == 1) {
+        // tables [B,S,H*D]: one cos and one sin per element
+        const int64_t t0 = ((int64_t)b * a.S + s) * a.N + h * a.D + c * 8;
+#pragma unroll
+        for (int part = 0; part < 2; ++part) {
+          const float4* cp = reinterpret_cast<const float4*>(a.cos + t0 + part * half);
+          const float4* sp = reinterpret_cast<const float4*>(a.sin + t0 + part * half);
+          const float4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
+          const float cc[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+          const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float x0 = y[part * 8 + 2 * j], x1 = y[part * 8 + 2 * j + 1];
+            o[part * 8 + 2 * j] = x0 * cc[2 * j] - x1 * sv[2 * j];
+            o[part * 8 + 2 * j + 1] = x1 * cc[2 * j + 1] + x0 * sv[2 * j + 1];
+          }
+        }
+      } else if (a.mode == 2) {
+        // tables [B,H,S,D/2]: element c*8+e of the first half pairs with the same element of the second half
+        const int64_t t0 = (((int64_t)b * a.H + h) * a.S + s) * half + c * 8;
+        const float4* cp = reinterpret_cast<const float4*>(a.cos + t0);
+        const float4* sp = reinterpret_cast<const float4*>(a.sin + t0);
+        const float4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
+        const float cc[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+        const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          o[j] = y[j] * cc[j] - y[8 + j] * sv[j];
+          o[8 + j] = y[8 + j] * cc[j] + y[j] * sv[j];
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) o[j] = y[j];
+      }
+      uint4* dst = a.x_out + ((b * a.out_sb + s * a.out_ss + h * a.out_sh + c * 8) >> 3);
+      st_nt(dst, pack8(o));
+      st_nt(dst + (a.D >> 4), pack8(o + 8));
+    }
+  }
+}
+
 }  // namespace mdattn
 
 using namespace mdattn;
@@ -265,3 +379,36 @@ extern "C" int mdattn_norm_rope_perhead(void* stream, const void* q_in, const vo
   else hipLaunchKernelGGL((norm_rope_perhead_kernel<32, RPT>), grid, block, 0, st, a);
   return launch_status();
 }
+
+extern "C" int mdattn_norm_rope_rows(void* stream, const void* x_in, int x_is_f32, void* x_out, const float* w,
+                                     const float* cos, const float* sin, int rope_mode, int B, int S, int H, int D,
+                                     float eps, int64_t in_stride_batch, int64_t in_stride_seq,
+                                     const mdattn_strides* out_strides) {
+  if (!x_in || !x_out || !w || B <= 0 || S <= 0 || H <= 0 || D <= 0 || !out_strides) return MDATTN_E_BADARG;
+  if (rope_mode < 0 || rope_mode > 2 || (rope_mode != 0 && (!cos || !sin)) || !(eps >= 0.f)) return MDATTN_E_BADARG;
+  if (B > 65535) return MDATTN_E_UNSUPPORTED;
+  if (D % 16 != 0) return MDATTN_E_UNSUPPORTED;
+  const int64_t N = (int64_t)H * D;
+  if (N / 16 > 2 * 256) return MDATTN_E_UNSUPPORTED;  // up to 8192 channels per row
+  const int in_mult = x_is_f32 ? 4 : 8;
+  if (!aligned16(x_in) || !aligned16(x_out) || !aligned16(w) || !aligned16(cos) || !aligned16(sin)) return MDATTN_E_ALIGN;
+  if (in_stride_batch % in_mult || in_stride_seq % in_mult || in_stride_seq < N || !strides_ok(out_strides, 8)) return MDATTN_E_ALIGN;
+  if (out_strides->head < D) return MDATTN_E_BADARG;
+  NormRopeRowsArgs a;
+  a.x_in = x_in; a.x_out = (uint4*)x_out; a.w = w; a.cos = cos; a.sin = sin;
+  a.S = S; a.H = H; a.D = D; a.N = (int)N; a.mode = rope_mode; a.eps = eps; a.inv_n = 1.0f / (float)N;
+  a.in_sb = in_stride_batch; a.in_ss = in_stride_seq;
+  a.out_sb = out_strides->batch; a.out_ss = out_strides->seq; a.out_sh = out_strides->head;
+  dim3 grid(S, B), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  const bool two = N / 16 > 256;
+  if (x_is_f32) {
+    if (two) hipLaunchKernelGGL((norm_rope_rows_kernel<2, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((norm_rope_rows_kernel<1, true>), grid, block, 0, st, a);
+  } else {
+    if (two) hipLaunchKernelGGL((norm_rope_rows_kernel<2, false>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((norm_rope_rows_kernel<1, false>), grid, block, 0, st, a);
+  }
+  return launch_status();
+}
+

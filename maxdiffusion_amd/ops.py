@@ -16,7 +16,7 @@ from . import _lib
 from ._lib import Strides
 
 __all__ = [
-    "norm_rope_fullrow", "norm_rope_perhead", "flash_attention", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
+    "norm_rope_fullrow", "norm_rope_perhead", "norm_rope_rows", "flash_attention", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
     "merge_partial", "finalize", "new_merge_state", "LSE_INIT",
 ]
 
@@ -83,6 +83,35 @@ def norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6, out
       b, s, heads, d, eps, q.stride(0), q.stride(1), ctypes.byref(st))
   _lib.check(rc, "mdattn_norm_rope_fullrow")
   return q_out, k_out
+
+
+def norm_rope_rows(x, w, cos=None, sin=None, heads: int = 1, mode: str = "none", eps: float = 1e-6, out_layout: str = "bshd"):
+  """One tensor x [B,S,H*D] (bf16 or f32) -> bf16 logical [B,S,H,D]: full-row RMSNorm with the f32 weight w [H*D],
+  then `mode` "none", "interleaved" (cos/sin f32 [B,S,H*D]) or "split" (cos/sin f32 [B,H,S,D/2])."""
+  _check_dev(x, w, cos, sin)
+  if x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float32) or x.stride(2) != 1:
+    raise ValueError("x must be bf16 or f32 [B, S, H*D] with a contiguous last axis")
+  b, s, n = x.shape
+  if n % heads:
+    raise ValueError(f"inner dim {n} is not divisible by heads={heads}")
+  d = n // heads
+  modes = {"none": 0, "interleaved": 1, "split": 2}
+  if mode not in modes:
+    raise ValueError(f"mode={mode!r} not supported. Choose between 'none', 'interleaved' and 'split'.")
+  if w.dtype != torch.float32 or w.numel() != n or not w.is_contiguous():
+    raise ValueError("w must be a contiguous f32 [H*D] tensor")
+  if mode != "none":
+    want = (b, s, n) if mode == "interleaved" else (b, heads, s, d // 2)
+    for name, t in (("cos", cos), ("sin", sin)):
+      if t is None or tuple(t.shape) != want or t.dtype != torch.float32 or not t.is_contiguous():
+        raise ValueError(f"{name} must be a contiguous f32 tensor of shape {want} for mode={mode!r}")
+  out = _alloc_like_layout(b, s, heads, d, out_layout, torch.bfloat16, x.device)
+  st = _strides(out)
+  rc = _lib.load().mdattn_norm_rope_rows(
+      _stream(), _ptr(x), int(x.dtype == torch.float32), _ptr(out), _ptr(w), _ptr(cos if mode != "none" else None),
+      _ptr(sin if mode != "none" else None), modes[mode], b, s, heads, d, eps, x.stride(0), x.stride(1), ctypes.byref(st))
+  _lib.check(rc, "mdattn_norm_rope_rows")
+  return out
 
 
 def norm_rope_perhead(q, k, wq, wk, cos, sin, eps: float = 1e-6, wq_txt=None, wk_txt=None, n_txt: int = 0,

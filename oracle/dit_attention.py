@@ -18,6 +18,9 @@ Pinning status of each function (what fixes it besides its own formula):
                                  tuple form == matrix form of apply_rope
   apply_rope_interleaved         complex128 multiply, composition, inverse,
                                  relative-position property
+  ltx2_apply_rotary_emb          equals apply_rope_interleaved on repeat-interleaved tables
+  ltx2_apply_split_rotary_emb    brute-force loop, norm preservation, and: split rotation of x equals
+                                 the interleaved rotation of x with each head's halves interleaved
   attention / attention_rows     scipy logsumexp, torch SDPA (fp32, CPU),
                                  invariants (K=0 -> mean(V), lse=ln Skv; ...),
                                  hand fixtures of tests/ltx2/test_attention_ltx2.py:38-116
@@ -42,7 +45,7 @@ __all__ = [
     "flux_ids", "flux_rope_angles", "flux_rope_table", "flux_rope_table_matrix",
     "apply_rope_interleaved", "apply_rope_matrix_form", "norm_rope_fullrow", "norm_rope_perhead",
     "norm_rope_wan_reference_flow", "attention", "attention_rows", "attention_dot_product_bf16",
-    "merge_lse", "merge_mlo", "merge_scan_ring", "ring_replay", "quant_e4m3", "attention_fp8_emulated",
+    "ltx2_apply_rotary_emb", "ltx2_apply_split_rotary_emb", "norm_rope_ltx2", "merge_lse", "merge_mlo", "merge_scan_ring", "ring_replay", "quant_e4m3", "attention_fp8_emulated",
     "LSE_INIT",
 ]
 
@@ -305,6 +308,42 @@ def attention_dot_product_bf16(q, k, v, scale: float):
   e = np.exp(s - m)
   p = bf16_round(e / e.sum(axis=-1, keepdims=True))
   return bf16_round(np.matmul(p, v))
+
+
+# --------------------------------------------------------------------------- LTX-2 rotary forms
+def ltx2_apply_rotary_emb(x, cos, sin, dtype=np.float64):
+  """Interleaved rotation with full-size tables: out = x*cos + rot(x)*sin, rot pairs neighbours as
+  (-x[2j+1], x[2j]) (models/ltx2/attention_ltx2.py:33-60).  x, cos, sin broadcast to [..., H*D]."""
+  x = np.asarray(x, dtype)
+  xr = x.reshape(*x.shape[:-1], -1, 2)
+  rot = np.stack([-xr[..., 1], xr[..., 0]], axis=-1).reshape(x.shape)
+  return x * np.asarray(cos, dtype) + rot * np.asarray(sin, dtype)
+
+
+def ltx2_apply_split_rotary_emb(x, cos, sin, dtype=np.float64):
+  """Split rotation (models/ltx2/attention_ltx2.py:62-102): x [B,S,H*D], cos/sin [B,H,S,D/2]; inside a head,
+  element i of the first half pairs with element i of the second half."""
+  x = np.asarray(x, dtype)
+  cos, sin = np.asarray(cos, dtype), np.asarray(sin, dtype)
+  b, s, n = x.shape
+  h, r = cos.shape[1], cos.shape[3]
+  xh = x.reshape(b, s, h, 2, r).transpose(0, 2, 1, 3, 4)  # [B,H,S,2,r]
+  first, second = xh[..., 0, :], xh[..., 1, :]
+  out = np.stack([first * cos - second * sin, second * cos + first * sin], axis=-2)  # [B,H,S,2,r]
+  return out.transpose(0, 2, 1, 3, 4).reshape(b, s, n)
+
+
+def norm_rope_ltx2(x, w, cos, sin, mode: str, eps: float = 1e-6, dtype=np.float64):
+  """LTX2Attention's prologue for one tensor (attention_ltx2.py:556-585): full-row RMSNorm with an f32 weight,
+  then no rotation (`mode` "none": cross-attention keys), the interleaved or the split one.  x [B,S,H*D]."""
+  y = rmsnorm(x, w, eps, dtype)
+  if mode == "none":
+    return y
+  if mode == "interleaved":
+    return ltx2_apply_rotary_emb(y, cos, sin, dtype)
+  if mode == "split":
+    return ltx2_apply_split_rotary_emb(y, cos, sin, dtype)
+  raise ValueError(mode)
 
 
 # --------------------------------------------------------------------------- A6 merges

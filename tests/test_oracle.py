@@ -298,6 +298,63 @@ def test_merge_algebra_and_mlo_form():
   np.testing.assert_allclose(mm + np.log(ll), ab[1], rtol=1e-12)
 
 
+# ----------------------------------------------------------------------------- LTX-2 rotary forms
+def _pair_rotate(x, ang):
+  """Neighbouring pairs as complex numbers times exp(i*angle): x [..., 2n], ang [..., n]."""
+  z = (x[..., 0::2] + 1j * x[..., 1::2]) * np.exp(1j * ang)
+  out = np.empty_like(x)
+  out[..., 0::2], out[..., 1::2] = z.real, z.imag
+  return out
+
+
+def test_ltx2_interleaved_form_equals_pair_rotation():
+  rng = np.random.default_rng(11)
+  B, S, H, D = 2, 5, 3, 16
+  x = rng.standard_normal((B, S, H * D))
+  ang = rng.uniform(-3, 3, (B, S, H * D // 2))
+  cos, sin = np.repeat(np.cos(ang), 2, axis=-1), np.repeat(np.sin(ang), 2, axis=-1)  # attention_ltx2.py:292-295
+  got = O.ltx2_apply_rotary_emb(x, cos, sin)
+  np.testing.assert_allclose(got, _pair_rotate(x, ang), rtol=0, atol=1e-14)
+
+
+def test_ltx2_split_form_brute_force_and_permutation_identity():
+  rng = np.random.default_rng(12)
+  B, S, H, D = 2, 4, 3, 8
+  r = D // 2
+  x = rng.standard_normal((B, S, H * D))
+  ang = rng.uniform(-3, 3, (B, H, S, r))
+  got = O.ltx2_apply_split_rotary_emb(x, np.cos(ang), np.sin(ang))
+  want = np.empty_like(x)
+  for b in range(B):
+    for s in range(S):
+      for h in range(H):
+        for i in range(r):
+          f, g = x[b, s, h * D + i], x[b, s, h * D + r + i]
+          c, sn = math.cos(ang[b, h, s, i]), math.sin(ang[b, h, s, i])
+          want[b, s, h * D + i] = f * c - g * sn
+          want[b, s, h * D + r + i] = g * c + f * sn
+  np.testing.assert_allclose(got, want, rtol=0, atol=1e-14)
+  # a rotation: every (i, i + D/2) pair keeps its length
+  xh, gh = x.reshape(B, S, H, 2, r), got.reshape(B, S, H, 2, r)
+  np.testing.assert_allclose((gh**2).sum(axis=3), (xh**2).sum(axis=3), rtol=1e-12)
+  # interleaving each head's halves turns the split form into the interleaved one
+  xi = xh.transpose(0, 1, 2, 4, 3).reshape(B, S, H * D)
+  ang_bs = ang.transpose(0, 2, 1, 3).reshape(B, S, H * r)
+  via = _pair_rotate(xi, ang_bs).reshape(B, S, H, r, 2).transpose(0, 1, 2, 4, 3).reshape(B, S, H * D)
+  np.testing.assert_allclose(got, via, rtol=0, atol=1e-14)
+
+
+def test_norm_rope_ltx2_modes():
+  rng = np.random.default_rng(13)
+  x = rng.standard_normal((1, 3, 32))
+  w = 1 + 0.1 * rng.standard_normal(32)
+  y = O.rmsnorm(x, w)
+  np.testing.assert_array_equal(O.norm_rope_ltx2(x, w, None, None, "none"), y)
+  zeros = np.zeros((1, 3, 32))
+  np.testing.assert_allclose(O.norm_rope_ltx2(x, w, zeros + 1, zeros, "interleaved"), y, atol=1e-15)
+  np.testing.assert_allclose(O.norm_rope_ltx2(x, w, np.ones((1, 2, 3, 8)), np.zeros((1, 2, 3, 8)), "split"), y, atol=1e-15)
+
+
 # ----------------------------------------------------------------------------- fp8 emulation
 def test_fp8_emulation_meets_cosine_bar():
   q = O.normal_bf16((2, 128, 128), 0)
