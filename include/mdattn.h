@@ -108,7 +108,8 @@ int mdattn_norm_rope_rows(void* stream, const void* x_in, int x_is_f32, void* x_
  *   lse          f32 [B,H,Sq] contiguous or NULL: natural-log logsumexp of scale*q.k
  *                (kernels/splash_attention/base.py:103-105)
  *   scale        applied to q.k inside the kernel (the reference pre-multiplies k, :1783)
- * Requires D == 128.  Any Sq, Skv >= 1 (ragged tails handled in-kernel).
+ * Requires D == 128, or D == 64 (LTX-2's audio stream, models/ltx2/transformer_ltx2.py:788-789).  Any Sq, Skv >= 1
+ * (ragged tails handled in-kernel).
  */
 int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* out, float* lse,
                     int B, int H, int Sq, int Skv, int D,

@@ -300,17 +300,25 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
 // 3-slot ring (50 KB of LDS) and at most 168 VGPRs, so that three workgroups share a CU and three waves
 // share each SIMD: while one wave runs its softmax on the vector ALU the other two keep the matrix
 // pipe busy.  Same tile layouts, same fragment reads, same arithmetic as the pipelined kernel.
+// Head dim 64 (template HD) uses 128-byte rows: one load instruction fills 8 rows, K chunk c of row r sits at
+// position c ^ ((r >> 1) & 7), V chunk c at c ^ 4*((r >> 1) & 1), both unpadded and conflict-free for the
+// same two read patterns.
 constexpr int kTS = 32;                               // keys per tile
 constexpr int kKTileS = (kTS / 4) * kGK;              // elements
 constexpr int kStageS = kKTileS + (kTS / 4) * kGV;    // elements per ring slot
 constexpr int kSlotsS = 3;
 
-template <int NW, bool BIAS>
+template <int NW, bool BIAS, int HD>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_fwd_bf16_flat_kernel(AttnArgs a) {
+  constexpr int NJ = HD / 16;                                    // QK MFMAs per 32-key tile
+  constexpr int ND = HD / 32;                                    // 32-wide slabs of d = O accumulators
+  constexpr int KTILE = HD == 128 ? kKTileS : kTS * 64;          // elements
+  constexpr int STAGE = HD == 128 ? kStageS : 2 * kTS * 64;
+  constexpr int RPI = HD == 128 ? 4 : 8;                          // rows one load instruction fills
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
   constexpr int BM = NW * 32;
-  constexpr int GPW = (kTS / 4) / NW;  // 4-row groups per wave, tile and tensor
+  constexpr int GPW = (kTS / RPI) / NW;  // row groups per wave, tile and tensor
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -332,69 +340,85 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   const float cs = BIAS ? 1.0f : c;
   const float* bias_row = BIAS ? a.bias + b * a.bias_sb + 4 * hh : nullptr;
 
-  bf16x8 qf[8];
+  bf16x8 qf[NJ];
   {
     int row = q0 + l32;
     row = row < a.Sq ? row : a.Sq - 1;
     const __bf16* p = qp + (int64_t)row * a.q_ss + hh * 8;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(p + s * 16);
+    for (int s = 0; s < NJ; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(p + s * 16);
   }
 
-  const int grow = lane >> 4;
-  const int kcol = ((lane & 15) ^ grow) * 8;
-  const int vcol = ((lane & 15) ^ (grow << 2)) * 8;
+  // lane -> (row of the group, logical 16-byte chunk stored at this lane's position)
+  const int grow = HD == 128 ? lane >> 4 : lane >> 3;
+  const int kcol = HD == 128 ? ((lane & 15) ^ grow) * 8 : ((lane & 7) ^ ((4 * (wave & 1) + (grow >> 1)) & 7)) * 8;
+  const int vcol = HD == 128 ? ((lane & 15) ^ (grow << 2)) * 8 : ((lane & 7) ^ (((grow >> 1) & 1) << 2)) * 8;
+  constexpr int KGS = HD == 128 ? kGK : 8 * 64;  // group strides in LDS, elements
+  constexpr int VGS = HD == 128 ? kGV : 8 * 64;
   const unsigned kofs = (unsigned)(grow * (int)a.k_ss + kcol) * 2u;
   const unsigned vofs = (unsigned)(grow * (int)a.v_ss + vcol) * 2u;
   const unsigned smem_addr = lds_addr_of(smem);
   auto dma = [&](int slot, int kt) __attribute__((always_inline)) {
-    const unsigned Ks = smem_addr + (unsigned)(slot * kStageS) * 2u;
-    const unsigned Vs = Ks + kKTileS * 2u;
+    const unsigned Ks = smem_addr + (unsigned)(slot * STAGE) * 2u;
+    const unsigned Vs = Ks + KTILE * 2u;
     if (kt * kTS + kTS <= a.Skv) {
-      const __bf16* kt0 = kp + (int64_t)(kt * kTS + 4 * wave) * a.k_ss;
-      const __bf16* vt0 = vp + (int64_t)(kt * kTS + 4 * wave) * a.v_ss;
+      const __bf16* kt0 = kp + (int64_t)(kt * kTS + RPI * wave) * a.k_ss;
+      const __bf16* vt0 = vp + (int64_t)(kt * kTS + RPI * wave) * a.v_ss;
 #pragma unroll
       for (int i = 0; i < GPW; ++i) {
-        lds_dma16(kt0 + (int64_t)(4 * NW * i) * a.k_ss, kofs, Ks + (unsigned)((wave + NW * i) * kGK) * 2u);
-        lds_dma16(vt0 + (int64_t)(4 * NW * i) * a.v_ss, vofs, Vs + (unsigned)((wave + NW * i) * kGV) * 2u);
+        lds_dma16(kt0 + (int64_t)(RPI * NW * i) * a.k_ss, kofs, Ks + (unsigned)((wave + NW * i) * KGS) * 2u);
+        lds_dma16(vt0 + (int64_t)(RPI * NW * i) * a.v_ss, vofs, Vs + (unsigned)((wave + NW * i) * VGS) * 2u);
       }
     } else {
 #pragma unroll
       for (int i = 0; i < GPW; ++i) {
         const int g = wave + NW * i;
-        int kk = kt * kTS + 4 * g + grow;
+        int kk = kt * kTS + RPI * g + grow;
         kk = kk < a.Skv ? kk : a.Skv - 1;
-        lds_dma16(kp + (int64_t)kk * a.k_ss + kcol, Ks + (unsigned)(g * kGK) * 2u);
-        lds_dma16(vp + (int64_t)kk * a.v_ss + vcol, Vs + (unsigned)(g * kGV) * 2u);
+        lds_dma16(kp + (int64_t)kk * a.k_ss + kcol, Ks + (unsigned)(g * KGS) * 2u);
+        lds_dma16(vp + (int64_t)kk * a.v_ss + vcol, Vs + (unsigned)(g * VGS) * 2u);
       }
     }
   };
 
-  f32x16 O[4];
+  f32x16 O[ND];
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < ND; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[db][i] = 0.f;
   float m = -1e30f, l = 0.f;
 
-  const int kx0 = l32 & 1, kx1 = (l32 >> 1) & 1;
-  const int k_base = (l32 >> 2) * kGK + (l32 & 3) * kD + (hh ^ kx0) * 8;
-  const int k_off_e = k_base + 16 * kx1, k_off_o = k_base - 16 * kx1;
+  // per-lane fragment offsets (elements): K fragment j, V slab sg; kV8 = offset of the second transposing read
+  // (rows + 8), kVH = offset of the second 16-key half of the tile
   const int vxr = (lane & 15) >> 2;
-  int v_off[4];
+  int k_off[NJ], v_off[ND];
+  constexpr int kV8 = HD == 128 ? 2 * kGV : 8 * 64, kVH = HD == 128 ? 4 * kGV : 16 * 64;
+  if constexpr (HD == 128) {
+    const int kx0 = l32 & 1, kx1 = (l32 >> 1) & 1;
+    const int k_base = (l32 >> 2) * kGK + (l32 & 3) * kD + (hh ^ kx0) * 8;
 #pragma unroll
-  for (int sg = 0; sg < 4; ++sg)
-    v_off[sg] = kKTileS + hh * kGV + vxr * kD + (sg ^ vxr) * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+    for (int j = 0; j < NJ; ++j) k_off[j] = k_base + ((j & 1) ? -16 : 16) * kx1 + j * 16;
+#pragma unroll
+    for (int sg = 0; sg < ND; ++sg)
+      v_off[sg] = KTILE + hh * kGV + vxr * kD + (sg ^ vxr) * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+  } else {
+    const int kx = (l32 >> 1) & 7, vx = (vxr >> 1) & 1;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) k_off[j] = l32 * 64 + (((2 * j + hh) ^ kx) * 8);
+#pragma unroll
+    for (int sg = 0; sg < ND; ++sg)
+      v_off[sg] = KTILE + (4 * hh + vxr) * 64 + (sg ^ vx) * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+  }
 
   auto tile = [&](int t, int slot, auto masked) __attribute__((always_inline)) {
-    const __bf16* base = smem + slot * kStageS;
-    // ---- S^T = K.Q^T: one chain of 8 MFMAs; the other waves of the SIMD fill the gaps between them
+    const __bf16* base = smem + slot * STAGE;
+    // ---- S^T = K.Q^T: one chain of MFMAs; the other waves of the SIMD fill the gaps between them
     f32x16 S;
 #pragma unroll
     for (int i = 0; i < 16; ++i) S[i] = 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + ((j & 1) ? k_off_o : k_off_e) + j * 16);
+    for (int j = 0; j < NJ; ++j) {
+      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + k_off[j]);
       S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[j], S, 0, 0, 0);
     }
     if constexpr (BIAS) {
@@ -424,7 +448,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       m = mnew;
       l *= alpha;
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int db = 0; db < ND; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[db][i] *= alpha;
     }
@@ -444,10 +468,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
     l += lsum;
     // ---- O^T += V^T.P^T
 #pragma unroll
-    for (int jv = 0; jv < 8; ++jv) {
-      const __bf16* vsrc = base + v_off[jv & 3] + (jv >> 2) * 4 * kGV;
-      const bf16x8 vf = read_vt(vsrc, vsrc + 2 * kGV);
-      O[jv & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P[jv >> 2], O[jv & 3], 0, 0, 0);
+    for (int jv = 0; jv < 2 * ND; ++jv) {
+      const __bf16* vsrc = base + v_off[jv % ND] + (jv / ND) * kVH;
+      const bf16x8 vf = read_vt(vsrc, vsrc + kV8);
+      O[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P[jv / ND], O[jv % ND], 0, 0, 0);
     }
   };
 
@@ -473,7 +497,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   if (row < a.Sq) {
     __bf16* orow = op + (int64_t)row * a.o_ss + 4 * hh;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < ND; ++db)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         uint2 u;
@@ -485,16 +509,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   }
 }
 
-template <int NW, bool BIAS>
+template <int NW, bool BIAS, int HD = 128>
 static int launch_flat(hipStream_t st, AttnArgs a, int B) {
   constexpr int BM = NW * 32;
-  constexpr int lds_bytes = kSlotsS * kStageS * 2;
+  constexpr int lds_bytes = kSlotsS * (HD == 128 ? kStageS : 2 * kTS * 64) * 2;
   a.nqt = (a.Sq + BM - 1) / BM;
   const int64_t total = (int64_t)B * a.H * a.nqt;
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
-  hipLaunchKernelGGL((attn_fwd_bf16_flat_kernel<NW, BIAS>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  hipLaunchKernelGGL((attn_fwd_bf16_flat_kernel<NW, BIAS, HD>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   return launch_status();
 }
 
@@ -525,7 +549,7 @@ static int fill_args(AttnArgs& a, const void* q, const void* k, const void* v, v
   if (!q || !k || !v || !out || B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return MDATTN_E_BADARG;
   if (!q_strides || !k_strides || !v_strides || !o_strides) return MDATTN_E_BADARG;
   if (!(scale > 0.f) || !(scale < 1e30f)) return MDATTN_E_BADARG;
-  if (D != kD) return MDATTN_E_UNSUPPORTED;
+  if (D != kD && D != 64) return MDATTN_E_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || (reinterpret_cast<uintptr_t>(lse) & 3u))
     return MDATTN_E_ALIGN;
   if (!strides_ok(q_strides, 8) || !strides_ok(k_strides, 8) || !strides_ok(v_strides, 8) || !strides_ok(o_strides, 8))
@@ -552,6 +576,7 @@ extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const
   const int rc = fill_args(a, q, k, v, out, lse, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides, scale);
   if (rc != MDATTN_OK) return rc;
   hipStream_t st = (hipStream_t)stream;
+  if (D == 64) return launch_flat<4, false, 64>(st, a, B);  // head dim 64: the flat schedule only
 
   // Two schedules.  The software-pipelined kernel (8 waves x 32 query rows, two waves per SIMD) is the faster one
   // on long key sequences; its prologue and epilogue (three tiles of look-ahead, one virtual block at each end)
@@ -584,5 +609,6 @@ extern "C" int mdattn_fwd_bf16_bias(void* stream, const void* q, const void* k, 
   if (!aligned16(key_bias)) return MDATTN_E_ALIGN;
   a.bias = key_bias;
   a.bias_sb = bias_stride;
+  if (D == 64) return launch_flat<4, true, 64>((hipStream_t)stream, a, B);
   return launch_flat<4, true>((hipStream_t)stream, a, B);
 }

@@ -68,7 +68,7 @@ def test_bad_arguments_are_rejected_on_the_host(lib):
   assert f(None, fake, fake, fake, fake, None, 1, 4, 0, 8, 128, st, st, st, st, 0.1) == _lib.E_BADARG
   assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 128, st, st, st, st, 0.0) == _lib.E_BADARG
   assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 128, st, st, st, st, float("nan")) == _lib.E_BADARG
-  assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 64, st, st, st, st, 0.1) == _lib.E_UNSUPPORTED
+  assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 32, st, st, st, st, 0.1) == _lib.E_UNSUPPORTED
   assert f(None, odd, fake, fake, fake, None, 1, 4, 8, 8, 128, st, st, st, st, 0.1) == _lib.E_ALIGN
   assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 128, _st(0, 516, 129), st, st, st, 0.1) == _lib.E_ALIGN
   assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 128, None, st, st, st, 0.1) == _lib.E_BADARG

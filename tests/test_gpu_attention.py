@@ -213,6 +213,28 @@ def test_host_side_validation_raises(dev):
     ops.flash_attention(q, q[:, :, :1], q[:, :, :1])
   from maxdiffusion_amd._lib import MdattnError
 
-  q64 = torch.zeros((1, 8, 2, 64), dtype=torch.bfloat16, device=dev)
+  q32 = torch.zeros((1, 8, 2, 32), dtype=torch.bfloat16, device=dev)  # head dims other than 128 and 64
   with pytest.raises(MdattnError, match="unsupported"):
-    ops.flash_attention(q64, q64, q64)
+    ops.flash_attention(q32, q32, q32)
+
+
+@pytest.mark.parametrize("sq,skv", [(1, 1), (31, 65), (257, 63), (300, 333), (64, 4097), (1000, 512)])
+def test_head_dim_64(dev, sq, skv):
+  # LTX-2's audio stream: 32 heads of 64 (models/ltx2/transformer_ltx2.py:788-789); flat schedule, 128-byte rows
+  H, D = 4, 64
+  q, k, v = O.normal_bf16((2, sq, H, D), 0), O.normal_bf16((2, skv, H, D), 1), O.normal_bf16((2, skv, H, D), 2)
+  out, lse = _run_np(q, k, v, dev)
+  for b in range(2):
+    ro, rl = O.attention(hsd(q[b:b + 1]), hsd(k[b:b + 1]), hsd(v[b:b + 1]), D**-0.5)
+    _check(hsd(out[b:b + 1]), lse[b], ro, rl, f"D=64 Sq={sq} Skv={skv} batch {b}")
+
+
+def test_head_dim_64_masked_and_sharp(dev):
+  H, D, sq, skv = 3, 64, 200, 333
+  q = O.bf16_round(O.normal_bf16((1, sq, H, D), 0) * np.float32(6.0))
+  k, v = O.normal_bf16((1, skv, H, D), 1), O.normal_bf16((1, skv, H, D), 2)
+  keep = np.random.default_rng(3).random((1, skv)) < 0.5
+  bias = ops.key_mask_bias(torch.from_numpy(keep).to(dev))
+  out, lse = ops.flash_attention(to_dev_bf16(q, dev), to_dev_bf16(k, dev), to_dev_bf16(v, dev), return_lse=True, key_bias=bias)
+  ro, rl = O.attention(hsd(q), hsd(k), hsd(v), D**-0.5, kv_mask=keep[0])
+  _check(hsd(to_np(out)), to_np(lse)[0], ro, rl, "D=64 masked, q x6")
