@@ -104,6 +104,22 @@ ffi::Error NormRopePerheadImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuf
                  "mdattn_norm_rope_perhead");
 }
 
+// x [B,S,H*D] bf16 or f32; w f32 [H*D]; cos/sin f32 [B,S,H*D] (mode 1) or [B,H,S,D/2] (mode 2), ignored for mode 0
+ffi::Error NormRopeRowsImpl(hipStream_t stream, ffi::AnyBuffer x, ffi::AnyBuffer w, ffi::AnyBuffer cos, ffi::AnyBuffer sin,
+                            ffi::Result<ffi::AnyBuffer> x_out, float eps, int64_t heads, int64_t mode) {
+  auto d = x.dimensions();
+  if (d.size() != 3 || heads <= 0 || d[2] % heads) return ffi::Error::InvalidArgument("mdattn_norm_rope_rows: x must be [B,S,H*D]");
+  if (x.element_type() != ffi::BF16 && x.element_type() != ffi::F32) return ffi::Error::InvalidArgument("mdattn_norm_rope_rows: x must be bf16 or f32");
+  const int64_t B = d[0], S = d[1], N = d[2], D = N / heads;
+  mdattn_strides so{S * N, N, D};  // x_out is [B,S,H,D]
+  return ToError(mdattn_norm_rope_rows(stream, x.untyped_data(), x.element_type() == ffi::F32, x_out->untyped_data(),
+                                       static_cast<const float*>(w.untyped_data()),
+                                       mode ? static_cast<const float*>(cos.untyped_data()) : nullptr,
+                                       mode ? static_cast<const float*>(sin.untyped_data()) : nullptr, (int)mode,
+                                       (int)B, (int)S, (int)heads, (int)D, eps, S * N, N, &so),
+                 "mdattn_norm_rope_rows");
+}
+
 // o_run / lse_run are donated by the caller (input_output_aliases) and updated in place.
 ffi::Error MergeImpl(hipStream_t stream, ffi::AnyBuffer o_run_in, ffi::AnyBuffer lse_run_in, ffi::AnyBuffer o_cur,
                      ffi::AnyBuffer lse_cur, ffi::Result<ffi::AnyBuffer> o_run, ffi::Result<ffi::AnyBuffer> lse_run) {
@@ -141,6 +157,13 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopeFullrow, NormRopeFullrowImpl,
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
                                   .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
                                   .Attr<float>("eps").Attr<int64_t>("heads").Attr<int64_t>("rope"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopeRows, NormRopeRowsImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>()
+                                  .Attr<float>("eps").Attr<int64_t>("heads").Attr<int64_t>("mode"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopePerhead, NormRopePerheadImpl,
                               ffi::Ffi::Bind()

@@ -21,6 +21,7 @@ FFI_TARGETS = {
     "mdattn_fwd_bf16_bias": "MdattnFwdBf16Bias",
     "mdattn_norm_rope_fullrow": "MdattnNormRopeFullrow",
     "mdattn_norm_rope_perhead": "MdattnNormRopePerhead",
+    "mdattn_norm_rope_rows": "MdattnNormRopeRows",
     "mdattn_merge": "MdattnMerge",
 }
 
@@ -89,6 +90,32 @@ def hip_norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6)
   out = jax.ShapeDtypeStruct((b, s, heads, d), jnp.bfloat16)
   call = jax.ffi.ffi_call("mdattn_norm_rope_fullrow", (out, out), vmap_method="sequential")
   return call(q, k, wq, wk, cos, sin, eps=np.float32(eps), heads=np.int64(heads), rope=np.int64(rope))
+
+
+def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotary_emb=None, k_rotary_emb=None,
+                       rope_type: str = "interleaved", is_self_attention: bool = True, eps: float = 1e-6):
+  """Fused prologue of LTX2Attention.__call__ (models/ltx2/attention_ltx2.py:556-585): see attention_op.hip_norm_rope_ltx2.
+  query/key [B,S,H*D] -> bf16 [B,S,H,D]; tables (cos, sin) as LTX2RotaryPosEmbed returns them."""
+  jax, jnp = _require_jax()
+  import numpy as np
+
+  if rope_type not in ("interleaved", "split"):
+    raise ValueError(f"{rope_type=} not supported. Choose between 'interleaved' and 'split'.")
+  q_tab = rotary_emb
+  k_tab = k_rotary_emb if k_rotary_emb is not None else (rotary_emb if is_self_attention else None)
+  if rotary_emb is None:
+    q_tab = k_tab = None
+  dummy = jnp.zeros((1,), jnp.float32)
+
+  def run(x, scale, tab):
+    b, s, n = x.shape
+    out = jax.ShapeDtypeStruct((b, s, heads, n // heads), jnp.bfloat16)
+    mode = 0 if tab is None else (1 if rope_type == "interleaved" else 2)
+    cos, sin = (dummy, dummy) if tab is None else (tab[0].astype(jnp.float32), tab[1].astype(jnp.float32))
+    call = jax.ffi.ffi_call("mdattn_norm_rope_rows", out, vmap_method="sequential")
+    return call(x, scale.astype(jnp.float32), cos, sin, eps=np.float32(eps), heads=np.int64(heads), mode=np.int64(mode))
+
+  return run(query, norm_q_scale, q_tab), (run(key, norm_k_scale, k_tab) if key is not None else None)
 
 
 def hip_flash_kernel(q, k, v, context):
