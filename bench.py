@@ -1,6 +1,6 @@
 """Benchmark of the DiT attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload wan14b|wan14b-ring|wan14b-fp8|wan1.3b|flux-dev]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload wan14b|wan14b-ring|wan14b-ulysses|wan14b-usp|wan14b-fp8|wan1.3b|flux-dev]
 
 One step = one pass of the path over one synthetic batch already resident in HBM: fused q/k
 RMSNorm + RoPE, then the bf16 self-attention forward (with LSE).  Prints ONE JSON line:

@@ -42,6 +42,11 @@ WORKLOADS = {
     "wan14b": Workload("wan14b", 40, 128, 75600, 75600, "fullrow", "wan", (21, 45, 80), cross_kv=512),
     "wan14b-ring": Workload("wan14b-ring", 40, 128, 9450, 9450, "fullrow", "wan", (21, 45, 80), ring_chunks=8),
     "wan14b-fp8": Workload("wan14b-fp8", 40, 128, 75600, 75600, "fullrow", "wan", (21, 45, 80)),
+    # single-GPU replays of the other context-parallel shards of configs[2] (attention_flax.py:875-986, :1305-1315):
+    # pure Ulysses over 8 GPUs = 5 heads at the full sequence; Ulysses 2 x ring 4 = 20 heads, a Q chunk of 18,900
+    # tokens against 4 KV chunks of 18,900
+    "wan14b-ulysses": Workload("wan14b-ulysses", 5, 128, 75600, 75600, "fullrow", "wan", (21, 45, 80)),
+    "wan14b-usp": Workload("wan14b-usp", 20, 128, 18900, 18900, "fullrow", "wan", (21, 45, 80), ring_chunks=4),
 }
 
 
