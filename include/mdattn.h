@@ -161,6 +161,23 @@ int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, const void* v8,
                    const float* q_scale, const float* k_scale, const float* v_scale);
 
 /*
+ * Backward of mdattn_fwd_bf16: dq, dk, dv from (q, k, v, out, dout, lse), non-causal, no mask.  Replaces: the
+ * backward of the reference's attention kernels, contract in kernels/splash_attention/base.py:108-160
+ * (`_attention_reference_custom_bwd`, "flash" form of di = rowsum(o * do)) and
+ * kernels/splash_attention/splash_attention_kernel.py:1277-1600, with `scale` applied inside (logits = scale*q.k).
+ *   dout, out    bf16 [B,Sq,H,D] by o_strides;  dq by q_strides;  dk by k_strides;  dv by v_strides
+ *   lse          f32 [B,H,Sq] as written by the forward
+ *   workspace    f32 device buffer of at least mdattn_bwd_workspace_floats(B,H,Sq) elements, 16-byte aligned
+ * Requires D == 128.
+ */
+int64_t mdattn_bwd_workspace_floats(int B, int H, int Sq);
+int mdattn_bwd_bf16(void* stream, const void* q, const void* k, const void* v, const void* out, const void* dout,
+                    const float* lse, void* dq, void* dk, void* dv, float* workspace, int64_t workspace_floats,
+                    int B, int H, int Sq, int Skv, int D,
+                    const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                    const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale);
+
+/*
  * In-place LSE-space merge of a normalised partial (o_cur, lse_cur) into the running
  * (o_run f32, lse_run f32); start from o_run = 0, lse_run = -1e30.
  * Replaces: kernels/splash_attention/ring_attention_kernel.py:1062-1073 (same result as the

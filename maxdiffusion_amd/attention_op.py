@@ -21,7 +21,7 @@ from . import ops
 
 __all__ = [
     "KERNEL_REGISTRY", "register_kernel", "AttentionOp", "hip_flash_kernel", "hip_flash_fp8_kernel",
-    "hip_norm_rope", "hip_norm_rope_ltx2", "HIP_KERNEL_NAMES",
+    "hip_norm_rope", "hip_norm_rope_ltx2", "hip_flash_attention_autograd", "HIP_KERNEL_NAMES",
 ]
 
 KERNEL_REGISTRY = {}
@@ -140,6 +140,30 @@ def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotar
   q = run(query, norm_q_scale, q_tab)
   k = run(key, norm_k_scale, k_tab) if key is not None else None
   return q, k
+
+
+
+class _HipFlashAttention(torch.autograd.Function):
+  """Forward + backward through the HIP kernels: what a trainer's custom_vjp around the attention kernel does in
+  the reference (kernels/splash_attention/splash_attention_kernel.py:1277-1600)."""
+
+  @staticmethod
+  def forward(ctx, q, k, v, scale):
+    out, lse = ops.flash_attention(q, k, v, scale=scale, return_lse=True)
+    ctx.save_for_backward(q, k, v, out, lse)
+    ctx.scale = scale
+    return out
+
+  @staticmethod
+  def backward(ctx, dout):
+    q, k, v, out, lse = ctx.saved_tensors
+    dq, dk, dv = ops.flash_attention_backward(q, k, v, out, dout.contiguous(), lse, scale=ctx.scale)
+    return dq, dk, dv, None
+
+
+def hip_flash_attention_autograd(q, k, v, scale: float):
+  """Differentiable attention on dense bf16 [B,S,H,D] tensors (torch autograd)."""
+  return _HipFlashAttention.apply(q, k, v, float(scale))
 
 
 def _apply_attention(

@@ -16,7 +16,7 @@ INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "libmdattn.so")
 FFI_LIB_PATH = os.path.join(PKG_DIR, "libmdattn_ffi.so")
 
-SOURCES = ["mdattn_api.hip", "norm_rope.hip", "attn_fwd_bf16.hip", "attn_fwd_fp8.hip", "merge_quant.hip"]
+SOURCES = ["mdattn_api.hip", "norm_rope.hip", "attn_fwd_bf16.hip", "attn_fwd_fp8.hip", "attn_bwd_bf16.hip", "merge_quant.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32 out of scalar float code.
 HIPCC_FLAGS = [

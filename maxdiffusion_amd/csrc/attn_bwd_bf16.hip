@@ -1,0 +1,323 @@
+// Backward of the non-causal attention forward for gfx950 (MI355X), bf16 MFMA, head_dim 128: dq, dk, dv from
+// (q, k, v, out, dout, lse).  With logits s = scale*q.k, p = exp(s - lse), dp = dout.v^T, delta = rowsum(dout*out):
+//   dv = p^T dout,   ds = p * (dp - delta),   dq = scale * ds k,   dk = scale * ds^T q.
+//
+// One kernel, three instantiations, no atomics: every gradient is accumulated by the waves that own its rows.
+//   "entity" rows: 32 per wave, their operands live in registers for the whole kernel (q and dout for dq; k and v
+//                  for dk; k for dv); the gradient rows are theirs.
+//   "stream" rows: walked in tiles of 32 through a 2-slot LDS ring filled by direct global->LDS loads (k and v for
+//                  dq; q and dout for dk and dv).
+// Per tile, with the forward kernel's layouts and fragment reads:
+//   S^T  = stream1 . entity1^T      (A = tile rows by ds_read_b128, B = entity fragments)   lane = entity row
+//   dP^T = stream2 . entity2^T      (not for dv)
+//   W    = exp2(c*S - lse*log2e) [* (dP - delta) * scale]     f32, packed to bf16 in B-operand order
+//   acc^T += stream3^T . W          (A = the tile through the transposing LDS read)
+// lse and delta belong to the q rows: per-lane scalars for dq, sixteen values per lane and tile for dk / dv, read
+// from a workspace that a small kernel fills first (delta, lse in log2 units, both padded to a multiple of 32 rows
+// with lse = +inf so that padded q rows get p = 0).
+#include "mdattn_common.h"
+
+namespace mdattn {
+namespace {
+
+constexpr int kBD = 128;                 // head dim
+constexpr int kBT = 32;                  // stream rows per tile
+constexpr int kBGK = 4 * kBD + 32;       // group stride of the row-read layout (see attn_fwd_bf16.hip)
+constexpr int kBGV = 4 * kBD;            // group stride of the transposed-read layout
+constexpr int kBTileA = (kBT / 4) * kBGK;
+constexpr int kBTileB = (kBT / 4) * kBGV;
+constexpr int kBStage = 2 * kBTileA + kBTileB;  // elements per ring slot
+
+typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr_b;
+typedef __attribute__((ext_vector_type(8))) short s16x8_b;
+
+__device__ __forceinline__ bf16x8 read_vt_b(const __bf16* p0, const __bf16* p1) {
+  s16x4 r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr_b)p0);
+  s16x4 r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr_b)p1);
+  s16x8_b r = __builtin_shufflevector(r0, r1, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, r);
+}
+
+struct BwdArgs {
+  const __bf16* e1;  // entity tensor of the score contraction
+  const __bf16* e2;  // entity tensor of the dP contraction (unused for dv)
+  const __bf16* s1;  // stream tensor of the score contraction
+  const __bf16* s2;  // stream tensor of the dP contraction (unused for dv)
+  const __bf16* s3;  // stream tensor the gradient accumulates with
+  __bf16* out;       // gradient of the entity rows
+  const float* lse2;   // [B,H,Sp] lse * log2(e), +inf on padded rows
+  const float* delta;  // [B,H,Sp]
+  int H, Se, Ss, Sp;
+  int net, total, chunk;
+  int64_t e1_sb, e1_ss, e1_sh, e2_sb, e2_ss, e2_sh;
+  int64_t s1_sb, s1_ss, s1_sh, s2_sb, s2_ss, s2_sh, s3_sb, s3_ss, s3_sh;
+  int64_t o_sb, o_ss, o_sh;
+  float c, scale;
+};
+
+// MODE 0: dq (entity = q rows, stream = keys), 1: dk, 2: dv (entity = key rows, stream = q rows)
+template <int MODE>
+__global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char smem_raw_b[];
+  __bf16* smem = reinterpret_cast<__bf16*>(smem_raw_b);
+  constexpr int NW = 4;
+  constexpr bool HAS2 = MODE != 2;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hh = lane >> 5;
+
+  const int wg = blockIdx.x;
+  const int w = (wg & 7) * a.chunk + (wg >> 3);
+  if (w >= a.total) return;
+  const int bh = w / a.net, et = w - bh * a.net;
+  const int b = bh / a.H, h = bh - b * a.H;
+  const int r0 = et * (NW * 32) + wave * 32;
+  const int nt = (a.Ss + kBT - 1) / kBT;
+  const float c = a.c;
+
+  // ---- entity fragments
+  int erow = r0 + l32;
+  erow = erow < a.Se ? erow : a.Se - 1;
+  bf16x8 ef1[8], ef2[8];
+  {
+    const __bf16* p = a.e1 + b * a.e1_sb + h * a.e1_sh + (int64_t)erow * a.e1_ss + hh * 8;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) ef1[s] = *reinterpret_cast<const bf16x8*>(p + s * 16);
+    if constexpr (HAS2) {
+      const __bf16* p2 = a.e2 + b * a.e2_sb + h * a.e2_sh + (int64_t)erow * a.e2_ss + hh * 8;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) ef2[s] = *reinterpret_cast<const bf16x8*>(p2 + s * 16);
+    }
+  }
+  const float* lrow = a.lse2 + ((int64_t)b * a.H + h) * a.Sp;
+  const float* drow = a.delta + ((int64_t)b * a.H + h) * a.Sp;
+  float lse_e = 0.f, delta_e = 0.f;
+  if constexpr (MODE == 0) {
+    lse_e = lrow[erow];
+    delta_e = drow[erow];
+  }
+
+  // ---- direct global -> LDS loads of one stream tile (layouts and lane maps of the forward kernel)
+  const __bf16* s1p = a.s1 + b * a.s1_sb + h * a.s1_sh;
+  const __bf16* s2p = HAS2 ? a.s2 + b * a.s2_sb + h * a.s2_sh : nullptr;
+  const __bf16* s3p = a.s3 + b * a.s3_sb + h * a.s3_sh;
+  const int grow = lane >> 4;
+  const int acol = ((lane & 15) ^ grow) * 8;         // row-read layout: chunk c of row r at position c ^ (r & 3)
+  const int bcol = ((lane & 15) ^ (grow << 2)) * 8;  // transposed-read layout: 64-byte segment s at s ^ (r & 3)
+  const unsigned smem_addr = lds_addr_of(smem);
+  auto dma = [&](int slot, int t) __attribute__((always_inline)) {
+    const unsigned A1 = smem_addr + (unsigned)(slot * kBStage) * 2u;
+    const unsigned A2 = A1 + kBTileA * 2u;
+    const unsigned Bt = A2 + kBTileA * 2u;
+#pragma unroll
+    for (int i = 0; i < (kBT / 4) / NW; ++i) {
+      const int g = wave + NW * i;
+      int rr = t * kBT + 4 * g + grow;
+      rr = rr < a.Ss ? rr : a.Ss - 1;
+      lds_dma16(s1p + (int64_t)rr * a.s1_ss + acol, A1 + (unsigned)(g * kBGK) * 2u);
+      if constexpr (HAS2) lds_dma16(s2p + (int64_t)rr * a.s2_ss + acol, A2 + (unsigned)(g * kBGK) * 2u);
+      lds_dma16(s3p + (int64_t)rr * a.s3_ss + bcol, Bt + (unsigned)(g * kBGV) * 2u);
+    }
+  };
+
+  f32x16 acc[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+
+  // per-lane fragment offsets (elements)
+  const int kx0 = l32 & 1, kx1 = (l32 >> 1) & 1;
+  const int k_base = (l32 >> 2) * kBGK + (l32 & 3) * kBD + (hh ^ kx0) * 8;
+  int k_off[8], v_off[4];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) k_off[j] = k_base + ((j & 1) ? -16 : 16) * kx1 + j * 16;
+  const int vxr = (lane & 15) >> 2;
+#pragma unroll
+  for (int sg = 0; sg < 4; ++sg)
+    v_off[sg] = 2 * kBTileA + hh * kBGV + vxr * kBD + (sg ^ vxr) * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+
+  dma(0, 0);
+  for (int t = 0; t < nt; ++t) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
+    __syncthreads();                      // ... and everyone's; the other slot (tile t-1) is free
+    if (t + 1 < nt) dma((t + 1) & 1, t + 1);
+    const __bf16* base = smem + (t & 1) * kBStage;
+
+    f32x16 S, dP;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { S[i] = 0.f; dP[i] = 0.f; }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bf16x8 f = *reinterpret_cast<const bf16x8*>(base + k_off[j]);
+      S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, ef1[j], S, 0, 0, 0);
+    }
+    if constexpr (HAS2) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const bf16x8 f = *reinterpret_cast<const bf16x8*>(base + kBTileA + k_off[j]);
+        dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, ef2[j], dP, 0, 0, 0);
+      }
+    }
+    // lse (log2 units) and delta of the q row each logit belongs to
+    float ls[16], dl[16];
+    if constexpr (MODE == 0) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { ls[i] = lse_e; dl[i] = delta_e; }
+      if (t == nt - 1) {  // keys past the end of a ragged last tile take no part
+        const int sbase = t * kBT + 4 * hh;
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (sbase + 8 * (i >> 2) + (i & 3) >= a.Ss) S[i] = -INFINITY;
+      }
+    } else {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 lv = *reinterpret_cast<const f32x4*>(lrow + t * kBT + 8 * g + 4 * hh);
+        const f32x4 dv = *reinterpret_cast<const f32x4*>(drow + t * kBT + 8 * g + 4 * hh);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { ls[4 * g + e] = lv[e]; dl[4 * g + e] = dv[e]; }
+      }
+    }
+    bf16x8 W[2];
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb) {
+      float wv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int i = 8 * hb + e;
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(S[i], c, -ls[i]));
+        wv[e] = HAS2 ? p * (dP[i] - dl[i]) * a.scale : p;
+      }
+      W[hb] = __builtin_bit_cast(bf16x8, pack8(wv));
+    }
+#pragma unroll
+    for (int jv = 0; jv < 8; ++jv) {
+      const __bf16* src = base + v_off[jv & 3] + (jv >> 2) * 4 * kBGV;
+      const bf16x8 f = read_vt_b(src, src + 2 * kBGV);
+      acc[jv & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, W[jv >> 2], acc[jv & 3], 0, 0, 0);
+    }
+  }
+
+  const int row = r0 + l32;
+  if (row < a.Se) {
+    __bf16* orow = a.out + b * a.o_sb + h * a.o_sh + (int64_t)row * a.o_ss + 4 * hh;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        uint2 u;
+        u.x = pack2(acc[db][4 * g], acc[db][4 * g + 1]);
+        u.y = pack2(acc[db][4 * g + 2], acc[db][4 * g + 3]);
+        *reinterpret_cast<uint2*>(orow + db * 32 + 8 * g) = u;
+      }
+  }
+}
+
+// delta[b,h,q] = sum_d dout*out, lse2 = lse*log2(e); rows q in [Sq, Sp) get delta 0, lse2 +inf.  16 lanes per row.
+__global__ __launch_bounds__(256) void bwd_prep_kernel(const __bf16* out, const __bf16* dout, const float* lse,
+                                                       float* lse2, float* delta, int H, int Sq, int Sp, int64_t rows,
+                                                       int64_t o_sb, int64_t o_ss, int64_t o_sh) {
+  const int64_t r = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (r >= rows) return;
+  const int lane = threadIdx.x & 15;
+  const int q = (int)(r % Sp);
+  const int64_t bh = r / Sp;
+  const int h = (int)(bh % H);
+  const int64_t b = bh / H;
+  float acc = 0.f;
+  if (q < Sq) {
+    const int64_t off = b * o_sb + (int64_t)q * o_ss + h * o_sh + lane * 8;
+    float x[8], y[8];
+    unpack8(*reinterpret_cast<const uint4*>(out + off), x);
+    unpack8(*reinterpret_cast<const uint4*>(dout + off), y);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc = __builtin_fmaf(x[j], y[j], acc);
+  }
+  acc = row16_sum(acc);
+  if (lane == 0) {
+    delta[r] = q < Sq ? acc : 0.f;
+    lse2[r] = q < Sq ? lse[bh * Sq + q] * kLog2e : INFINITY;
+  }
+}
+
+template <int MODE>
+int launch_bwd(hipStream_t st, BwdArgs a, int B) {
+  constexpr int lds_bytes = 2 * kBStage * 2;
+  a.net = (a.Se + 127) / 128;
+  const int64_t total = (int64_t)B * a.H * a.net;
+  if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
+  a.total = (int)total;
+  a.chunk = (a.total + 7) / 8;
+  auto kern = attn_bwd_kernel<MODE>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+    return MDATTN_E_LAUNCH;
+  hipLaunchKernelGGL(kern, dim3(a.chunk * 8), dim3(256), lds_bytes, st, a);
+  return launch_status();
+}
+
+}  // namespace
+}  // namespace mdattn
+
+using namespace mdattn;
+
+extern "C" int64_t mdattn_bwd_workspace_floats(int B, int H, int Sq) {
+  if (B <= 0 || H <= 0 || Sq <= 0) return 0;
+  return 2 * (int64_t)B * H * (((int64_t)Sq + 31) / 32 * 32);
+}
+
+extern "C" int mdattn_bwd_bf16(void* stream, const void* q, const void* k, const void* v, const void* out, const void* dout,
+                               const float* lse, void* dq, void* dk, void* dv, float* workspace, int64_t workspace_floats,
+                               int B, int H, int Sq, int Skv, int D,
+                               const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                               const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
+  if (!q || !k || !v || !out || !dout || !lse || !dq || !dk || !dv || !workspace) return MDATTN_E_BADARG;
+  if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return MDATTN_E_BADARG;
+  if (!q_strides || !k_strides || !v_strides || !o_strides) return MDATTN_E_BADARG;
+  if (!(scale > 0.f) || !(scale < 1e30f)) return MDATTN_E_BADARG;
+  if (D != kBD) return MDATTN_E_UNSUPPORTED;
+  if (workspace_floats < mdattn_bwd_workspace_floats(B, H, Sq)) return MDATTN_E_BADARG;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || !aligned16(dout) || !aligned16(dq) ||
+      !aligned16(dk) || !aligned16(dv) || !aligned16(workspace) || (reinterpret_cast<uintptr_t>(lse) & 3u))
+    return MDATTN_E_ALIGN;
+  if (!strides_ok(q_strides, 8) || !strides_ok(k_strides, 8) || !strides_ok(v_strides, 8) || !strides_ok(o_strides, 8))
+    return MDATTN_E_ALIGN;
+  if (q_strides->seq < D || k_strides->seq < D || v_strides->seq < D || o_strides->seq < D) return MDATTN_E_BADARG;
+
+  hipStream_t st = (hipStream_t)stream;
+  const int Sp = (Sq + 31) / 32 * 32;
+  float* lse2 = workspace;
+  float* delta = workspace + (int64_t)B * H * Sp;
+  const int64_t rows = (int64_t)B * H * Sp;
+  if ((rows + 15) / 16 > 0x7FFFFFFF) return MDATTN_E_UNSUPPORTED;
+  hipLaunchKernelGGL(bwd_prep_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const __bf16*)out,
+                     (const __bf16*)dout, lse, lse2, delta, H, Sq, Sp, rows, o_strides->batch, o_strides->seq, o_strides->head);
+  if (launch_status() != MDATTN_OK) return MDATTN_E_LAUNCH;
+
+  BwdArgs a;
+  a.lse2 = lse2; a.delta = delta; a.H = H; a.Sp = Sp; a.c = scale * kLog2e; a.scale = scale;
+  auto set = [](int64_t& sb, int64_t& ss, int64_t& sh, const mdattn_strides* s) { sb = s->batch; ss = s->seq; sh = s->head; };
+  // dq: entity q / dout, stream k (scores), v (dP), k (accumulate)
+  a.e1 = (const __bf16*)q; a.e2 = (const __bf16*)dout; a.s1 = (const __bf16*)k; a.s2 = (const __bf16*)v; a.s3 = (const __bf16*)k;
+  a.out = (__bf16*)dq; a.Se = Sq; a.Ss = Skv;
+  set(a.e1_sb, a.e1_ss, a.e1_sh, q_strides); set(a.e2_sb, a.e2_ss, a.e2_sh, o_strides);
+  set(a.s1_sb, a.s1_ss, a.s1_sh, k_strides); set(a.s2_sb, a.s2_ss, a.s2_sh, v_strides); set(a.s3_sb, a.s3_ss, a.s3_sh, k_strides);
+  set(a.o_sb, a.o_ss, a.o_sh, q_strides);
+  int rc = launch_bwd<0>(st, a, B);
+  if (rc != MDATTN_OK) return rc;
+  // dk: entity k / v, stream q (scores), dout (dP), q (accumulate)
+  a.e1 = (const __bf16*)k; a.e2 = (const __bf16*)v; a.s1 = (const __bf16*)q; a.s2 = (const __bf16*)dout; a.s3 = (const __bf16*)q;
+  a.out = (__bf16*)dk; a.Se = Skv; a.Ss = Sq;
+  set(a.e1_sb, a.e1_ss, a.e1_sh, k_strides); set(a.e2_sb, a.e2_ss, a.e2_sh, v_strides);
+  set(a.s1_sb, a.s1_ss, a.s1_sh, q_strides); set(a.s2_sb, a.s2_ss, a.s2_sh, o_strides); set(a.s3_sb, a.s3_ss, a.s3_sh, q_strides);
+  set(a.o_sb, a.o_ss, a.o_sh, k_strides);
+  rc = launch_bwd<1>(st, a, B);
+  if (rc != MDATTN_OK) return rc;
+  // dv: entity k, stream q (scores), dout (accumulate)
+  a.e2 = nullptr; a.s2 = nullptr; a.s3 = (const __bf16*)dout;
+  a.out = (__bf16*)dv;
+  set(a.s3_sb, a.s3_ss, a.s3_sh, o_strides);
+  set(a.o_sb, a.o_ss, a.o_sh, v_strides);
+  return launch_bwd<2>(st, a, B);
+}

@@ -104,6 +104,22 @@ ffi::Error NormRopePerheadImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuf
                  "mdattn_norm_rope_perhead");
 }
 
+// q, out, dout, dq [B,Sq,H,D]; k, v, dk, dv [B,Skv,H,D] (layout 0); lse f32 [B,H,Sq]; workspace f32 [>= mdattn_bwd_workspace_floats]
+ffi::Error BwdBf16Impl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v, ffi::AnyBuffer out,
+                       ffi::AnyBuffer dout, ffi::AnyBuffer lse, ffi::Result<ffi::AnyBuffer> dq, ffi::Result<ffi::AnyBuffer> dk,
+                       ffi::Result<ffi::AnyBuffer> dv, ffi::Result<ffi::AnyBuffer> workspace, float scale) {
+  int64_t B, Sq, H, D, Bk, Skv, Hk, Dk;
+  mdattn_strides sq, sk;
+  if (!Describe(q.dimensions(), 0, &B, &Sq, &H, &D, &sq) || !Describe(k.dimensions(), 0, &Bk, &Skv, &Hk, &Dk, &sk))
+    return ffi::Error::InvalidArgument("mdattn_bwd_bf16: rank-4 [B,S,H,D] buffers expected");
+  if (Bk != B || Hk != H || Dk != D) return ffi::Error::InvalidArgument("mdattn_bwd_bf16: inconsistent shapes");
+  return ToError(mdattn_bwd_bf16(stream, q.untyped_data(), k.untyped_data(), v.untyped_data(), out.untyped_data(),
+                                 dout.untyped_data(), static_cast<const float*>(lse.untyped_data()), dq->untyped_data(),
+                                 dk->untyped_data(), dv->untyped_data(), static_cast<float*>(workspace->untyped_data()),
+                                 (int64_t)workspace->element_count(), (int)B, (int)H, (int)Sq, (int)Skv, (int)D, &sq, &sk, &sk, &sq, scale),
+                 "mdattn_bwd_bf16");
+}
+
 // x [B,S,H*D] bf16 or f32; w f32 [H*D]; cos/sin f32 [B,S,H*D] (mode 1) or [B,H,S,D/2] (mode 2), ignored for mode 0
 ffi::Error NormRopeRowsImpl(hipStream_t stream, ffi::AnyBuffer x, ffi::AnyBuffer w, ffi::AnyBuffer cos, ffi::AnyBuffer sin,
                             ffi::Result<ffi::AnyBuffer> x_out, float eps, int64_t heads, int64_t mode) {
@@ -157,6 +173,14 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopeFullrow, NormRopeFullrowImpl,
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
                                   .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
                                   .Attr<float>("eps").Attr<int64_t>("heads").Attr<int64_t>("rope"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnBwdBf16, BwdBf16Impl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
+                                  .Attr<float>("scale"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopeRows, NormRopeRowsImpl,
                               ffi::Ffi::Bind()

@@ -19,6 +19,7 @@ from .build import FFI_LIB_PATH, build_ffi_library
 FFI_TARGETS = {
     "mdattn_fwd_bf16": "MdattnFwdBf16",
     "mdattn_fwd_bf16_bias": "MdattnFwdBf16Bias",
+    "mdattn_bwd_bf16": "MdattnBwdBf16",
     "mdattn_norm_rope_fullrow": "MdattnNormRopeFullrow",
     "mdattn_norm_rope_perhead": "MdattnNormRopePerhead",
     "mdattn_norm_rope_rows": "MdattnNormRopeRows",
@@ -75,6 +76,37 @@ def hip_flash_attention(q, k, v, scale: float, layout: int, keep_mask=None):
     )
     return call(q, k, v, bias, scale=np.float32(scale), layout=np.int64(layout))
   return call(q, k, v, scale=np.float32(scale), layout=np.int64(layout))
+
+
+def hip_flash_attention_vjp(q, k, v, scale: float):
+  """Differentiable attention on [B,S,H,D] bf16 arrays: jax.custom_vjp around the forward and backward custom calls
+  (what kernels/splash_attention/splash_attention_kernel.py:1277-1600 does for the Pallas kernel)."""
+  jax, jnp = _require_jax()
+  import numpy as np
+
+  @jax.custom_vjp
+  def attn(q, k, v):
+    return hip_flash_attention(q, k, v, scale, 0)[0]
+
+  def fwd(q, k, v):
+    out, lse = hip_flash_attention(q, k, v, scale, 0)
+    return out, (q, k, v, out, lse)
+
+  def bwd(res, dout):
+    q, k, v, out, lse = res
+    b, sq, h, d = q.shape
+    nws = 2 * b * h * ((sq + 31) // 32 * 32)  # mdattn_bwd_workspace_floats
+    call = jax.ffi.ffi_call(
+        "mdattn_bwd_bf16",
+        (jax.ShapeDtypeStruct(q.shape, jnp.bfloat16), jax.ShapeDtypeStruct(k.shape, jnp.bfloat16),
+         jax.ShapeDtypeStruct(v.shape, jnp.bfloat16), jax.ShapeDtypeStruct((nws,), jnp.float32)),
+        vmap_method="sequential",
+    )
+    dq, dk, dv, _ = call(q, k, v, out, dout.astype(jnp.bfloat16), lse, scale=np.float32(scale))
+    return dq, dk, dv
+
+  attn.defvjp(fwd, bwd)
+  return attn(q, k, v)
 
 
 def hip_norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6):

@@ -16,7 +16,7 @@ from . import _lib
 from ._lib import Strides
 
 __all__ = [
-    "norm_rope_fullrow", "norm_rope_perhead", "norm_rope_rows", "flash_attention", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
+    "norm_rope_fullrow", "norm_rope_perhead", "norm_rope_rows", "flash_attention", "flash_attention_backward", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
     "merge_partial", "finalize", "new_merge_state", "LSE_INIT",
 ]
 
@@ -183,6 +183,37 @@ def flash_attention(q, k, v, scale: float | None = None, return_lse: bool = Fals
         _ptr(key_bias), key_bias.stride(0))
     _lib.check(rc, "mdattn_fwd_bf16_bias")
   return (out, lse) if return_lse else out
+
+
+def flash_attention_backward(q, k, v, out, dout, lse, scale: float | None = None):
+  """Gradients of `flash_attention`: q, out, dout [B,Sq,H,D]; k, v [B,Skv,H,D] logical views, bf16; lse f32 [B,H,Sq] as
+  returned by the forward.  out and dout must share strides.  Returns (dq, dk, dv) shaped and laid out like q, k, v."""
+  _check_dev(q, k, v, out, dout, lse)
+  if not all(t.dtype == torch.bfloat16 for t in (q, k, v, out, dout)):
+    raise ValueError("flash_attention_backward needs bf16 q, k, v, out, dout")
+  b, sq, h, d = q.shape
+  skv = k.shape[1]
+  if out.shape != q.shape or dout.shape != q.shape or k.shape != v.shape or tuple(lse.shape) != (b, h, sq):
+    raise ValueError("inconsistent shapes")
+  if dout.stride() != out.stride():
+    dout = dout.contiguous() if out.is_contiguous() else dout.clone(memory_format=torch.preserve_format).as_strided(out.shape, out.stride())
+  if dout.stride() != out.stride():
+    raise ValueError("out and dout must share strides")
+  if scale is None:
+    scale = 1.0 / math.sqrt(d)
+  lse = lse.contiguous()
+  dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+  if dq.stride() != q.stride() or dk.stride() != k.stride() or dv.stride() != v.stride():
+    raise ValueError("q, k, v must be dense tensors (their gradients take the same strides)")
+  lib = _lib.load()
+  nws = lib.mdattn_bwd_workspace_floats(b, h, sq)
+  ws = torch.empty(nws, dtype=torch.float32, device=q.device)
+  sq_, sk_, sv_, so_ = _strides(q), _strides(k), _strides(v), _strides(out)
+  rc = lib.mdattn_bwd_bf16(
+      _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), nws,
+      b, h, sq, skv, d, ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale))
+  _lib.check(rc, "mdattn_bwd_bf16")
+  return dq, dk, dv
 
 
 def quant_e4m3(x: torch.Tensor):

@@ -24,6 +24,7 @@ Pinning status of each function (what fixes it besides its own formula):
   attention / attention_rows     scipy logsumexp, torch SDPA (fp32, CPU),
                                  invariants (K=0 -> mean(V), lse=ln Skv; ...),
                                  hand fixtures of tests/ltx2/test_attention_ltx2.py:38-116
+  attention_bwd                  torch autograd through torch SDPA (fp64, CPU), finite differences
   merge_lse / merge_mlo /        attention over a union of KV chunks equals the
   merge_scan_ring                merge of per-chunk results (brute force)
   attention_dot_product_bf16     PARITY UNPINNED at bit level: the rounding points
@@ -45,7 +46,7 @@ __all__ = [
     "flux_ids", "flux_rope_angles", "flux_rope_table", "flux_rope_table_matrix",
     "apply_rope_interleaved", "apply_rope_matrix_form", "norm_rope_fullrow", "norm_rope_perhead",
     "norm_rope_wan_reference_flow", "attention", "attention_rows", "attention_dot_product_bf16",
-    "ltx2_apply_rotary_emb", "ltx2_apply_split_rotary_emb", "norm_rope_ltx2", "merge_lse", "merge_mlo", "merge_scan_ring", "ring_replay", "quant_e4m3", "attention_fp8_emulated",
+    "ltx2_apply_rotary_emb", "ltx2_apply_split_rotary_emb", "norm_rope_ltx2", "attention_bwd", "merge_lse", "merge_mlo", "merge_scan_ring", "ring_replay", "quant_e4m3", "attention_fp8_emulated",
     "LSE_INIT",
 ]
 
@@ -344,6 +345,30 @@ def norm_rope_ltx2(x, w, cos, sin, mode: str, eps: float = 1e-6, dtype=np.float6
   if mode == "split":
     return ltx2_apply_split_rotary_emb(y, cos, sin, dtype)
   raise ValueError(mode)
+
+
+# --------------------------------------------------------------------------- backward
+def attention_bwd(q, k, v, do, scale: float, dtype=np.float64):
+  """Gradients of `attention` w.r.t. q, k, v for an upstream gradient `do` of the output.
+
+  kernels/splash_attention/base.py:108-160 (`_attention_reference_custom_bwd`, "flash" form
+  di = rowsum(o * do)) with the dispatcher's `scale` applied inside: logits = scale * q k^T.
+  q, do [H,Sq,D]; k, v [H,Skv,D] -> (dq, dk, dv).
+  """
+  q, k, v, do = (np.asarray(x, dtype) for x in (q, k, v, do))
+  s = np.matmul(q, np.swapaxes(k, -1, -2)) * dtype(scale)
+  m = s.max(axis=-1, keepdims=True)
+  e = np.exp(s - m)
+  lse = m + np.log(e.sum(axis=-1, keepdims=True))
+  p = np.exp(s - lse)
+  o = np.matmul(p, v)
+  dv = np.matmul(np.swapaxes(p, -1, -2), do)
+  dp = np.matmul(do, np.swapaxes(v, -1, -2))
+  di = (o * do).sum(axis=-1, keepdims=True)
+  ds = (dp - di) * p
+  dq = np.matmul(ds, k) * dtype(scale)
+  dk = np.matmul(np.swapaxes(ds, -1, -2), q) * dtype(scale)
+  return dq, dk, dv
 
 
 # --------------------------------------------------------------------------- A6 merges

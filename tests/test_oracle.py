@@ -355,6 +355,32 @@ def test_norm_rope_ltx2_modes():
   np.testing.assert_allclose(O.norm_rope_ltx2(x, w, np.ones((1, 2, 3, 8)), np.zeros((1, 2, 3, 8)), "split"), y, atol=1e-15)
 
 
+# ----------------------------------------------------------------------------- backward
+def test_attention_bwd_matches_torch_autograd_and_finite_differences():
+  import torch
+
+  rng = np.random.default_rng(31)
+  H, Sq, Skv, D = 2, 7, 11, 16
+  q, k, v, do = (rng.standard_normal(s) for s in ((H, Sq, D), (H, Skv, D), (H, Skv, D), (H, Sq, D)))
+  scale = 0.3
+  dq, dk, dv = O.attention_bwd(q, k, v, do, scale)
+  tq, tk, tv = (torch.tensor(x, dtype=torch.float64, requires_grad=True) for x in (q, k, v))
+  out = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, scale=scale)
+  out.backward(torch.tensor(do))
+  np.testing.assert_allclose(dq, tq.grad.numpy(), rtol=1e-9, atol=1e-12)
+  np.testing.assert_allclose(dk, tk.grad.numpy(), rtol=1e-9, atol=1e-12)
+  np.testing.assert_allclose(dv, tv.grad.numpy(), rtol=1e-9, atol=1e-12)
+  # one directional finite difference per input
+  f = lambda a, b, c: float((O.attention(a, b, c, scale)[0] * do).sum())
+  eps = 1e-6
+  for idx, (x, g) in enumerate(((q, dq), (k, dk), (v, dv))):
+    d = rng.standard_normal(x.shape)
+    args_p, args_m = [q, k, v], [q, k, v]
+    args_p[idx], args_m[idx] = x + eps * d, x - eps * d
+    fd = (f(*args_p) - f(*args_m)) / (2 * eps)
+    assert abs(fd - float((g * d).sum())) <= 1e-6 * max(1.0, abs(fd))
+
+
 # ----------------------------------------------------------------------------- fp8 emulation
 def test_fp8_emulation_meets_cosine_bar():
   q = O.normal_bf16((2, 128, 128), 0)
