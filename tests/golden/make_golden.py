@@ -78,6 +78,32 @@ def main():
     if f.endswith(".npz"):
       print(f, os.path.getsize(os.path.join(HERE, f)))
 
+  # LTX-2 prologue: 2 batches x 9 tokens, 4 heads x 64, both rotation forms (tables as LTX2RotaryPosEmbed shapes them)
+  rng = np.random.default_rng(40)
+  B, S, H, D = 2, 9, 4, 64
+  x = O.normal_bf16((B, S, H * D), 0)
+  w = (1 + 0.1 * rng.standard_normal(H * D)).astype(np.float32)
+  ang_i = rng.uniform(-3, 3, (B, S, H * D // 2))
+  ang_s = rng.uniform(-3, 3, (B, H, S, D // 2))
+  cos_i, sin_i = np.repeat(np.cos(ang_i), 2, -1).astype(np.float32), np.repeat(np.sin(ang_i), 2, -1).astype(np.float32)
+  cos_s, sin_s = np.cos(ang_s).astype(np.float32), np.sin(ang_s).astype(np.float32)
+  np.savez_compressed(
+      os.path.join(HERE, "norm_rope_ltx2.npz"), x=bits(x), w=w, heads=H, cos_i=cos_i, sin_i=sin_i, cos_s=cos_s, sin_s=sin_s,
+      out_none=O.norm_rope_ltx2(x, w, None, None, "none").astype(np.float32),
+      out_interleaved=O.norm_rope_ltx2(x, w, cos_i, sin_i, "interleaved").astype(np.float32),
+      out_split=O.norm_rope_ltx2(x, w, cos_s, sin_s, "split").astype(np.float32))
+
+  # backward: ragged Sq and Skv, 2 heads
+  q = O.normal_bf16((1, 45, 2, 128), 0)
+  k = O.normal_bf16((1, 70, 2, 128), 1)
+  v = O.normal_bf16((1, 70, 2, 128), 2)
+  do = O.normal_bf16((1, 45, 2, 128), 3)
+  t = lambda a: a[0].transpose(1, 0, 2)
+  dq, dk, dv = O.attention_bwd(t(q), t(k), t(v), t(do), 128**-0.5)
+  u = lambda a: a.transpose(1, 0, 2)[None].astype(np.float32)
+  np.savez_compressed(os.path.join(HERE, "attention_bwd_small.npz"), q=bits(q), k=bits(k), v=bits(v), do=bits(do),
+                      scale=128**-0.5, dq=u(dq), dk=u(dk), dv=u(dv))
+
 
 if __name__ == "__main__":
   main()

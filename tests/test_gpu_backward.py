@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import oracle as O
-from helpers import hsd, rel_l2, to_dev_bf16, to_np
+from helpers import bits_to_dev, golden, hsd, rel_l2, to_dev_bf16, to_np
 from maxdiffusion_amd import ops
 
 pytestmark = pytest.mark.gpu
@@ -92,3 +92,13 @@ def test_autograd_function(dev):
   _check(hsd(to_np(q.grad)), rq, "autograd dq")
   _check(hsd(to_np(k.grad)), rk, "autograd dk")
   _check(hsd(to_np(v.grad)), rv, "autograd dv")
+
+
+def test_backward_golden(dev):
+  g = golden("attention_bwd_small.npz")
+  q, k, v, do = (bits_to_dev(g[n], dev) for n in ("q", "k", "v", "do"))
+  out, lse = ops.flash_attention(q, k, v, scale=float(g["scale"]), return_lse=True)
+  dq, dk, dv = ops.flash_attention_backward(q, k, v, out, do, lse, scale=float(g["scale"]))
+  _check(to_np(dq), g["dq"], "golden dq")
+  _check(to_np(dk), g["dk"], "golden dk")
+  _check(to_np(dv), g["dv"], "golden dv")

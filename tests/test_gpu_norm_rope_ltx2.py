@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import oracle as O
-from helpers import err_stats, to_dev_bf16, to_np
+from helpers import bits_to_dev, err_stats, golden, to_dev_bf16, to_np
 from maxdiffusion_amd import attention_op, ops
 
 pytestmark = pytest.mark.gpu
@@ -70,3 +70,14 @@ def test_call_flow_of_the_attention_module(dev):
     _assert_close(to_np(ko).reshape(B, Sk, -1), O.norm_rope_ltx2(k_cross, wk, *tab_k, mode), f"{mode} cross k with its own table")
   with pytest.raises(ValueError, match="not supported"):
     attention_op.hip_norm_rope_ltx2(t(q), None, t(wq), t(wk), H, rope_type="rotate_half")
+
+
+def test_golden_ltx2(dev):
+  g = golden("norm_rope_ltx2.npz")
+  x, H = bits_to_dev(g["x"], dev), int(g["heads"])
+  t = lambda a: torch.from_numpy(a).to(dev)
+  B, S, N = x.shape
+  for mode, cs in (("none", (None, None)), ("interleaved", (g["cos_i"], g["sin_i"])), ("split", (g["cos_s"], g["sin_s"]))):
+    cos, sin = (None if a is None else t(a) for a in cs)
+    out = ops.norm_rope_rows(x, t(g["w"]), cos, sin, heads=H, mode=mode)
+    _assert_close(to_np(out).reshape(B, S, N), g[f"out_{mode}"], f"ltx2 golden {mode}")

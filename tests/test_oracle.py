@@ -423,6 +423,14 @@ def test_committed_golden_vectors_follow_the_oracle():
   g = golden("norm_rope_flux.npz")
   got = O.norm_rope_perhead(bits_to_f32(g["k"]), bits_to_f32(g["wk"]), g["cos"], g["sin"], w_txt=bits_to_f32(g["wk_txt"]), n_txt=int(g["n_txt"]))
   np.testing.assert_allclose(got, g["k_out"], atol=1e-6)
+  g = golden("norm_rope_ltx2.npz")
+  x = bits_to_f32(g["x"])
+  np.testing.assert_allclose(O.norm_rope_ltx2(x, g["w"], g["cos_i"], g["sin_i"], "interleaved"), g["out_interleaved"], atol=1e-6)
+  np.testing.assert_allclose(O.norm_rope_ltx2(x, g["w"], g["cos_s"], g["sin_s"], "split"), g["out_split"], atol=1e-6)
+  g = golden("attention_bwd_small.npz")
+  dq, dk, dv = O.attention_bwd(*(hsd(bits_to_f32(g[n])) for n in ("q", "k", "v", "do")), float(g["scale"]))
+  np.testing.assert_allclose(dv.transpose(1, 0, 2)[None], g["dv"], atol=1e-6)
+  np.testing.assert_allclose(dq.transpose(1, 0, 2)[None], g["dq"], atol=1e-6)
   g = golden("merge_small.npz")
   o_run, l_run = np.zeros((1, 2, 70, 128)), np.full((1, 2, 70), O.LSE_INIT)
   for ob, lb in zip(g["parts_o"], g["parts_l"]):
