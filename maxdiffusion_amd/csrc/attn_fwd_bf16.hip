@@ -8,25 +8,23 @@
 //                period; the loads of slots t+2 and t+3 are in flight while period t runs.
 //   S^T = K.Q^T with v_mfma_f32_32x32x16_bf16: A = K rows from LDS (ds_read_b128), B = Q fragment
 //                held in registers for the whole kernel.  In the 32x32 accumulator layout every lane
-//                then holds 16 keys of ONE query row, so the row max / row sum are in-lane
-//                reductions plus a single swap between the two wave halves, and the running
-//                max / sum / rescale factor are per-lane scalars.
+//                then holds 16 keys of ONE query row, so the row sum (and the row max, when needed) are
+//                in-lane reductions plus a single swap between the two wave halves, and the reference
+//                point / sum / rescale factor are per-lane scalars.
 //   O^T += V^T.P^T: the accumulator layout of S^T is already the B-operand layout of the next MFMA
 //                (after the bf16 convert), and the A operand V^T comes from the row-major V tile
 //                through the transposing LDS read (ds_read_b64_tr_b16).
-//   softmax    = exp2 with scale*log2(e) folded into one FMA per logit; f32 state; the accumulator
-//                rescale is lazy (only when a row max moves by more than 2^8) and deferred to points
-//                where no PV MFMA of the affected tile half is outstanding.
-//   pipelining = the vector ALU needs ~5 instructions per MFMA for the softmax.  Measured on this
-//                chip, waves that issue "1 MFMA + up to 6 VALU" groups keep the matrix pipe ~94 % busy
-//                (two waves per SIMD), while phases of pure MFMA followed by phases of pure VALU leave
-//                it idle half of the time.  The keys are therefore walked in blocks of 32, and in
-//                iteration b every wave issues, interleaved in one instruction stream,
+//   softmax    = exp2 with scale*log2(e) folded into one FMA per logit; f32 state.  A row's reference
+//                point m is not its running maximum: it moves only when a logit exceeds it by more than
+//                2^8, which the row's partial sum reveals, so the hot stream computes no maximum at all
+//                and the accumulator rescale sits in a cold branch.
+//   pipelining = the vector ALU issues through the same port as the MFMAs.  Phases of pure MFMA
+//                followed by phases of pure VALU leave the matrix pipe idle half of the time, so the
+//                keys are walked in blocks of 32, and in iteration b every wave issues, interleaved in
+//                one instruction stream,
 //                    matrix pipe : O^T += V^T(b-1).P^T(b-1)  (8 MFMAs)  and  S^T(b+1) = K(b+1).Q^T  (8 MFMAs)
-//                    vector ALU  : P(b) = exp2(c*S(b) - c*m), row sums, bf16 convert
-//                    LDS         : the K / V^T fragment of the next MFMA of the same kind (a longer look-ahead
-//                                  measured slower: the read would overwrite a register an MFMA issued just
-//                                  before may still be reading)
+//                    vector ALU  : P(b) = exp2(c*S(b) - c*m), row sums, bf16 convert (3.5 instructions per MFMA)
+//                    LDS         : the K / V^T fragment of the next MFMA of the same kind
 //                PV and QK MFMAs alternate, so no MFMA depends on the one issued just before it.  The
 //                loop body is the same for every iteration: the iterations before the first and after
 //                the last real block run on fully masked logits (P = 0) instead of being peeled.
@@ -57,6 +55,10 @@ constexpr int kGV = 4 * kD;       // V group stride (1024 B)
 constexpr int kKTile = (kBN / 4) * kGK;
 constexpr int kStage = kKTile + (kBN / 4) * kGV;  // elements per ring stage
 constexpr float kLazy = 8.0f;    // log2 units a row max may lag behind before accumulators are rescaled
+constexpr float kTrig = 128.0f;  // a 16-key partial row sum above this sends the wave to the rescale branch (< 2^kLazy)
+constexpr int kS0 = 2;           // first slot of an iteration that touches the block's logits
+constexpr int kLA = 1;           // LDS look-ahead: a slot requests the fragment of the kLA-th next MFMA of its kind
+                                 // (1, 2 and 3 measure the same)
 
 typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
@@ -147,6 +149,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[db][i] = 0.f;
   float m = -1e30f, l = 0.f;
+  float mc = m * c;  // the rows' reference point in log2 units
 
   // lane-constant LDS offsets
   // K fragment j (logical chunk 2j + hh) of row l32 sits at chunk position (2j + hh) ^ (l32 & 3): pair j ^ x1,
@@ -162,23 +165,29 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
     v_off[sg] = kKTile + hh * kGV + vxr * kD + (sg ^ vxr) * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
 
   f32x16 Sa, Sb;        // logits of odd / even blocks
-  bf16x8 Pa[2], Pb[2];  // probabilities of odd / even blocks (PV B-operand layout, 16 keys each)
+  u32x4 Pa[2], Pb[2];   // probabilities of odd / even blocks (PV B-operand layout, 16 keys each), bf16 pairs
   bf16x8 kfr[4], vfr[4];  // rotating fragment windows
 #pragma unroll
   for (int i = 0; i < 16; ++i) { Sa[i] = -INFINITY; Sb[i] = 0.f; }  // block -1: fully masked
 #pragma unroll
-  for (int i = 0; i < 2; ++i) { Pa[i] = __builtin_bit_cast(bf16x8, make_uint4(0, 0, 0, 0)); Pb[i] = Pa[i]; }
+  for (int i = 0; i < 2; ++i) { Pa[i] = u32x4{0u, 0u, 0u, 0u}; Pb[i] = Pa[i]; }
 
   // One iteration.  SC holds the logits of block BLK; SN receives those of block BLK+1.
   // KC/KN: K rows of block BLK+1 / BLK+2; VC/VN: V rows of block BLK-1 / BLK.
   // Slot n of the stream: n even -> PV MFMA n/2, n odd -> QK MFMA n/2, each followed by the LDS
-  // request for the next MFMA of the same kind, then a chunk of the softmax of block BLK.  The
-  // softmax starts at slot 5 (row max) and 7 (exp2 chunks): the last QK MFMA of block BLK was issued at
-  // slot 15 of the previous iteration, and reading its result earlier stalls the wave's whole stream.
+  // request for the next MFMA of the same kind, then a share of the softmax of block BLK.  The vector
+  // ALU issues through the same port as the MFMAs and is nearly as busy, so the hot stream carries the
+  // bare minimum per pair of logits: two FMAs, two exp2, one bf16 pack and one dot2 that adds the pair
+  // (as rounded, i.e. exactly what the PV MFMA consumes) to the row sum.  There is no row max in it: the
+  // reference point m of a row moves only when a logit exceeds it by more than kLazy, and then that row's
+  // partial sum exceeds 2^kLazy, so the sum itself is the trigger.  A triggered wave (every row's first
+  // block, then almost never) redoes the block's softmax from the logits with the proper maximum in a
+  // cold branch at the end of the iteration, where no PV MFMA of the previous block is outstanding.
+  // The softmax starts at slot kS0: the last QK MFMA of block BLK was issued at slot 15 of the
+  // previous iteration, and reading its result earlier stalls the wave's whole stream.
 #define MDATTN_ITER(SC, SN, PC, PP, KC, KN, VC, VN, BLK) /* KC.. : base pointers [even j, odd j]; VC.. : [segment] */                                                     \
   {                                                                                                           \
-    float alpha = 1.f, mc = 0.f, lsum = 0.f, p[8];                                                            \
-    bool need = false;                                                                                        \
+    float lsum = 0.f, pe = 0.f;                                                                               \
     if ((BLK) * 32 + 32 > a.Skv) { /* ragged tail and the virtual blocks past the end: -inf logits */         \
       asm volatile("" ::: "memory");                                                                          \
       const int kv_base = (BLK) * 32 + 4 * hh;                                                                \
@@ -186,9 +195,9 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
         if (kv_base + 8 * (i >> 2) + (i & 3) >= a.Skv) SC[i] = -INFINITY;                                     \
     }                                                                                                         \
     _Pragma("unroll") for (int n = 0; n < 16; ++n) {                                                          \
-      const int j = n >> 1, jn = j + 1;                                                                       \
+      const int j = n >> 1, jn = j + kLA;                                                                     \
       if ((n & 1) == 0) {                                                                                     \
-        O[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[j & 3], PP[j >> 2], O[j & 3], 0, 0, 0);        \
+        O[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[j & 3], __builtin_bit_cast(bf16x8, PP[j >> 2]), O[j & 3], 0, 0, 0); \
         const __bf16* vsrc = (jn < 8 ? (VC) : (VN))[jn & 3] + ((jn & 7) >> 2) * 4 * kGV;                      \
         vfr[jn & 3] = read_vt(vsrc, vsrc + 2 * kGV);                                                          \
       } else {                                                                                                \
@@ -201,40 +210,45 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
         }                                                                                                     \
         kfr[jn & 3] = *reinterpret_cast<const bf16x8*>((jn < 8 ? (KC) : (KN))[jn & 1] + (jn & 7) * 16);       \
       }                                                                                                       \
-      if (n == 5) {                                                                                           \
-        /* row max + lazy-rescale decision: a row's max moves only when it would otherwise see an exp2    */  \
-        /* argument above kLazy (per-lane select: the stream stays one basic block); the accumulator      */  \
-        /* multiply waits until every PV MFMA of the previous block has been issued (iteration end)       */  \
-        float mloc = SC[0];                                                                                   \
-        _Pragma("unroll") for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, SC[i]);                             \
-        mloc = xhalf_max(mloc);                                                                               \
-        const bool moved = (mloc - m) * c > kLazy;                                                            \
-        const float mnew = moved ? mloc : m;                                                                  \
-        alpha = __builtin_amdgcn_exp2f((m - mnew) * c); /* exactly 1 for rows that keep their max */          \
-        m = mnew;                                                                                             \
-        need = __builtin_amdgcn_ballot_w64(moved) != 0;                                                       \
-        mc = m * c;                                                                                           \
-        asm volatile("" : "+v"(alpha), "+v"(mc));                                                             \
-      }                                                                                                       \
-      if (n >= 7 && n <= 14) {                                                                                \
-        const int e = (n - 7) * 2;                                                                            \
-        p[e & 7] = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[e], c, -mc));                                     \
-        p[(e & 7) + 1] = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[e + 1], c, -mc));                           \
-        lsum += p[e & 7] + p[(e & 7) + 1];                                                                    \
-        /* pins the chunk in its slot: otherwise the compiler sinks the softmax below the MFMA stream */      \
-        asm volatile("" : "+v"(p[e & 7]), "+v"(p[(e & 7) + 1]), "+v"(lsum));                                  \
-        if ((e & 7) == 6) {                                                                                   \
-          PC[e >> 3] = __builtin_bit_cast(bf16x8, pack8(p));                                                  \
-          asm volatile("" : "+v"(PC[e >> 3]));                                                                \
+      const int e0 = n < kS0 ? 0 : ((n - kS0) * 16) / (16 - kS0);                                             \
+      const int e1 = n < kS0 ? 0 : ((n + 1 - kS0) * 16) / (16 - kS0);                                         \
+      _Pragma("unroll") for (int e = 0; e < 16; ++e) {                                                        \
+        if (e >= e0 && e < e1) {                                                                              \
+          const float x = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[e], c, -mc));                              \
+          if ((e & 1) == 0) {                                                                                 \
+            pe = x;                                                                                           \
+            /* pins the work in its slot: otherwise the compiler sinks the softmax below the MFMA stream */  \
+            asm volatile("" : "+v"(pe));                                                                      \
+          } else {                                                                                            \
+            unsigned pk = pack2(pe, x);                                                                       \
+            lsum += pe + x;                                                                                   \
+            asm volatile("" : "+v"(pk), "+v"(lsum));                                                          \
+            PC[e >> 3][(e >> 1) & 3] = pk;                                                                    \
+          }                                                                                                   \
         }                                                                                                     \
       }                                                                                                       \
       __builtin_amdgcn_sched_barrier(0);                                                                      \
     }                                                                                                         \
-    l = l * alpha + lsum;                                                                                     \
-    if (need) {                                                                                               \
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lsum <= kTrig)) != 0, 0)) {                            \
+      float mloc = SC[0];                                                                                     \
+      _Pragma("unroll") for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, SC[i]);                               \
+      mloc = xhalf_max(mloc);                                                                                 \
+      const float mnew = (mloc - m) * c > kLazy ? mloc : m;                                                   \
+      const float alpha = __builtin_amdgcn_exp2f((m - mnew) * c); /* exactly 1 for rows that keep m */        \
+      m = mnew;                                                                                               \
+      mc = m * c;                                                                                             \
+      lsum = 0.f;                                                                                             \
+      _Pragma("unroll") for (int e = 0; e < 16; e += 2) {                                                     \
+        const float x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[e], c, -mc));                               \
+        const float x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[e + 1], c, -mc));                           \
+        lsum += x0 + x1;                                                                                      \
+        PC[e >> 3][(e >> 1) & 3] = pack2(x0, x1);                                                             \
+      }                                                                                                       \
+      l *= alpha;                                                                                             \
       _Pragma("unroll") for (int db = 0; db < 4; ++db)                                                        \
         _Pragma("unroll") for (int i = 0; i < 16; ++i) O[db][i] *= alpha;                                     \
     }                                                                                                         \
+    l += lsum;                                                                                                \
   }
 
   // ring bookkeeping: period t uses slot t%4 (K(t), V(t-1)) and looks ahead into slot (t+1)%4
@@ -243,7 +257,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): Q fragments and this wave's share of slots 0..2
   __syncthreads();
 #pragma unroll
-  for (int s = 0; s < 1; ++s) {
+  for (int s = 0; s < kLA; ++s) {
     kfr[s] = *reinterpret_cast<const bf16x8*>(smem + ((s & 1) ? k_off_o : k_off_e) + s * 16);
     const __bf16* vsrc = smem + v_off[s];
     vfr[s] = read_vt(vsrc, vsrc + 2 * kGV);
@@ -254,7 +268,6 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
     // Slot s_fill was last read in period t-1 and now receives K(t+3), V(t+2).
     __builtin_amdgcn_s_waitcnt(0x0F70 | (32 / NW));
     __syncthreads();
-    dma(s_fill, t + 3);
     const __bf16* cur = smem + s_cur * kStage;
     const __bf16* nxt = smem + s_nxt * kStage;
     const __bf16* Kc0[2] = {cur + k_off_e, cur + k_off_o};
@@ -265,6 +278,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
     const __bf16* Vn0[4] = {nxt + v_off[0], nxt + v_off[1], nxt + v_off[2], nxt + v_off[3]};
     // iteration 2t-1: softmax(2t-1), PV(2t-2), QK(2t)
     MDATTN_ITER(Sa, Sb, Pa, Pb, Kc0, Kc1, Vc0, Vc1, 2 * t - 1)
+    dma(s_fill, t + 3);
     // iteration 2t: softmax(2t), PV(2t-1), QK(2t+1)
     MDATTN_ITER(Sb, Sa, Pb, Pa, Kc1, Kn0, Vc1, Vn0, 2 * t)
     const int tmp = s_cur;
@@ -291,7 +305,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
         u.y = pack2(O[db][4 * g + 2] * inv, O[db][4 * g + 3] * inv);
         *reinterpret_cast<uint2*>(orow + db * 32 + 8 * g) = u;
       }
-    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (m * c + __log2f(lt)) * kLn2;
+    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (mc + __log2f(lt)) * kLn2;
   }
 }
 
