@@ -181,7 +181,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   // (as rounded, i.e. exactly what the PV MFMA consumes) to the row sum.  There is no row max in it: the
   // reference point m of a row moves only when a logit exceeds it by more than kLazy, and then that row's
   // partial sum exceeds 2^kLazy, so the sum itself is the trigger.  A triggered wave (every row's first
-  // block, then almost never) redoes the block's softmax from the logits with the proper maximum in a
+  // block, then almost never) redoes the block's softmax from the logits with the true maximum in a
   // cold branch at the end of the iteration, where no PV MFMA of the previous block is outstanding.
   // The softmax starts at slot kS0: the last QK MFMA of block BLK was issued at slot 15 of the
   // previous iteration, and reading its result earlier stalls the wave's whole stream.
@@ -233,7 +233,9 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
       float mloc = SC[0];                                                                                     \
       _Pragma("unroll") for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, SC[i]);                               \
       mloc = xhalf_max(mloc);                                                                                 \
-      const float mnew = (mloc - m) * c > kLazy ? mloc : m;                                                   \
+      /* every row of a triggered wave moves to its true maximum: right after, the block's sum is at most */  \
+      /* 16, so a row can trigger again only when its maximum has grown by another 3 log2 units           */  \
+      const float mnew = fmaxf(m, mloc);                                                                      \
       const float alpha = __builtin_amdgcn_exp2f((m - mnew) * c); /* exactly 1 for rows that keep m */        \
       m = mnew;                                                                                               \
       mc = m * c;                                                                                             \
@@ -262,6 +264,15 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
     const __bf16* vsrc = smem + v_off[s];
     vfr[s] = read_vt(vsrc, vsrc + 2 * kGV);
   }
+  const int nfull = a.Skv / kBN;  // tiles that lie fully inside the sequence
+  const __bf16* kdma = kp + (int64_t)(3 * kBN + 4 * wave) * a.k_ss;  // this wave's first row group of K(t+3) ...
+  const __bf16* vdma = vp + (int64_t)(2 * kBN + 4 * wave) * a.v_ss;  // ... and of V(t+2)
+  unsigned kofs_i[16 / NW], vofs_i[16 / NW];                          // lane offsets of its further row groups
+#pragma unroll
+  for (int i = 0; i < 16 / NW; ++i) {
+    kofs_i[i] = kofs + (unsigned)(4 * NW * i * (int)a.k_ss) * 2u;
+    vofs_i[i] = vofs + (unsigned)(4 * NW * i * (int)a.v_ss) * 2u;
+  }
   for (int t = 0; t <= nt; ++t) {
     // every wave's loads into slot s_nxt (issued two periods ago) have landed once all waves pass the
     // barrier: only the loads of the previous period (2 * 16 / NW per wave) may still be in flight.
@@ -278,7 +289,22 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
     const __bf16* Vn0[4] = {nxt + v_off[0], nxt + v_off[1], nxt + v_off[2], nxt + v_off[3]};
     // iteration 2t-1: softmax(2t-1), PV(2t-2), QK(2t)
     MDATTN_ITER(Sa, Sb, Pa, Pb, Kc0, Kc1, Vc0, Vc1, 2 * t - 1)
-    dma(s_fill, t + 3);
+    // K(t+3) and V(t+2) into slot s_fill, issued here rather than right after the barrier (where all eight
+    // waves would queue their loads before their first MFMA).  Tiles inside the sequence: running pointers
+    // and constant lane offsets, a handful of scalar instructions per load.
+    if (t + 3 < nfull) {
+      const unsigned Ks = smem_addr + (unsigned)(s_fill * kStage + wave * kGK) * 2u;
+      const unsigned Vs = smem_addr + (unsigned)(s_fill * kStage + kKTile + wave * kGV) * 2u;
+#pragma unroll
+      for (int i = 0; i < 16 / NW; ++i) {
+        lds_dma16(kdma, kofs_i[i], Ks + (unsigned)(NW * i * kGK) * 2u);
+        lds_dma16(vdma, vofs_i[i], Vs + (unsigned)(NW * i * kGV) * 2u);
+      }
+    } else {
+      dma(s_fill, t + 3);
+    }
+    kdma += kBN * a.k_ss;
+    vdma += kBN * a.v_ss;
     // iteration 2t: softmax(2t), PV(2t-1), QK(2t+1)
     MDATTN_ITER(Sb, Sa, Pb, Pa, Kc1, Kn0, Vc1, Vn0, 2 * t)
     const int tmp = s_cur;
@@ -401,6 +427,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[db][i] = 0.f;
   float m = -1e30f, l = 0.f;
+  float mc = m * cs;  // the rows' reference point in log2 units
 
   // per-lane fragment offsets (elements): K fragment j, V slab sg; kV8 = offset of the second transposing read
   // (rows + 8), kVH = offset of the second 16-key half of the tile
@@ -449,35 +476,42 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       for (int i = 0; i < 16; ++i)
         if (kv_base + 8 * (i >> 2) + (i & 3) >= a.Skv) S[i] = -INFINITY;
     }
-    // ---- online softmax with lazy rescale
-    float mloc = S[0];
+    // ---- online softmax.  The hot path takes no row maximum: P and its sum are formed against the row's
+    // current reference point, and only a partial sum above kTrig (a logit far above the reference, or
+    // many a little above) sends the wave through the branch that moves every row's reference to its true
+    // maximum, rescales the accumulators and redoes the tile's P.
+    bf16x8 P[2];
+    auto soft = [&](float rf) __attribute__((always_inline)) {
+      float lsum = 0.f;
 #pragma unroll
-    for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, S[i]);
-    mloc = xhalf_max(mloc);
-    const bool moved = (mloc - m) * cs > kLazy;
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(moved) != 0, 0)) {
-      const float mnew = moved ? mloc : m;
+      for (int hb = 0; hb < 2; ++hb) {
+        float p[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[8 * hb + e], cs, -rf));
+          lsum += p[e];
+        }
+        P[hb] = __builtin_bit_cast(bf16x8, pack8(p));
+      }
+      return lsum;
+    };
+    float lsum = soft(mc);
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lsum <= kTrig)) != 0, 0)) {
+      float mloc = S[0];
+#pragma unroll
+      for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, S[i]);
+      mloc = xhalf_max(mloc);
+      const float mnew = fmaxf(m, mloc);
       float alpha = __builtin_amdgcn_exp2f((m - mnew) * cs);
       asm volatile("" : "+v"(alpha));  // keeps the rescale inside this rarely taken branch
       m = mnew;
+      mc = m * cs;
       l *= alpha;
 #pragma unroll
       for (int db = 0; db < ND; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[db][i] *= alpha;
-    }
-    const float mc = m * cs;
-    bf16x8 P[2];
-    float lsum = 0.f;
-#pragma unroll
-    for (int hb = 0; hb < 2; ++hb) {
-      float p[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[8 * hb + e], cs, -mc));
-        lsum += p[e];
-      }
-      P[hb] = __builtin_bit_cast(bf16x8, pack8(p));
+      lsum = soft(mc);
     }
     l += lsum;
     // ---- O^T += V^T.P^T

@@ -9,9 +9,10 @@
 //                same k-slot order, so a lane simply holds 32 contiguous bytes of its row.
 //   softmax      in f32 on the 32 logits a lane holds for its query row; q_scale*k_scale*scale*log2(e)
 //                is folded into the exp2 argument.  P is kept 2^4 above the usual normalisation
-//                (reference point = running max - 4) so that e4m3's normal range [2^-6, 448] covers
-//                probabilities down to 2^-10 of the row max; the reference point only moves when a
-//                new maximum would push P beyond 2^8 (lazy rescale).  The row sum uses the f32 P.
+//                (reference point = a row maximum - 4) so that e4m3's normal range [2^-6, 448] covers
+//                probabilities down to 2^-10 of the row max; the reference point only moves when
+//                some P may have passed 2^8, which the partial row sums reveal (no row maximum in the
+//                hot path).  The row sum uses the f32 P.
 //   O^T += V^T.P^T  one MFMA per 32-wide slab of d with all 64 keys of the tile as K.  P goes from the
 //                accumulator layout to the B operand by the e4m3 convert alone (operand byte s = value
 //                s%16 of block s/16).  V^T comes from the row-major V tile through ds_read_b64_tr_b8:
@@ -37,7 +38,7 @@ constexpr int kVS8 = kD8;                                 // V row stride in LDS
 constexpr int kStage8 = kBN8 * kKS8 + kBN8 * kVS8;        // bytes per LDS stage
 constexpr int kSlots8 = 3;                                // LDS ring depth
 constexpr float kPOff = 4.0f;                             // P = exp2(logit - max + kPOff) at a fresh maximum
-constexpr float kPLazy = 4.0f;                            // extra headroom before the reference point moves
+constexpr float kPTrig = 256.0f;                          // a 4-key partial row sum above this sends the wave to the rescale branch
 
 typedef __attribute__((ext_vector_type(2))) int i32x2;
 typedef i32x2 __attribute__((address_space(3))) * lds_i32x2_ptr;
@@ -162,40 +163,76 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   auto tile = [&](int t, int slot, auto masked) __attribute__((always_inline)) {
     const char* Ks = smem8 + slot * kStage8;
     // ---- S^T = K.Q^T for the two 32-key blocks
-    f32x16 S[2];
+    auto qk = [&](f32x16* S, const char* Kb) __attribute__((always_inline)) {
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
-      i32x8 kf[2];
+      for (int blk = 0; blk < 2; ++blk) {
+        i32x8 kf[2];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const u32x4 lo = *reinterpret_cast<const u32x4*>(Ks + k_off[j][0] + blk * 32 * kKS8);
-        const u32x4 hi = *reinterpret_cast<const u32x4*>(Ks + k_off[j][1] + blk * 32 * kKS8);
-        kf[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+        for (int j = 0; j < 2; ++j) {
+          const u32x4 lo = *reinterpret_cast<const u32x4*>(Kb + k_off[j][0] + blk * 32 * kKS8);
+          const u32x4 hi = *reinterpret_cast<const u32x4*>(Kb + k_off[j][1] + blk * 32 * kKS8);
+          kf[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+        }
+        f32x16 z;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) z[i] = 0.f;
+        z = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[0], qf[0], z, 0, 0, 0, 0, 0, 0);
+        S[blk] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], z, 0, 0, 0, 0, 0, 0);
       }
-      f32x16 z;
+      if constexpr (decltype(masked)::value) {
+        const int kbase = t * kBN8 + 4 * hh;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) z[i] = 0.f;
-      z = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[0], qf[0], z, 0, 0, 0, 0, 0, 0);
-      S[blk] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], z, 0, 0, 0, 0, 0, 0);
-    }
-    if constexpr (decltype(masked)::value) {
-      const int kbase = t * kBN8 + 4 * hh;
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            if (kbase + 32 * blk + 8 * (i >> 2) + (i & 3) >= a.Skv) S[blk][i] = -INFINITY;
+      }
+    };
+    // ---- P = exp2(c*S - ref), f32 row sum, e4m3 pack in B-operand order.  The hot path takes no row
+    // maximum: P is formed against the current reference point, and only a group of four probabilities
+    // that sums beyond 2^8 (so possibly one beyond it: e4m3 ends at 448) sends the wave through the branch
+    // that moves every row's reference to its true maximum - kPOff, rescales the accumulators and redoes
+    // the tile's logits and P.  Right after a move a group sums to at most 4 * 2^kPOff, so a row triggers again only
+    // when its maximum has grown by two more log2 units.
+    i32x8 pk;
+    float gmax;
+    auto soft = [&](const f32x16* S, float rf) __attribute__((always_inline)) {
+      float ls = 0.f;
+      gmax = 0.f;
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-        for (int i = 0; i < 16; ++i)
-          if (kbase + 32 * blk + 8 * (i >> 2) + (i & 3) >= a.Skv) S[blk][i] = -INFINITY;
+        for (int g = 0; g < 4; ++g) {
+          float p[4];
+#pragma unroll
+          for (int x = 0; x < 4; ++x) p[x] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[blk][4 * g + x], c, -rf));
+          const float s4 = (p[0] + p[1]) + (p[2] + p[3]);
+          ls += s4;
+          gmax = fmaxf(gmax, s4);
+          int u = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
+          u = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], u, true);
+          pk[4 * blk + g] = u;
+        }
+      return ls;
+    };
+    float ls;
+    {
+      f32x16 S[2];
+      qk(S, Ks);
+      ls = soft(S, ref);
     }
-    // ---- row max over the tile; move the reference point only when P would leave [0, 2^8]
-    float mx = S[0][0];
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(gmax <= kPTrig)) != 0, 0)) {
+      f32x16 S[2];  // recomputed rather than kept: the hot path then holds the logits only while it forms P
+      const char* Kb = Ks;
+      asm volatile("" : "+s"(Kb));  // an address the compiler cannot match with the hot path's: no reuse of its logits
+      qk(S, Kb);
+      float mx = S[0][0];
 #pragma unroll
-    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, S[0][i]);
+      for (int i = 1; i < 16; ++i) mx = fmaxf(mx, S[0][i]);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, S[1][i]);
-    mx = xhalf_max(mx) * c;
-    const bool need = mx > ref + (kPOff + kPLazy);
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(need) != 0, 0)) {
-      const float nref = need ? mx - kPOff : ref;
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, S[1][i]);
+      mx = xhalf_max(mx) * c;
+      const float nref = fmaxf(ref, mx - kPOff);
       float alpha = __builtin_amdgcn_exp2f(ref - nref);
       asm volatile("" : "+v"(alpha));  // keeps the rescale inside this rarely taken branch
       ref = nref;
@@ -204,24 +241,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       for (int sl = 0; sl < 4; ++sl)
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[sl][i] *= alpha;
+      ls = soft(S, ref);
     }
-    // ---- P = exp2(c*S - ref), f32 row sum, e4m3 pack in B-operand order
-    i32x8 pk;
-    float ls = 0.f;
-#pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        float p[4];
-#pragma unroll
-        for (int x = 0; x < 4; ++x) {
-          p[x] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[blk][4 * g + x], c, -ref));
-          ls += p[x];
-        }
-        int u = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
-        u = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], u, true);
-        pk[4 * blk + g] = u;
-      }
     l += ls;
     // ---- O^T += V^T.P^T
 #pragma unroll

@@ -431,16 +431,19 @@ def quant_e4m3(x):
   return e4m3_round(x / s), s
 
 
-def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: float = 4.0, p_lazy: float = 4.0):
+def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: float = 4.0, p_trig: float = 256.0,
+                           rows_per_wave: int = 32):
   """Emulation of the fp8 kernel's arithmetic (no reference counterpart).
 
   Q, K, V quantised per tensor; logits from the quantised operands in f32; online softmax per
   KV tile in base 2 with P rounded to e4m3 before the PV product; f32 accumulation; the row
-  sum uses the un-rounded P.  P = exp2(logit - ref) where the reference point `ref` is set to
-  (row max - p_offset) whenever the running row max exceeds ref + p_offset + p_lazy: P then
-  stays within [0, 2^(p_offset+p_lazy)] = [0, 256], inside e4m3's range, and probabilities
-  down to 2^-(6+p_offset) of the row max stay in e4m3's normal range.  The result does not
-  depend on `ref` except through the e4m3 rounding.  q [H,Sq,D], k/v [H,Skv,D].
+  sum uses the un-rounded P.  P = exp2(logit - ref).  The reference point `ref` of a row moves
+  as the kernel moves it: when, in a tile, some aligned group of four keys of some row of the
+  same wave (rows_per_wave consecutive query rows) has probabilities summing beyond p_trig,
+  every row of that wave takes ref = max(ref, tile max - p_offset).  P then stays within
+  [0, p_trig], inside e4m3's range, and probabilities down to 2^-(6+p_offset) of the row max
+  stay in e4m3's normal range.  The result does not depend on `ref` except through the e4m3
+  rounding.  q [H,Sq,D], k/v [H,Skv,D].
   """
   q8, sq = quant_e4m3(q)
   k8, sk = quant_e4m3(k)
@@ -451,11 +454,20 @@ def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: f
   l = np.zeros((H, Sq), np.float32)
   o = np.zeros((H, Sq, D), np.float32)
   c = np.float32(np.float32(scale) * np.float32(np.log2(np.e)) * sq * sk)
+  nw = -(-Sq // rows_per_wave)
   for t0 in range(0, Skv, kv_tile):
     s = np.einsum("hqd,hkd->hqk", q8, k8[:, t0:t0 + kv_tile])
+    with np.errstate(over="ignore"):
+      p = np.exp2(s * c - ref[..., None]).astype(np.float32)
+    n = p.shape[-1]
+    pg = np.zeros((H, Sq, -(-n // 4) * 4), np.float32)
+    pg[..., :n] = p
+    row_trig = ~(pg.reshape(H, Sq, -1, 4).sum(axis=-1).max(axis=-1) <= np.float32(p_trig))
+    wt = np.zeros((H, nw * rows_per_wave), bool)
+    wt[:, :Sq] = row_trig
+    wave_trig = np.repeat(wt.reshape(H, nw, rows_per_wave).any(axis=-1), rows_per_wave, axis=1)[:, :Sq]
     mx = s.max(axis=-1) * c
-    need = mx > ref + np.float32(p_offset + p_lazy)
-    nref = np.where(need, mx - np.float32(p_offset), ref).astype(np.float32)
+    nref = np.where(wave_trig, np.maximum(ref, mx - np.float32(p_offset)), ref).astype(np.float32)
     a = np.exp2(ref - nref)
     ref = nref
     p = np.exp2(s * c - ref[..., None]).astype(np.float32)
