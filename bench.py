@@ -88,20 +88,24 @@ def main():
   q_in, k_in = randn(1, S, H * D), randn(1, S, H * D)
   v = randn(1, Skv * ring, H, D)
   k_extra = randn(1, Skv * (ring - 1), H, D) if ring > 1 else None
+  fp8 = args.workload.endswith("-fp8")
+  # bf16: the prologue emits q * scale * log2(e) (still one rounding) and the attention kernel is given scale = ln 2,
+  # so that it sees scale * log2(e) == 1 and its logits need no multiply; same result as scale = D^-1/2 on plain q
+  q_mul = 1.0 if fp8 else ops.folded_q_mul(D, w.scale)
+  att_scale = w.scale if fp8 else ops.FOLDED_SCALE
   if w.norm == "fullrow":
     wq, wk = tb(O.norm_weight(H * D, 3)), tb(O.norm_weight(H * D, 4))
     # a ring shard owns the first S tokens of the full latent grid
     cos, sin = (torch.from_numpy(t[:S].copy()).to(dev) for t in O.wan_rope_table(w.grid, D))
-    prologue = lambda: ops.norm_rope_fullrow(q_in, k_in, wq, wk, cos, sin, H)
+    prologue = lambda: ops.norm_rope_fullrow(q_in, k_in, wq, wk, cos, sin, H, q_mul=q_mul)
   else:
     wq, wk = tb(O.norm_weight(D, 3)), tb(O.norm_weight(D, 4))
     cos, sin = (torch.from_numpy(t).to(dev) for t in O.flux_rope_table(O.flux_ids(*w.grid)))
     q4, k4 = q_in.view(1, S, H, D), k_in.view(1, S, H, D)
-    prologue = lambda: ops.norm_rope_perhead(q4, k4, wq, wk, cos, sin)
+    prologue = lambda: ops.norm_rope_perhead(q4, k4, wq, wk, cos, sin, q_mul=q_mul)
 
   ev = lambda: torch.cuda.Event(enable_timing=True)
   t_pro, t_att, t_quant = [], [], []
-  fp8 = args.workload.endswith("-fp8")
 
   def step(record: bool):
     e0, e1, e2, eq = ev(), ev(), ev(), ev()
@@ -113,12 +117,12 @@ def main():
       eq.record()
       ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=w.scale, return_lse=True)
     elif ring == 1:
-      ops.flash_attention(qn, kn, v, scale=w.scale, return_lse=True)
+      ops.flash_attention(qn, kn, v, scale=att_scale, return_lse=True)
     else:  # one ring shard: this Q chunk against `ring` successive KV chunks, merged in LSE space
       o_run, l_run = ops.new_merge_state(1, S, H, D, dev)
       for i in range(ring):
         kc = kn if i == 0 else k_extra[:, (i - 1) * Skv:i * Skv]
-        o, l = ops.flash_attention(qn, kc, v[:, i * Skv:(i + 1) * Skv], scale=w.scale, return_lse=True)
+        o, l = ops.flash_attention(qn, kc, v[:, i * Skv:(i + 1) * Skv], scale=att_scale, return_lse=True)
         ops.merge_partial(o_run, l_run, o, l)
       ops.finalize(o_run)
     e2.record()
@@ -162,11 +166,11 @@ def main():
     qn, _ = prologue()
     kc, vc = randn(1, w.cross_kv, H, D), randn(1, w.cross_kv, H, D)
     for _ in range(2):
-      ops.flash_attention(qn, kc, vc, scale=w.scale, return_lse=True)
+      ops.flash_attention(qn, kc, vc, scale=att_scale, return_lse=True)
     e0, e1 = ev(), ev()
     e0.record()
     for _ in range(reps):
-      ops.flash_attention(qn, kc, vc, scale=w.scale, return_lse=True)
+      ops.flash_attention(qn, kc, vc, scale=att_scale, return_lse=True)
     e1.record()
     torch.cuda.synchronize()
     cms = e0.elapsed_time(e1) / reps
@@ -201,7 +205,7 @@ def main():
       "config": {"workload": f"{args.workload}: B=1 H={H} D={D} Sq={S} Skv={Skv * ring} norm={w.norm} rope={w.rope}"
                              + (f" ring_chunks={ring} (merge per chunk)" if ring > 1 else ""),
                  "step": "fused q/k RMSNorm+RoPE -> " + ("per-tensor e4m3 quantisation of q, k, v -> fp8 flash-attention forward with LSE"
-                                                             if fp8 else "bf16 flash-attention forward with LSE")},
+                                                             if fp8 else "bf16 flash-attention forward with LSE (softmax scale * log2 e carried by the prologue's q output)")},
       "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                    "frac": achieved / peak, "traffic": traffic.get(kname), "kernel": kname,
                    "kernel_ms": att_ms, "flop_per_launch": flops / ring},

@@ -57,12 +57,16 @@ const char* mdattn_strerror(int code);
  *   cos, sin     f32 [S, D/2]: real/imaginary part of the rotary table the unchanged host
  *                code builds (WanRotaryPosEmbed, models/wan/transformers/transformer_wan.py:63-95);
  *                both NULL = norm only (cross-attention, rotary_emb is None, attention_flax.py:2671)
+ *   q_mul        constant multiplied into q_out before its rounding (1.0f = none).  With
+ *                q_mul = scale * log2(e) and scale = ln 2 handed to the attention entry points the
+ *                softmax scale costs no rounding and no instruction: the reference multiplies k by
+ *                scale and q by log2(e) in bf16 before its kernels (attention_flax.py:1783, :610, :890).
  * Arithmetic: statistics, scale and rotation in f32, ONE rounding to bf16.
  * Requires D % 8 == 0, H*D <= 8192, 16-byte aligned pointers, strides % 8 == 0.
  */
 int mdattn_norm_rope_fullrow(void* stream, const void* q_in, const void* k_in, void* q_out, void* k_out,
                              const void* wq, const void* wk, const float* cos, const float* sin,
-                             int B, int S, int H, int D, float eps,
+                             int B, int S, int H, int D, float eps, float q_mul,
                              int64_t in_stride_batch, int64_t in_stride_seq,
                              const mdattn_strides* out_strides);
 
@@ -75,11 +79,12 @@ int mdattn_norm_rope_fullrow(void* stream, const void* q_in, const void* k_in, v
  *   q_in, k_in   bf16 [B,S,H,D] described by in_strides (k_in may be NULL)
  *   wq, wk       bf16 [D]; wq_txt / wk_txt (nullable) are used for tokens [0, n_txt)
  *   cos, sin     f32 [S, D/2] from FluxPosEmbed (models/embeddings_flax.py:437-469); NULL = norm only
+ *   q_mul        as for mdattn_norm_rope_fullrow
  * Requires D in {64,128,256}.
  */
 int mdattn_norm_rope_perhead(void* stream, const void* q_in, const void* k_in, void* q_out, void* k_out,
                              const void* wq, const void* wk, const void* wq_txt, const void* wk_txt, int n_txt,
-                             const float* cos, const float* sin, int B, int S, int H, int D, float eps,
+                             const float* cos, const float* sin, int B, int S, int H, int D, float eps, float q_mul,
                              const mdattn_strides* in_strides, const mdattn_strides* out_strides);
 
 /*

@@ -33,8 +33,8 @@ _S = ctypes.POINTER(Strides)
 SIGNATURES = {
     "mdattn_version": ([], _I),
     "mdattn_strerror": ([_I], ctypes.c_char_p),
-    "mdattn_norm_rope_fullrow": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _L, _L, _S], _I),
-    "mdattn_norm_rope_perhead": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _F, _S, _S], _I),
+    "mdattn_norm_rope_fullrow": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _L, _L, _S], _I),
+    "mdattn_norm_rope_perhead": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _F, _F, _S, _S], _I),
     "mdattn_norm_rope_rows": ([_P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _L, _L, _S], _I),
     "mdattn_fwd_bf16": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),
     "mdattn_fwd_bf16_bias": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F, _P, _L], _I),

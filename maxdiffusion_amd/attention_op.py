@@ -117,13 +117,15 @@ def hip_flash_fp8_kernel(q, k, v, context):
 
 
 def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotary_emb=None, k_rotary_emb=None,
-                       rope_type: str = "interleaved", is_self_attention: bool = True, eps: float = 1e-6):
+                       rope_type: str = "interleaved", is_self_attention: bool = True, eps: float = 1e-6,
+                       q_mul: float = 1.0):
   """Fused prologue of LTX2Attention.__call__ (models/ltx2/attention_ltx2.py:556-585).
 
   query/key [B,S,H*D] (bf16 or f32) are normalised over the full inner dim with the f32 scales; the query is rotated
   by `rotary_emb`, the key by `k_rotary_emb` if given, else by `rotary_emb` when this is self-attention, else not
   at all.  Tables are (cos, sin) as LTX2RotaryPosEmbed returns them: [B,S,H*D] (interleaved) or [B,H,S,D/2] (split).
-  Returns (q, k) bf16 [B,S,H,D], ready for `hip_flash`.  `key` None (cached K/V): only the query is processed."""
+  Returns (q, k) bf16 [B,S,H,D], ready for `hip_flash`.  `key` None (cached K/V): only the query is processed.
+  `q_mul` (see hip_norm_rope) is folded into the f32 query scale on the host."""
   if rope_type not in ("interleaved", "split"):
     raise ValueError(f"{rope_type=} not supported. Choose between 'interleaved' and 'split'.")  # :145-146
   q_tab = rotary_emb
@@ -137,7 +139,7 @@ def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotar
     cos, sin = (t.to(torch.float32).contiguous() for t in tab)
     return ops.norm_rope_rows(x, scale, cos, sin, heads=heads, mode=rope_type, eps=eps)
 
-  q = run(query, norm_q_scale, q_tab)
+  q = run(query, norm_q_scale if q_mul == 1.0 else norm_q_scale * q_mul, q_tab)
   k = run(key, norm_k_scale, k_tab) if key is not None else None
   return q, k
 
@@ -342,18 +344,21 @@ def _split_table(freqs_cis, seq: int, d: int):
 
 
 def hip_norm_rope(q, k, wq, wk, freqs_cis, heads: int, eps: float = 1e-6, per_head: bool = False,
-                  wq_txt=None, wk_txt=None, n_txt: int = 0, out_layout: str = "bshd"):
+                  wq_txt=None, wk_txt=None, n_txt: int = 0, out_layout: str = "bshd", q_mul: float = 1.0):
   """The fused prologue the attention modules call in place of their inline norm + rope.
 
   per_head=False: FlaxWanAttention.__call__ lines attention_flax.py:2655-2677 (q, k are [B,S,H*D]).
   per_head=True : FlaxFluxAttention.__call__ lines :2989-3020 (q, k are [B,S,H,D] views).
   freqs_cis=None is the norm-only mode of the cross-attention (:2671).  Returns logical [B,S,H,D]
   views laid out as `out_layout`, ready for `hip_flash` with no transpose in between.
+  `q_mul` is multiplied into the query before its single rounding: with q_mul=ops.folded_q_mul(D) and
+  context["scale"]=ops.FOLDED_SCALE the softmax scale is carried by the prologue, where the reference carries it by
+  two bf16 multiplies of k and q (:1783, :610), and the attention kernel saves its multiply per logit.
   """
   if per_head:
     b, s, h, d = q.shape
     cos, sin = _split_table(freqs_cis, s, d)
-    return ops.norm_rope_perhead(q, k, wq, wk, cos, sin, eps, wq_txt, wk_txt, n_txt, out_layout)
+    return ops.norm_rope_perhead(q, k, wq, wk, cos, sin, eps, wq_txt, wk_txt, n_txt, out_layout, q_mul)
   b, s, n = q.shape
   cos, sin = _split_table(freqs_cis, s, n // heads)
-  return ops.norm_rope_fullrow(q, k, wq, wk, cos, sin, heads, eps, out_layout)
+  return ops.norm_rope_fullrow(q, k, wq, wk, cos, sin, heads, eps, out_layout, q_mul)

@@ -70,7 +70,7 @@ __device__ __forceinline__ bf16x8 read_vt(const __bf16* p0, const __bf16* p1) {
   return __builtin_bit_cast(bf16x8, r);
 }
 
-template <int NW>
+template <int NW, bool PRE>
 __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
@@ -149,7 +149,13 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[db][i] = 0.f;
   float m = -1e30f, l = 0.f;
-  float mc = m * c;  // the rows' reference point in log2 units
+  float mc = PRE ? 0.f : m * c;  // the rows' reference point in log2 units
+  // PRE (scale * log2(e) == 1: the caller's q already carries the factor): the logits need no multiply, and the
+  // reference point is subtracted by the MFMA itself, as the start value of every QK accumulator chain.  The
+  // first key block then always takes the cold branch, which puts the reference at that block's maximum.
+  f32x16 negm;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) negm[i] = 0.f;
 
   // lane-constant LDS offsets
   // K fragment j (logical chunk 2j + hh) of row l32 sits at chunk position (2j + hh) ^ (l32 & 3): pair j ^ x1,
@@ -204,7 +210,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
         if (j == 0) {                                                                                         \
           f32x16 z;                                                                                           \
           _Pragma("unroll") for (int i = 0; i < 16; ++i) z[i] = 0.f;                                          \
-          SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[0], qf[0], z, 0, 0, 0);                            \
+          SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[0], qf[0], PRE ? negm : z, 0, 0, 0);               \
         } else {                                                                                              \
           SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[j & 3], qf[j], SN, 0, 0, 0);                       \
         }                                                                                                     \
@@ -214,7 +220,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
       const int e1 = n < kS0 ? 0 : ((n + 1 - kS0) * 16) / (16 - kS0);                                         \
       _Pragma("unroll") for (int e = 0; e < 16; ++e) {                                                        \
         if (e >= e0 && e < e1) {                                                                              \
-          const float x = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[e], c, -mc));                              \
+          const float x = __builtin_amdgcn_exp2f(PRE ? SC[e] : __builtin_fmaf(SC[e], c, -mc));                \
           if ((e & 1) == 0) {                                                                                 \
             pe = x;                                                                                           \
             /* pins the work in its slot: otherwise the compiler sinks the softmax below the MFMA stream */  \
@@ -229,20 +235,28 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
       }                                                                                                       \
       __builtin_amdgcn_sched_barrier(0);                                                                      \
     }                                                                                                         \
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lsum <= kTrig)) != 0, 0)) {                            \
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lsum <= kTrig)) != 0 || (PRE && (BLK) == 0), 0)) {     \
       float mloc = SC[0];                                                                                     \
       _Pragma("unroll") for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, SC[i]);                               \
       mloc = xhalf_max(mloc);                                                                                 \
       /* every row of a triggered wave moves to its true maximum: right after, the block's sum is at most */  \
       /* 16, so a row can trigger again only when its maximum has grown by another 3 log2 units           */  \
-      const float mnew = fmaxf(m, mloc);                                                                      \
-      const float alpha = __builtin_amdgcn_exp2f((m - mnew) * c); /* exactly 1 for rows that keep m */        \
-      m = mnew;                                                                                               \
-      mc = m * c;                                                                                             \
+      float alpha;                                                                                            \
+      if (PRE) { /* SC and SN hold logits minus the old reference: shift them, and the chains' start value */ \
+        const float dm = (BLK) == 0 ? mloc : fmaxf(mloc, 0.f);                                                \
+        alpha = (BLK) == 0 ? 0.f : __builtin_amdgcn_exp2f(-dm);                                               \
+        mc += dm;                                                                                             \
+        _Pragma("unroll") for (int i = 0; i < 16; ++i) { SC[i] -= dm; SN[i] -= dm; negm[i] = -mc; }           \
+      } else {                                                                                                \
+        const float mnew = fmaxf(m, mloc);                                                                    \
+        alpha = __builtin_amdgcn_exp2f((m - mnew) * c); /* exactly 1 for rows that keep m */                  \
+        m = mnew;                                                                                             \
+        mc = m * c;                                                                                           \
+      }                                                                                                       \
       lsum = 0.f;                                                                                             \
       _Pragma("unroll") for (int e = 0; e < 16; e += 2) {                                                     \
-        const float x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[e], c, -mc));                               \
-        const float x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(SC[e + 1], c, -mc));                           \
+        const float x0 = __builtin_amdgcn_exp2f(PRE ? SC[e] : __builtin_fmaf(SC[e], c, -mc));                 \
+        const float x1 = __builtin_amdgcn_exp2f(PRE ? SC[e + 1] : __builtin_fmaf(SC[e + 1], c, -mc));         \
         lsum += x0 + x1;                                                                                      \
         PC[e >> 3][(e >> 1) & 3] = pack2(x0, x1);                                                             \
       }                                                                                                       \
@@ -579,7 +593,9 @@ static int launch_fwd(hipStream_t st, AttnArgs a, int B) {
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
-  auto kern = attn_fwd_bf16_kernel<NW>;
+  // scale * log2(e) == 1 (to f32 round-off): the caller folded the factor into q; the logits need no multiply
+  const bool pre = a.c > 1.0f - 1e-6f && a.c < 1.0f + 1e-6f;
+  auto kern = pre ? attn_fwd_bf16_kernel<NW, true> : attn_fwd_bf16_kernel<NW, false>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
     return MDATTN_E_LAUNCH;
   hipLaunchKernelGGL(kern, dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);

@@ -77,7 +77,7 @@ ffi::Error FwdBf16BiasImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer 
 
 ffi::Error NormRopeFullrowImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer wq, ffi::AnyBuffer wk,
                                ffi::AnyBuffer cos, ffi::AnyBuffer sin, ffi::Result<ffi::AnyBuffer> q_out,
-                               ffi::Result<ffi::AnyBuffer> k_out, float eps, int64_t heads, int64_t rope) {
+                               ffi::Result<ffi::AnyBuffer> k_out, float eps, float q_mul, int64_t heads, int64_t rope) {
   auto d = q.dimensions();
   if (d.size() != 3 || heads <= 0 || d[2] % heads) return ffi::Error::InvalidArgument("mdattn_norm_rope_fullrow: q must be [B,S,H*D]");
   const int64_t B = d[0], S = d[1], N = d[2], D = N / heads;
@@ -86,13 +86,13 @@ ffi::Error NormRopeFullrowImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuf
                                           wq.untyped_data(), wk.untyped_data(),
                                           rope ? static_cast<const float*>(cos.untyped_data()) : nullptr,
                                           rope ? static_cast<const float*>(sin.untyped_data()) : nullptr,
-                                          (int)B, (int)S, (int)heads, (int)D, eps, S * N, N, &so),
+                                          (int)B, (int)S, (int)heads, (int)D, eps, q_mul, S * N, N, &so),
                  "mdattn_norm_rope_fullrow");
 }
 
 ffi::Error NormRopePerheadImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer wq, ffi::AnyBuffer wk,
                                ffi::AnyBuffer cos, ffi::AnyBuffer sin, ffi::Result<ffi::AnyBuffer> q_out,
-                               ffi::Result<ffi::AnyBuffer> k_out, float eps, int64_t rope) {
+                               ffi::Result<ffi::AnyBuffer> k_out, float eps, float q_mul, int64_t rope) {
   int64_t B, S, H, D;
   mdattn_strides si;
   if (!Describe(q.dimensions(), 0, &B, &S, &H, &D, &si)) return ffi::Error::InvalidArgument("mdattn_norm_rope_perhead: q must be [B,S,H,D]");
@@ -100,7 +100,7 @@ ffi::Error NormRopePerheadImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuf
                                           wq.untyped_data(), wk.untyped_data(), nullptr, nullptr, 0,
                                           rope ? static_cast<const float*>(cos.untyped_data()) : nullptr,
                                           rope ? static_cast<const float*>(sin.untyped_data()) : nullptr,
-                                          (int)B, (int)S, (int)H, (int)D, eps, &si, &si),
+                                          (int)B, (int)S, (int)H, (int)D, eps, q_mul, &si, &si),
                  "mdattn_norm_rope_perhead");
 }
 
@@ -132,7 +132,7 @@ ffi::Error NormRopeRowsImpl(hipStream_t stream, ffi::AnyBuffer x, ffi::AnyBuffer
                                        static_cast<const float*>(w.untyped_data()),
                                        mode ? static_cast<const float*>(cos.untyped_data()) : nullptr,
                                        mode ? static_cast<const float*>(sin.untyped_data()) : nullptr, (int)mode,
-                                       (int)B, (int)S, (int)heads, (int)D, eps, S * N, N, &so),
+                                       (int)B, (int)S, (int)heads, (int)D, eps, q_mul, S * N, N, &so),
                  "mdattn_norm_rope_rows");
 }
 
@@ -172,7 +172,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopeFullrow, NormRopeFullrowImpl,
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
                                   .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
-                                  .Attr<float>("eps").Attr<int64_t>("heads").Attr<int64_t>("rope"));
+                                  .Attr<float>("eps").Attr<float>("q_mul").Attr<int64_t>("heads").Attr<int64_t>("rope"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnBwdBf16, BwdBf16Impl,
                               ffi::Ffi::Bind()
@@ -195,7 +195,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopePerhead, NormRopePerheadImpl,
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
                                   .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
-                                  .Attr<float>("eps").Attr<int64_t>("rope"));
+                                  .Attr<float>("eps").Attr<float>("q_mul").Attr<int64_t>("rope"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnMerge, MergeImpl,
                               ffi::Ffi::Bind()

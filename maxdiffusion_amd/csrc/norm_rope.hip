@@ -13,6 +13,7 @@ struct NormRopeFullArgs {
   const float4* sin;
   int S, H, D, N;         // N = H*D
   float eps, inv_n;
+  float q_mul;            // constant folded into the q output before its rounding
   int64_t in_sb, in_ss;
   int64_t out_sb, out_ss, out_sh;
 };
@@ -68,6 +69,7 @@ __global__ __launch_bounds__(256) void norm_rope_fullrow_kernel(NormRopeFullArgs
       const float y = __builtin_amdgcn_rsqf(x);
       // one Newton step brings v_rsq_f32 (1 ulp) to f32 round-off: y*(1.5 - 0.5*x*y*y)
       inv[t] = y * (1.5f - 0.5f * x * y * y);
+      if (t == 0) inv[t] *= a.q_mul;
     }
   }
 
@@ -116,6 +118,7 @@ struct NormRopeHeadArgs {
   int S, H, n_txt;
   int64_t rows;  // B*S*H
   float eps;
+  float q_mul;   // constant folded into the q output before its rounding
   int64_t in_sb, in_ss, in_sh, out_sb, out_ss, out_sh;
 };
 
@@ -174,6 +177,7 @@ __global__ __launch_bounds__(256) void norm_rope_perhead_kernel(NormRopeHeadArgs
         const float x = ss * (1.0f / D) + a.eps;
         float inv = __builtin_amdgcn_rsqf(x);
         inv = inv * (1.5f - 0.5f * x * inv * inv);
+        if (t == 0) inv *= a.q_mul;
         const uint4* wp = (a.w_txt[t] && tok[r] < a.n_txt) ? a.w_txt[t] : a.w[t];
         unpack8(wp[lane], w);
 #pragma unroll
@@ -309,13 +313,13 @@ using namespace mdattn;
 
 extern "C" int mdattn_norm_rope_fullrow(void* stream, const void* q_in, const void* k_in, void* q_out, void* k_out,
                                         const void* wq, const void* wk, const float* cos, const float* sin,
-                                        int B, int S, int H, int D, float eps,
+                                        int B, int S, int H, int D, float eps, float q_mul,
                                         int64_t in_stride_batch, int64_t in_stride_seq,
                                         const mdattn_strides* out_strides) {
   if (!q_in || !q_out || !wq || B <= 0 || S <= 0 || H <= 0 || D <= 0 || !out_strides) return MDATTN_E_BADARG;
   if ((k_in == nullptr) != (k_out == nullptr) || (k_in && !wk)) return MDATTN_E_BADARG;
   if ((cos == nullptr) != (sin == nullptr)) return MDATTN_E_BADARG;
-  if (!(eps >= 0.f)) return MDATTN_E_BADARG;
+  if (!(eps >= 0.f) || !(q_mul > 0.f) || !(q_mul < 1e30f)) return MDATTN_E_BADARG;
   const int64_t N = (int64_t)H * D;
   if (D % 8 != 0 || N > 8192) return MDATTN_E_UNSUPPORTED;
   if (B > 65535) return MDATTN_E_UNSUPPORTED;
@@ -330,7 +334,7 @@ extern "C" int mdattn_norm_rope_fullrow(void* stream, const void* q_in, const vo
   a.x_out[0] = (uint4*)q_out; a.x_out[1] = (uint4*)k_out;
   a.w[0] = (const uint4*)wq; a.w[1] = (const uint4*)wk;
   a.cos = (const float4*)cos; a.sin = (const float4*)sin;
-  a.S = S; a.H = H; a.D = D; a.N = (int)N; a.eps = eps; a.inv_n = 1.0f / (float)N;
+  a.S = S; a.H = H; a.D = D; a.N = (int)N; a.eps = eps; a.inv_n = 1.0f / (float)N; a.q_mul = q_mul;
   a.in_sb = in_stride_batch; a.in_ss = in_stride_seq;
   a.out_sb = out_strides->batch; a.out_ss = out_strides->seq; a.out_sh = out_strides->head;
   dim3 grid(S, B), block(256);
@@ -346,12 +350,12 @@ extern "C" int mdattn_norm_rope_fullrow(void* stream, const void* q_in, const vo
 extern "C" int mdattn_norm_rope_perhead(void* stream, const void* q_in, const void* k_in, void* q_out, void* k_out,
                                         const void* wq, const void* wk, const void* wq_txt, const void* wk_txt,
                                         int n_txt, const float* cos, const float* sin, int B, int S, int H, int D,
-                                        float eps, const mdattn_strides* in_strides,
+                                        float eps, float q_mul, const mdattn_strides* in_strides,
                                         const mdattn_strides* out_strides) {
   if (!q_in || !q_out || !wq || B <= 0 || S <= 0 || H <= 0 || D <= 0 || !in_strides || !out_strides) return MDATTN_E_BADARG;
   if ((k_in == nullptr) != (k_out == nullptr) || (k_in && !wk)) return MDATTN_E_BADARG;
   if ((cos == nullptr) != (sin == nullptr)) return MDATTN_E_BADARG;
-  if (n_txt < 0 || n_txt > S || !(eps >= 0.f)) return MDATTN_E_BADARG;
+  if (n_txt < 0 || n_txt > S || !(eps >= 0.f) || !(q_mul > 0.f) || !(q_mul < 1e30f)) return MDATTN_E_BADARG;
   if (D != 64 && D != 128 && D != 256) return MDATTN_E_UNSUPPORTED;
   if (!aligned16(q_in) || !aligned16(q_out) || !aligned16(wq) || !aligned16(k_in) || !aligned16(k_out) ||
       !aligned16(wk) || !aligned16(wq_txt) || !aligned16(wk_txt) || !aligned16(cos) || !aligned16(sin))
@@ -364,7 +368,7 @@ extern "C" int mdattn_norm_rope_perhead(void* stream, const void* q_in, const vo
   a.w[0] = (const uint4*)wq; a.w[1] = (const uint4*)wk;
   a.w_txt[0] = (const uint4*)wq_txt; a.w_txt[1] = k_in ? (const uint4*)wk_txt : nullptr;
   a.cos = (const float4*)cos; a.sin = (const float4*)sin;
-  a.S = S; a.H = H; a.n_txt = n_txt; a.rows = (int64_t)B * S * H; a.eps = eps;
+  a.S = S; a.H = H; a.n_txt = n_txt; a.rows = (int64_t)B * S * H; a.eps = eps; a.q_mul = q_mul;
   a.in_sb = in_strides->batch; a.in_ss = in_strides->seq; a.in_sh = in_strides->head;
   a.out_sb = out_strides->batch; a.out_ss = out_strides->seq; a.out_sh = out_strides->head;
   constexpr int RPT = 4;

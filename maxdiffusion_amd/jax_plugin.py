@@ -109,8 +109,10 @@ def hip_flash_attention_vjp(q, k, v, scale: float):
   return attn(q, k, v)
 
 
-def hip_norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6):
-  """q, k [B,S,H*D] bf16; cos/sin f32 [S,D/2] or None -> (q_out, k_out) [B,S,H,D] bf16."""
+def hip_norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6, q_mul: float = 1.0):
+  """q, k [B,S,H*D] bf16; cos/sin f32 [S,D/2] or None -> (q_out, k_out) [B,S,H,D] bf16.  `q_mul` is multiplied into
+  q_out before its rounding: D**-0.5 * log2(e) here and scale = ln 2 in hip_flash_attention carry the softmax scale
+  in the prologue."""
   jax, jnp = _require_jax()
   import numpy as np
 
@@ -121,7 +123,7 @@ def hip_norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6)
     cos = sin = jnp.zeros((1, 1), jnp.float32)
   out = jax.ShapeDtypeStruct((b, s, heads, d), jnp.bfloat16)
   call = jax.ffi.ffi_call("mdattn_norm_rope_fullrow", (out, out), vmap_method="sequential")
-  return call(q, k, wq, wk, cos, sin, eps=np.float32(eps), heads=np.int64(heads), rope=np.int64(rope))
+  return call(q, k, wq, wk, cos, sin, eps=np.float32(eps), q_mul=np.float32(q_mul), heads=np.int64(heads), rope=np.int64(rope))
 
 
 def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotary_emb=None, k_rotary_emb=None,

@@ -17,10 +17,19 @@ from ._lib import Strides
 
 __all__ = [
     "norm_rope_fullrow", "norm_rope_perhead", "norm_rope_rows", "flash_attention", "flash_attention_backward", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
-    "merge_partial", "finalize", "new_merge_state", "LSE_INIT",
+    "merge_partial", "finalize", "new_merge_state", "LSE_INIT", "FOLDED_SCALE", "folded_q_mul",
 ]
 
 LSE_INIT = -1e30
+
+# Folding the softmax scale into the prologue: norm_rope_*(..., q_mul=folded_q_mul(D)) emits q * D^-1/2 * log2(e)
+# (still one rounding), and the attention entry points, given scale=FOLDED_SCALE = ln 2, see scale * log2(e) == 1:
+# their logits come out of the MFMA in log2 units and need no multiply.  Results are those of scale = D^-1/2.
+FOLDED_SCALE = math.log(2.0)
+
+
+def folded_q_mul(head_dim: int, scale: float | None = None) -> float:
+  return (head_dim**-0.5 if scale is None else scale) * math.log2(math.e)
 
 
 def _ptr(t):
@@ -60,10 +69,11 @@ def _table(t, s, d, name):
   return t
 
 
-def norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6, out_layout: str = "bshd"):
+def norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6, out_layout: str = "bshd", q_mul: float = 1.0):
   """q, k: bf16 [B, S, H*D] (k may be None) -> (q_out, k_out) logical [B,S,H,D] views in `out_layout`.
 
   RMSNorm over H*D, then rotation of interleaved pairs by the [S, D/2] table (cos/sin None: norm only).
+  `q_mul` is multiplied into q_out before its single rounding (see FOLDED_Q_MUL / FOLDED_SCALE).
   """
   _check_dev(q, k, wq, wk, cos, sin)
   if q.dim() != 3 or q.dtype != torch.bfloat16 or q.stride(2) != 1:
@@ -80,7 +90,7 @@ def norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6, out
   st = _strides(q_out)
   rc = _lib.load().mdattn_norm_rope_fullrow(
       _stream(), _ptr(q), _ptr(k), _ptr(q_out), _ptr(k_out), _ptr(wq), _ptr(wk), _ptr(cos), _ptr(sin),
-      b, s, heads, d, eps, q.stride(0), q.stride(1), ctypes.byref(st))
+      b, s, heads, d, eps, q_mul, q.stride(0), q.stride(1), ctypes.byref(st))
   _lib.check(rc, "mdattn_norm_rope_fullrow")
   return q_out, k_out
 
@@ -115,8 +125,9 @@ def norm_rope_rows(x, w, cos=None, sin=None, heads: int = 1, mode: str = "none",
 
 
 def norm_rope_perhead(q, k, wq, wk, cos, sin, eps: float = 1e-6, wq_txt=None, wk_txt=None, n_txt: int = 0,
-                      out_layout: str = "bshd"):
-  """q, k: bf16 logical [B, S, H, D] views (k may be None); RMSNorm over D per head, then RoPE."""
+                      out_layout: str = "bshd", q_mul: float = 1.0):
+  """q, k: bf16 logical [B, S, H, D] views (k may be None); RMSNorm over D per head, then RoPE.
+  `q_mul` is multiplied into q_out before its single rounding."""
   _check_dev(q, k, wq, wk, wq_txt, wk_txt, cos, sin)
   if q.dtype != torch.bfloat16:
     raise ValueError("q must be bf16")
@@ -129,7 +140,7 @@ def norm_rope_perhead(q, k, wq, wk, cos, sin, eps: float = 1e-6, wq_txt=None, wk
   si, so = _strides(q), _strides(q_out)
   rc = _lib.load().mdattn_norm_rope_perhead(
       _stream(), _ptr(q), _ptr(k), _ptr(q_out), _ptr(k_out), _ptr(wq), _ptr(wk), _ptr(wq_txt), _ptr(wk_txt), n_txt,
-      _ptr(cos), _ptr(sin), b, s, h, d, eps, ctypes.byref(si), ctypes.byref(so))
+      _ptr(cos), _ptr(sin), b, s, h, d, eps, q_mul, ctypes.byref(si), ctypes.byref(so))
   _lib.check(rc, "mdattn_norm_rope_perhead")
   return q_out, k_out
 

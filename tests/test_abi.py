@@ -74,17 +74,18 @@ def test_bad_arguments_are_rejected_on_the_host(lib):
   assert f(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 128, None, st, st, st, 0.1) == _lib.E_BADARG
 
   g = lib.mdattn_norm_rope_fullrow
-  assert g(None, None, None, fake, None, fake, None, None, None, 1, 8, 4, 128, 1e-6, 0, 512, st) == _lib.E_BADARG
-  assert g(None, fake, fake, fake, None, fake, fake, None, None, 1, 8, 4, 128, 1e-6, 0, 512, st) == _lib.E_BADARG  # k_in without k_out
-  assert g(None, fake, None, fake, None, fake, None, fake, None, 1, 8, 4, 128, 1e-6, 0, 512, st) == _lib.E_BADARG  # cos without sin
-  assert g(None, fake, None, fake, None, fake, None, None, None, 1, 8, 80, 128, 1e-6, 0, 10240, st) == _lib.E_UNSUPPORTED  # H*D > 8192
-  assert g(None, fake, None, fake, None, fake, None, None, None, 1, 8, 4, 128, 1e-6, 0, 100, st) == _lib.E_BADARG  # row stride < H*D
-  assert g(None, fake, None, odd, None, fake, None, None, None, 1, 8, 4, 128, 1e-6, 0, 512, st) == _lib.E_ALIGN
+  assert g(None, None, None, fake, None, fake, None, None, None, 1, 8, 4, 128, 1e-6, 1.0, 0, 512, st) == _lib.E_BADARG
+  assert g(None, fake, fake, fake, None, fake, fake, None, None, 1, 8, 4, 128, 1e-6, 1.0, 0, 512, st) == _lib.E_BADARG  # k_in without k_out
+  assert g(None, fake, None, fake, None, fake, None, fake, None, 1, 8, 4, 128, 1e-6, 1.0, 0, 512, st) == _lib.E_BADARG  # cos without sin
+  assert g(None, fake, None, fake, None, fake, None, None, None, 1, 8, 80, 128, 1e-6, 1.0, 0, 10240, st) == _lib.E_UNSUPPORTED  # H*D > 8192
+  assert g(None, fake, None, fake, None, fake, None, None, None, 1, 8, 4, 128, 1e-6, 1.0, 0, 100, st) == _lib.E_BADARG  # row stride < H*D
+  assert g(None, fake, None, odd, None, fake, None, None, None, 1, 8, 4, 128, 1e-6, 1.0, 0, 512, st) == _lib.E_ALIGN
+  assert g(None, fake, None, fake, None, fake, None, None, None, 1, 8, 4, 128, 1e-6, 0.0, 0, 512, st) == _lib.E_BADARG  # q_mul must be > 0
 
   p = lib.mdattn_norm_rope_perhead
-  assert p(None, fake, None, fake, None, fake, None, None, None, 0, None, None, 1, 8, 4, 96, 1e-6, st, st) == _lib.E_UNSUPPORTED
-  assert p(None, fake, None, fake, None, fake, None, None, None, 9, None, None, 1, 8, 4, 128, 1e-6, st, st) == _lib.E_BADARG  # n_txt > S
-  assert p(None, fake, None, fake, None, None, None, None, None, 0, None, None, 1, 8, 4, 128, 1e-6, st, st) == _lib.E_BADARG
+  assert p(None, fake, None, fake, None, fake, None, None, None, 0, None, None, 1, 8, 4, 96, 1e-6, 1.0, st, st) == _lib.E_UNSUPPORTED
+  assert p(None, fake, None, fake, None, fake, None, None, None, 9, None, None, 1, 8, 4, 128, 1e-6, 1.0, st, st) == _lib.E_BADARG  # n_txt > S
+  assert p(None, fake, None, fake, None, None, None, None, None, 0, None, None, 1, 8, 4, 128, 1e-6, 1.0, st, st) == _lib.E_BADARG
 
   m = lib.mdattn_merge
   assert m(None, fake, fake, fake, None, 0, 1, 4, 8, 128, st, st) == _lib.E_BADARG

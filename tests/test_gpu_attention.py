@@ -296,3 +296,68 @@ def test_reference_point_moves_head_dim_64_and_masked(dev, profile):
   out, lse = ops.flash_attention(to_dev_bf16(q, dev), to_dev_bf16(k, dev), to_dev_bf16(v, dev), return_lse=True, key_bias=bias)
   ro, rl = O.attention(hsd(q), hsd(k), hsd(v), 128**-0.5, kv_mask=keep[0])
   _check(hsd(to_np(out)), to_np(lse)[0], ro, rl, f"masked {profile}", lse_abs=2e-3 if profile == "late_spike" else LSE_ABS)
+
+
+def _folded_run(q_f32, k, v, dev):
+  """What the prologue hands over with q_mul = D^-1/2 * log2(e): bf16(q * q_mul); the kernel is given scale = ln 2."""
+  D = q_f32.shape[-1]
+  qp = O.bf16_round((q_f32 * np.float32(ops.folded_q_mul(D))).astype(np.float32))
+  out, lse = ops.flash_attention(to_dev_bf16(qp, dev), to_dev_bf16(k, dev), to_dev_bf16(v, dev), scale=ops.FOLDED_SCALE, return_lse=True)
+  ro, rl = O.attention(hsd(qp), hsd(k), hsd(v), ops.FOLDED_SCALE)
+  return hsd(to_np(out)), to_np(lse)[0], ro, rl
+
+
+@pytest.mark.parametrize("var", [1, 2, 3])
+@pytest.mark.parametrize("sq,skv,mult", [(1, 1, 1.0), (31, 65, 1.0), (257, 63, 1.0), (300, 333, 1.0), (100, 4097, 1.0), (500, 700, 6.0)])
+def test_folded_scale_ragged_and_sharp(dev, variant, var, sq, skv, mult):
+  """scale * log2(e) == 1: the pipelined kernel takes its path without a multiply per logit, the reference point
+  being subtracted by the MFMA's start accumulator; the flat schedule sees an ordinary scale."""
+  variant(var)
+  H = 2
+  q = (np.random.default_rng(0).standard_normal((1, sq, H, 128)) * mult).astype(np.float32)
+  k, v = O.normal_bf16((1, skv, H, 128), 1), O.normal_bf16((1, skv, H, 128), 2)
+  out, lse, ro, rl = _folded_run(q, k, v, dev)
+  _check(out, lse, ro, rl, f"folded scale, variant {var} Sq={sq} Skv={skv} x{mult}")
+
+
+@pytest.mark.parametrize("profile", ["ascending", "descending", "plateau", "late_spike", "all_far_below_zero"])
+def test_folded_scale_reference_point_moves(dev, variant, profile):
+  variant(1)
+  H, sq, skv = 2, 150, 1500
+  if profile == "all_far_below_zero":  # every logit ~ -140 log2 units: the first block has to set the reference point
+    q = np.full((1, sq, H, 128), -3.0, np.float32)
+    k = np.full((1, skv, H, 128), 3.0, np.float32)
+    k[0, :, :, 0] += (np.arange(skv, dtype=np.float32) * 0.01)[:, None]
+    k = O.bf16_round(k)
+  else:
+    qs, ks = zip(*(_structured_logits(sq, skv, 128, profile, seed=5 + h) for h in range(H)))
+    q, k = np.stack(qs, 1)[None], np.stack(ks, 1)[None]
+  v = O.normal_bf16((1, skv, H, 128), 2)
+  out, lse, ro, rl = _folded_run(q, k, v, dev)
+  _check(out, lse, ro, rl, f"folded scale {profile}", lse_abs=2e-3 if profile == "late_spike" else LSE_ABS)
+
+
+def test_folded_scale_equals_plain_scale_through_the_prologue(dev):
+  """The product path of the benchmark: prologue with q_mul, attention with scale = ln 2, against the oracle chain
+  norm -> rope -> attention(scale = D^-1/2) and against the un-folded kernels."""
+  w = O.WORKLOADS["wan1.3b"]
+  H, S, D = w.heads, 3 * 10 * 13 * 4, 128
+  cos, sin = O.wan_rope_table((3, 20, 26), D)
+  q, k, v = (O.normal_bf16((1, S, H * D), s) for s in (0, 1, 2))
+  wq, wk = O.norm_weight(H * D, 3), O.norm_weight(H * D, 4)
+  qd, kd, vd = (to_dev_bf16(x, dev) for x in (q, k, v))
+  args = (to_dev_bf16(wq, dev), to_dev_bf16(wk, dev), torch.from_numpy(cos).to(dev), torch.from_numpy(sin).to(dev), H)
+  qn, kn = ops.norm_rope_fullrow(qd, kd, *args, q_mul=ops.folded_q_mul(D))
+  out, lse = ops.flash_attention(qn, kn, vd.view(1, S, H, D), scale=ops.FOLDED_SCALE, return_lse=True)
+  qe, ke = O.norm_rope_fullrow(q, wq, cos, sin, H), O.norm_rope_fullrow(k, wk, cos, sin, H)
+  # the prologue's q is the oracle's times q_mul, rounded once
+  mx, _ = err_stats(to_np(qn), qe * ops.folded_q_mul(D))
+  assert mx <= 4e-3  # half an ulp of bf16 values up to 2
+  ro, rl = O.attention(hsd(qe), hsd(ke), hsd(v.reshape(1, S, H, D)), w.scale)
+  # the oracle chain keeps q and k unrounded between prologue and attention, the kernels round them to bf16 once:
+  # that rounding alone moves the LSE by ~1e-3 (the 1e-3 bar is for attention on given bf16 inputs)
+  _check(hsd(to_np(out)), to_np(lse)[0], ro, rl, "prologue with folded scale -> attention", lse_abs=3e-3)
+  q0, k0 = ops.norm_rope_fullrow(qd, kd, *args)
+  out0, lse0 = ops.flash_attention(q0, k0, vd.view(1, S, H, D), scale=w.scale, return_lse=True)
+  _check(hsd(to_np(out0)), to_np(lse0)[0], ro, rl, "plain prologue -> attention", lse_abs=3e-3)
+  assert float((out.float() - out0.float()).abs().max()) <= 4e-3 and float((lse - lse0).abs().max()) <= 3e-3

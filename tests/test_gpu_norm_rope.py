@@ -153,3 +153,22 @@ def test_host_side_validation_raises(dev):
     ops.norm_rope_fullrow(q, None, w, None, torch.zeros(8, 60, device=dev), torch.zeros(8, 60, device=dev), heads=4)
   with pytest.raises(ValueError, match="no CPU path"):
     ops.norm_rope_fullrow(q.cpu(), None, w.cpu(), None, None, None, heads=4)
+
+
+def test_q_mul_scales_the_query_only(dev):
+  """q_mul is folded into the query before its single rounding; the key is untouched."""
+  g = golden("norm_rope_wan.npz")
+  H = int(g["heads"])
+  q, k = bits_to_dev(g["q"], dev), bits_to_dev(g["k"], dev)
+  wq, wk = bits_to_dev(g["wq"], dev), bits_to_dev(g["wk"], dev)
+  cos, sin = _t(g["cos"], dev), _t(g["sin"], dev)
+  m = ops.folded_q_mul(128)
+  qo, ko = ops.norm_rope_fullrow(q, k, wq, wk, cos, sin, H, q_mul=m)
+  _assert_close(to_np(qo) / m, g["q_out"], "wan golden q with q_mul")
+  _assert_close(to_np(ko), g["k_out"], "wan golden k with q_mul")
+  f = golden("norm_rope_flux.npz")
+  q, k = bits_to_dev(f["q"], dev), bits_to_dev(f["k"], dev)
+  w = [bits_to_dev(f[n], dev) for n in ("wq", "wk", "wq_txt", "wk_txt")]
+  qo, ko = ops.norm_rope_perhead(q, k, w[0], w[1], _t(f["cos"], dev), _t(f["sin"], dev), wq_txt=w[2], wk_txt=w[3], n_txt=int(f["n_txt"]), q_mul=m)
+  _assert_close(to_np(qo) / m, f["q_out"], "flux golden q with q_mul")
+  _assert_close(to_np(ko), f["k_out"], "flux golden k with q_mul")
