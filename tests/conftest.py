@@ -11,7 +11,7 @@ for _p in (ROOT, os.path.join(ROOT, "tests")):
 
 
 def pytest_configure(config):
-  config.addinivalue_line("markers", "gpu: needs a real MI355X (run through gpurun / at round end)")
+  config.addinivalue_line("markers", "gpu: needs a real MI355X")
 
 
 def _has_gpu() -> bool:
