@@ -15,9 +15,9 @@
 //                (after the bf16 convert), and the A operand V^T comes from the row-major V tile
 //                through the transposing LDS read (ds_read_b64_tr_b16).
 //   softmax    = exp2 with scale*log2(e) folded into one FMA per logit; f32 state.  A row's reference
-//                point m is not its running maximum: it moves only when a logit exceeds it by more than
-//                2^8, which the row's partial sum reveals, so the hot stream computes no maximum at all
-//                and the accumulator rescale sits in a cold branch.
+//                point m is not its running maximum: it only keeps P, l and O inside the f32 exponent range and
+//                moves when a logit exceeds it by about 20 log2 units, which the row's partial sum reveals, so
+//                the hot stream computes no maximum at all and the accumulator rescale sits in a cold branch.
 //   pipelining = the vector ALU issues through the same port as the MFMAs.  Phases of pure MFMA
 //                followed by phases of pure VALU leave the matrix pipe idle half of the time, so the
 //                keys are walked in blocks of 32, and in iteration b every wave issues, interleaved in
@@ -54,8 +54,11 @@ constexpr int kGK = 4 * kD + 32;  // K group stride (1088 B)
 constexpr int kGV = 4 * kD;       // V group stride (1024 B)
 constexpr int kKTile = (kBN / 4) * kGK;
 constexpr int kStage = kKTile + (kBN / 4) * kGV;  // elements per ring stage
-constexpr float kLazy = 8.0f;    // log2 units a row max may lag behind before accumulators are rescaled
-constexpr float kTrig = 128.0f;  // a 16-key partial row sum above this sends the wave to the rescale branch (< 2^kLazy)
+// A 16-key partial row sum above this sends the wave to the branch that moves the rows' reference points.  The
+// reference point only has to keep P, l and O inside the f32 / bf16 exponent range (the result does not depend on it,
+// and bf16's relative precision is the same at every magnitude), so the alarm can sit far out: 2^24 lets a row's
+// logits climb 20 log2 units above its reference before anything happens, and leaves 100 binades of headroom.
+constexpr float kTrig = 16777216.0f;
 constexpr int kS0 = 2;           // first slot of an iteration that touches the block's logits
 constexpr int kLA = 1;           // LDS look-ahead: a slot requests the fragment of the kLA-th next MFMA of its kind
                                  // (1, 2 and 3 measure the same)
@@ -182,13 +185,12 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   // KC/KN: K rows of block BLK+1 / BLK+2; VC/VN: V rows of block BLK-1 / BLK.
   // Slot n of the stream: n even -> PV MFMA n/2, n odd -> QK MFMA n/2, each followed by the LDS
   // request for the next MFMA of the same kind, then a share of the softmax of block BLK.  The vector
-  // ALU issues through the same port as the MFMAs and is nearly as busy, so the hot stream carries the
-  // bare minimum per pair of logits: two FMAs, two exp2, one bf16 pack and one dot2 that adds the pair
-  // (as rounded, i.e. exactly what the PV MFMA consumes) to the row sum.  There is no row max in it: the
-  // reference point m of a row moves only when a logit exceeds it by more than kLazy, and then that row's
-  // partial sum exceeds 2^kLazy, so the sum itself is the trigger.  A triggered wave (every row's first
-  // block, then almost never) redoes the block's softmax from the logits with the true maximum in a
-  // cold branch at the end of the iteration, where no PV MFMA of the previous block is outstanding.
+  // ALU issues through the same port as the MFMAs, so the hot stream carries the bare minimum per pair of
+  // logits: two FMAs (none when PRE), two exp2, two adds for the f32 row sum and one bf16 pack.  There is no row
+  // max in it: a row's reference point m moves only when a 16-key partial sum of P exceeds kTrig, which also
+  // catches the +inf that the first block of a row produces from m = -1e30.  A triggered wave (every row's first
+  // block, then almost never) redoes the block's softmax from the logits with the true maximum in a cold branch
+  // at the end of the iteration, where no PV MFMA of the previous block is outstanding.
   // The softmax starts at slot kS0: the last QK MFMA of block BLK was issued at slot 15 of the
   // previous iteration, and reading its result earlier stalls the wave's whole stream.
 #define MDATTN_ITER(SC, SN, PC, PP, KC, KN, VC, VN, BLK) /* KC.. : base pointers [even j, odd j]; VC.. : [segment] */                                                     \
@@ -240,7 +242,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
       _Pragma("unroll") for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, SC[i]);                               \
       mloc = xhalf_max(mloc);                                                                                 \
       /* every row of a triggered wave moves to its true maximum: right after, the block's sum is at most */  \
-      /* 16, so a row can trigger again only when its maximum has grown by another 3 log2 units           */  \
+      /* 16, so a row can trigger again only when its maximum has grown by another 20 log2 units          */  \
       float alpha;                                                                                            \
       if (PRE) { /* SC and SN hold logits minus the old reference: shift them, and the chains' start value */ \
         const float dm = (BLK) == 0 ? mloc : fmaxf(mloc, 0.f);                                                \
