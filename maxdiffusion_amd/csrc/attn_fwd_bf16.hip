@@ -364,7 +364,7 @@ constexpr int kKTileS = (kTS / 4) * kGK;              // elements
 constexpr int kStageS = kKTileS + (kTS / 4) * kGV;    // elements per ring slot
 constexpr int kSlotsS = 3;
 
-template <int NW, bool BIAS, int HD>
+template <int NW, bool BIAS, int HD, bool PRE>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_fwd_bf16_flat_kernel(AttnArgs a) {
   constexpr int NJ = HD / 16;                                    // QK MFMAs per 32-key tile
   constexpr int ND = HD / 32;                                    // 32-wide slabs of d = O accumulators
@@ -443,7 +443,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[db][i] = 0.f;
   float m = -1e30f, l = 0.f;
-  float mc = m * cs;  // the rows' reference point in log2 units
+  float mc = PRE ? 0.f : m * cs;  // the rows' reference point in log2 units
+  f32x16 negm;                    // PRE (see the pipelined kernel): start value of every score accumulator chain
+#pragma unroll
+  for (int i = 0; i < 16; ++i) negm[i] = 0.f;
 
   // per-lane fragment offsets (elements): K fragment j, V slab sg; kV8 = offset of the second transposing read
   // (rows + 8), kVH = offset of the second 16-key half of the tile
@@ -476,7 +479,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + k_off[j]);
-      S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[j], S, 0, 0, 0);
+      S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[j], (PRE && j == 0) ? negm : S, 0, 0, 0);
     }
     if constexpr (BIAS) {
 #pragma unroll
@@ -504,7 +507,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
         float p[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[8 * hb + e], cs, -rf));
+          p[e] = __builtin_amdgcn_exp2f(PRE ? S[8 * hb + e] : __builtin_fmaf(S[8 * hb + e], cs, -rf));
           lsum += p[e];
         }
         P[hb] = __builtin_bit_cast(bf16x8, pack8(p));
@@ -512,16 +515,25 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       return lsum;
     };
     float lsum = soft(mc);
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lsum <= kTrig)) != 0, 0)) {
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lsum <= kTrig)) != 0 || (PRE && t == 0), 0)) {
       float mloc = S[0];
 #pragma unroll
       for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, S[i]);
       mloc = xhalf_max(mloc);
-      const float mnew = fmaxf(m, mloc);
-      float alpha = __builtin_amdgcn_exp2f((m - mnew) * cs);
+      float alpha;
+      if constexpr (PRE) {  // S holds logits minus the old reference: shift them and the chains' start value
+        const float dm = t == 0 ? mloc : fmaxf(mloc, 0.f);
+        alpha = t == 0 ? 0.f : __builtin_amdgcn_exp2f(-dm);
+        mc += dm;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { S[i] -= dm; negm[i] = -mc; }
+      } else {
+        const float mnew = fmaxf(m, mloc);
+        alpha = __builtin_amdgcn_exp2f((m - mnew) * cs);
+        m = mnew;
+        mc = m * cs;
+      }
       asm volatile("" : "+v"(alpha));  // keeps the rescale inside this rarely taken branch
-      m = mnew;
-      mc = m * cs;
       l *= alpha;
 #pragma unroll
       for (int db = 0; db < ND; ++db)
@@ -569,7 +581,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
         u.y = pack2(O[db][4 * g + 2] * inv, O[db][4 * g + 3] * inv);
         *reinterpret_cast<uint2*>(orow + db * 32 + 8 * g) = u;
       }
-    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (m * cs + __log2f(lt)) * kLn2;
+    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (mc + __log2f(lt)) * kLn2;
   }
 }
 
@@ -582,7 +594,11 @@ static int launch_flat(hipStream_t st, AttnArgs a, int B) {
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
-  hipLaunchKernelGGL((attn_fwd_bf16_flat_kernel<NW, BIAS, HD>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  // scale * log2(e) == 1 (to f32 round-off): the caller folded the factor into q; the logits need no multiply.
+  // With a key bias the logits are touched after the MFMAs anyway, so that variant keeps its FMA.
+  const bool pre = !BIAS && a.c > 1.0f - 1e-6f && a.c < 1.0f + 1e-6f;
+  if (pre) hipLaunchKernelGGL((attn_fwd_bf16_flat_kernel<NW, BIAS, HD, !BIAS>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  else hipLaunchKernelGGL((attn_fwd_bf16_flat_kernel<NW, BIAS, HD, false>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   return launch_status();
 }
 
