@@ -68,6 +68,11 @@ def test_call_flow_of_the_attention_module(dev):
     qo, ko = attention_op.hip_norm_rope_ltx2(t(q), t(k_cross), t(wq), t(wk), H, rotary_emb=emb_q, k_rotary_emb=emb_k, rope_type=mode,
                                             is_self_attention=False)
     _assert_close(to_np(ko).reshape(B, Sk, -1), O.norm_rope_ltx2(k_cross, wk, *tab_k, mode), f"{mode} cross k with its own table")
+    # q_mul (softmax scale carried by the prologue) goes into the f32 query scale: q scaled, k untouched
+    m = ops.folded_q_mul(D)
+    qo, ko = attention_op.hip_norm_rope_ltx2(t(q), t(k_self), t(wq), t(wk), H, rotary_emb=emb_q, rope_type=mode, q_mul=m)
+    _assert_close(to_np(qo).reshape(B, Sq, -1) / m, O.norm_rope_ltx2(q, wq, *tab_q, mode), f"{mode} self q with q_mul")
+    _assert_close(to_np(ko).reshape(B, Sq, -1), O.norm_rope_ltx2(k_self, wk, *tab_q, mode), f"{mode} self k with q_mul")
   with pytest.raises(ValueError, match="not supported"):
     attention_op.hip_norm_rope_ltx2(t(q), None, t(wq), t(wk), H, rope_type="rotate_half")
 
