@@ -32,9 +32,10 @@ Pinning status of each function (what fixes it besides its own formula):
                                  any reference test; it is pinned only to tolerance
                                  (2e-2) against `attention`, like the reference's
                                  own tests do (tests/attention_test.py:90-147).
-  attention_fp8_emulated         no reference counterpart (BASELINE configs[4]);
-                                 defined by this file, pinned only through
-                                 e4m3_round and cosine vs `attention`.
+  attention_fp8_emulated         PARITY UNPINNED: no reference counterpart (BASELINE
+                                 configs[4]); it restates the fp8 kernel's rounding points
+                                 and reference-point rule, and is held only to e4m3_round
+                                 and to the cosine bar against `attention`.
 """
 from __future__ import annotations
 
