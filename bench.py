@@ -113,9 +113,12 @@ def main():
     qn, kn = prologue()
     e1.record()
     if fp8:  # per-tensor absmax e4m3 quantisation of q, k, v, then the fp8 kernel
-      (q8, sq), (k8, sk), (v8, sv) = (ops.quant_e4m3(x) for x in (qn, kn, v))
+      # q's quantiser carries scale * log2(e); power-of-two q and k scales: the kernel scales the logits in its MFMAs
+      q8, sq = ops.quant_e4m3(qn, premul=ops.folded_q_mul(D, w.scale), pow2_scale=True)
+      k8, sk = ops.quant_e4m3(kn, pow2_scale=True)
+      v8, sv = ops.quant_e4m3(v)
       eq.record()
-      ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=w.scale, return_lse=True)
+      ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=ops.FOLDED_SCALE, return_lse=True)
     elif ring == 1:
       ops.flash_attention(qn, kn, v, scale=att_scale, return_lse=True)
     else:  # one ring shard: this Q chunk against `ring` successive KV chunks, merged in LSE space

@@ -149,10 +149,18 @@ int mdattn_key_mask_bias(void* stream, const void* keep, float* bias, int B, int
  * Per-tensor absmax quantisation bf16 -> OCP float8 e4m3fn (BASELINE configs[4]; no reference
  * counterpart: the reference's fp8 is qwix quantisation of dense layers, pipelines/wan/wan_pipeline.py:581-626).
  *   x_bf16 [n] contiguous, x_fp8 [n] bytes,
- *   scale_out f32[2] device: [0] = absmax/448 (x ~= x_fp8 * scale_out[0]), [1] = absmax (scratch of the reduction)
+ *   premul       constant multiplied into x before the (single) rounding to e4m3; 1.0f = none.  For q,
+ *                scale * log2(e) here and scale = ln 2 in mdattn_fwd_fp8 carry the softmax scale at no cost.
+ *   pow2_scale   non-zero: the scale is rounded up to a power of two (e4m3 is a floating-point format: no
+ *                precision is lost, at most one binade of range).  With power-of-two q and k scales and the
+ *                softmax scale carried by premul, mdattn_fwd_fp8 applies the whole logit scale through the
+ *                MFMA's block-scale operand and saves its multiply per logit.
+ *   scale_out f32[2] device: [0] = s with x * premul ~= x_fp8 * s (absmax(x * premul) / 448, or the next
+ *                power of two), [1] = absmax(x) (scratch of the reduction)
  * n % 16 == 0.
  */
-int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, float* scale_out, int64_t n);
+int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, float* scale_out, int64_t n,
+                      float premul, int pow2_scale);
 
 /*
  * fp8-e4m3 attention forward: q8/k8/v8 are e4m3 bytes [B,S,H,D] by strides, *_scale device f32[1]

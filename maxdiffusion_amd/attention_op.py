@@ -15,6 +15,8 @@ to a CPU implementation.
 """
 from __future__ import annotations
 
+import math
+
 import torch
 
 from . import ops
@@ -107,10 +109,12 @@ def hip_flash_fp8_kernel(q, k, v, context):
   _reject_unsupported(context, masks_ok=False)
   heads = context["heads"]
   qv, kv, vv = (_as_bshd(t, heads).to(torch.bfloat16).contiguous() for t in (q, k, v))
-  q8, sq = ops.quant_e4m3(qv)
-  k8, sk = ops.quant_e4m3(kv)
+  # the softmax scale rides on q's quantisation (one rounding either way) and the q and k scales are powers of two:
+  # the kernel then applies the whole logit scale inside its MFMAs
+  q8, sq = ops.quant_e4m3(qv, premul=context["scale"] * math.log2(math.e), pow2_scale=True)
+  k8, sk = ops.quant_e4m3(kv, pow2_scale=True)
   v8, sv = ops.quant_e4m3(vv)
-  out = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=context["scale"])
+  out = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=ops.FOLDED_SCALE)
   b, s, h, d = out.shape
   return out.reshape(b, s, h * d).to(q.dtype)
 

@@ -63,7 +63,7 @@ struct Fp8Args {
 
 // Register budget: three waves per SIMD (<= 168 VGPRs).  The kernel is bound by the vector ALU (softmax)
 // and by latencies a single wave cannot hide, so the third wave per SIMD is worth more than registers.
-template <int NW>
+template <int NW, bool PRE>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_fwd_fp8_kernel(Fp8Args a) {
   extern __shared__ __attribute__((aligned(16))) char smem8[];
   constexpr int NT = NW * 64;
@@ -85,6 +85,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   const int q0 = qt * BM + wave * 32;
   const int nt = (a.Skv + kBN8 - 1) / kBN8;
   const float c = a.c * a.q_scale[0] * a.k_scale[0];
+  // The scales live in device memory, so the host cannot know which of the two instances of this kernel applies:
+  // it launches both, and the one whose case this is not ends here.
+  {
+    const unsigned cbits = __float_as_uint(c);
+    const bool c_pow2 = (cbits & 0x007FFFFFu) == 0u && cbits > 0x00800000u && cbits < 0x7F000000u;
+    if (c_pow2 != PRE) return;
+  }
 
   // ---- Q fragments: lane (row l32, half hh) holds bytes 64*j + 32*hh .. +31 of its row
   i32x8 qf[2];
@@ -141,7 +148,15 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   for (int sl = 0; sl < 4; ++sl)
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[sl][i] = 0.f;
-  float ref = -1e30f, l = 0.f;  // reference point of P (log2 units), per-lane partial row sum
+  // When the whole logit scale c is a power of two (power-of-two q and k scales from the quantiser, the softmax
+  // scale already inside q), the MFMAs apply it through their block-scale operand and start every logit chain at
+  // minus the row's reference point: the logits arrive in log2 units relative to it and the softmax needs no
+  // multiply.  The reference then starts at 0 and the first tile always takes the branch that sets it.
+  const int sexp = (int)(__float_as_uint(c) >> 23);  // E8M0 code of c
+  float ref = PRE ? 0.f : -1e30f, l = 0.f;           // reference point of P (log2 units), per-lane partial row sum
+  f32x16 negref;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) negref[i] = 0.f;
 
   // lane-constant LDS offsets (bytes)
   // K fragment (d half j, 16-byte half i) of row l32 is logical chunk 4j + 2hh + i
@@ -162,30 +177,30 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
 
   auto tile = [&](int t, int slot, auto masked) __attribute__((always_inline)) {
     const char* Ks = smem8 + slot * kStage8;
-    // ---- S^T = K.Q^T for the two 32-key blocks
-    auto qk = [&](f32x16* S, const char* Kb) __attribute__((always_inline)) {
+    // ---- S^T = K.Q^T for one 32-key block
+    auto qk = [&](f32x16& S, int blk, const char* Kb) __attribute__((always_inline)) {
+      i32x8 kf[2];
 #pragma unroll
-      for (int blk = 0; blk < 2; ++blk) {
-        i32x8 kf[2];
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const u32x4 lo = *reinterpret_cast<const u32x4*>(Kb + k_off[j][0] + blk * 32 * kKS8);
-          const u32x4 hi = *reinterpret_cast<const u32x4*>(Kb + k_off[j][1] + blk * 32 * kKS8);
-          kf[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-        }
+      for (int j = 0; j < 2; ++j) {
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(Kb + k_off[j][0] + blk * 32 * kKS8);
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(Kb + k_off[j][1] + blk * 32 * kKS8);
+        kf[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+      }
+      if constexpr (PRE) {  // logits in log2 units minus the reference point, straight out of the MFMAs
+        const f32x16 z = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[0], qf[0], negref, 0, 0, 0, 127, 0, sexp);
+        S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], z, 0, 0, 0, 127, 0, sexp);
+      } else {
         f32x16 z;
 #pragma unroll
         for (int i = 0; i < 16; ++i) z[i] = 0.f;
         z = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[0], qf[0], z, 0, 0, 0, 0, 0, 0);
-        S[blk] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], z, 0, 0, 0, 0, 0, 0);
+        S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], z, 0, 0, 0, 0, 0, 0);
       }
       if constexpr (decltype(masked)::value) {
-        const int kbase = t * kBN8 + 4 * hh;
+        const int kbase = t * kBN8 + 4 * hh + 32 * blk;
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-          for (int i = 0; i < 16; ++i)
-            if (kbase + 32 * blk + 8 * (i >> 2) + (i & 3) >= a.Skv) S[blk][i] = -INFINITY;
+        for (int i = 0; i < 16; ++i)
+          if (kbase + 8 * (i >> 2) + (i & 3) >= a.Skv) S[i] = -INFINITY;
       }
     };
     // ---- P = exp2(c*S - ref), f32 row sum, e4m3 pack in B-operand order.  The hot path takes no row
@@ -193,55 +208,75 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
     // that sums beyond 2^8 (so possibly one beyond it: e4m3 ends at 448) sends the wave through the branch
     // that moves every row's reference to its true maximum - kPOff, rescales the accumulators and redoes
     // the tile's logits and P.  Right after a move a group sums to at most 4 * 2^kPOff, so a row triggers again only
-    // when its maximum has grown by two more log2 units.
+    // when its maximum has grown by two more log2 units.  The two 32-key blocks of the tile are taken one after
+    // the other, so that only 16 logits per lane are alive at a time.
     i32x8 pk;
-    float gmax;
-    auto soft = [&](const f32x16* S, float rf) __attribute__((always_inline)) {
-      float ls = 0.f;
-      gmax = 0.f;
+    float gmax, ls;
+    auto soft = [&](const f32x16& S, int blk, float rf) __attribute__((always_inline)) {
 #pragma unroll
-      for (int blk = 0; blk < 2; ++blk)
+      for (int g = 0; g < 4; ++g) {
+        float p[4];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          float p[4];
-#pragma unroll
-          for (int x = 0; x < 4; ++x) p[x] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[blk][4 * g + x], c, -rf));
-          const float s4 = (p[0] + p[1]) + (p[2] + p[3]);
-          ls += s4;
-          gmax = fmaxf(gmax, s4);
-          int u = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
-          u = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], u, true);
-          pk[4 * blk + g] = u;
-        }
-      return ls;
+        for (int x = 0; x < 4; ++x) p[x] = __builtin_amdgcn_exp2f(PRE ? S[4 * g + x] : __builtin_fmaf(S[4 * g + x], c, -rf));
+        const float s4 = (p[0] + p[1]) + (p[2] + p[3]);
+        ls += s4;
+        gmax = fmaxf(gmax, s4);
+        int u = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
+        u = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], u, true);
+        pk[4 * blk + g] = u;
+      }
     };
-    float ls;
-    {
-      f32x16 S[2];
-      qk(S, Ks);
-      ls = soft(S, ref);
+    ls = 0.f;
+    gmax = 0.f;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      f32x16 S;
+      qk(S, blk, Ks);
+      soft(S, blk, ref);
+      if (PRE) __builtin_amdgcn_sched_barrier(0);  // keeps the second block's logits from being hoisted over the first's softmax
     }
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(gmax <= kPTrig)) != 0, 0)) {
-      f32x16 S[2];  // recomputed rather than kept: the hot path then holds the logits only while it forms P
-      const char* Kb = Ks;
-      asm volatile("" : "+s"(Kb));  // an address the compiler cannot match with the hot path's: no reuse of its logits
-      qk(S, Kb);
-      float mx = S[0][0];
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(gmax <= kPTrig)) != 0 || (PRE && t == 0), 0)) {
+      // The logits are recomputed rather than kept: the hot path holds them only while it forms P.
+      int zero = 0;
+      asm volatile("" : "+s"(zero));  // an address the compiler cannot match with the hot path's: no reuse of its logits
+      float mx = -INFINITY;
 #pragma unroll
-      for (int i = 1; i < 16; ++i) mx = fmaxf(mx, S[0][i]);
+      for (int blk = 0; blk < 2; ++blk) {
+        f32x16 S;
+        qk(S, blk, Ks + zero);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, S[1][i]);
-      mx = xhalf_max(mx) * c;
-      const float nref = fmaxf(ref, mx - kPOff);
-      float alpha = __builtin_amdgcn_exp2f(ref - nref);
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, S[i]);
+      }
+      float alpha;
+      if constexpr (PRE) {  // the logits are relative to the old reference
+        mx = xhalf_max(mx);
+        const float dm = t == 0 ? mx - kPOff : fmaxf(mx - kPOff, 0.f);
+        alpha = t == 0 ? 0.f : __builtin_amdgcn_exp2f(-dm);
+        ref += dm;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) negref[i] = -ref;
+      } else {
+        mx = xhalf_max(mx) * c;
+        const float nref = fmaxf(ref, mx - kPOff);
+        alpha = __builtin_amdgcn_exp2f(ref - nref);
+        ref = nref;
+      }
       asm volatile("" : "+v"(alpha));  // keeps the rescale inside this rarely taken branch
-      ref = nref;
       l *= alpha;
 #pragma unroll
       for (int sl = 0; sl < 4; ++sl)
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[sl][i] *= alpha;
-      ls = soft(S, ref);
+      // once more against the new reference points
+      asm volatile("" : "+s"(zero));
+      ls = 0.f;
+      gmax = 0.f;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        f32x16 S;
+        qk(S, blk, Ks + zero);
+        soft(S, blk, ref);
+      }
     }
     l += ls;
     // ---- O^T += V^T.P^T
@@ -303,7 +338,8 @@ int launch_fwd8(hipStream_t st, Fp8Args a, int B) {
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
-  hipLaunchKernelGGL(attn_fwd_fp8_kernel<NW>, dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, false>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, true>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   return launch_status();
 }
 
@@ -342,6 +378,7 @@ extern "C" int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, cons
   a.v_sb = v_strides->batch; a.v_ss = v_strides->seq; a.v_sh = v_strides->head;
   a.o_sb = o_strides->batch; a.o_ss = o_strides->seq; a.o_sh = o_strides->head;
   a.c = scale * kLog2e;
+  if (a.c > 1.0f - 1e-6f && a.c < 1.0f + 1e-6f) a.c = 1.0f;  // scale = ln 2: the caller's q carries the softmax scale
   hipStream_t st = (hipStream_t)stream;
   // Four waves per workgroup (three workgroups per CU) measured faster than eight at every shape tried;
   // MDATTN_FP8_VARIANT (1: 8 waves, 2: 4 waves per workgroup) overrides the choice for experiments.

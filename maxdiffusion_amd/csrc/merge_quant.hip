@@ -83,11 +83,18 @@ __global__ __launch_bounds__(256) void absmax_kernel(const uint4* __restrict__ x
   if ((threadIdx.x & 63) == 0 && m) atomicMax(amax_bits, m);
 }
 
-__global__ __launch_bounds__(256) void quant_kernel(const uint4* __restrict__ x, uint4* __restrict__ y, int64_t n16, float* scale) {
-  float amax = scale[1];
+// x8 = e4m3(x * premul / s) with s = absmax(x * premul) / 448, or the next power of two above it (pow2): a
+// power-of-two scale costs e4m3, a floating-point format, no precision, only up to one binade of its range.
+__global__ __launch_bounds__(256) void quant_kernel(const uint4* __restrict__ x, uint4* __restrict__ y, int64_t n16, float* scale,
+                                                    float premul, int pow2) {
+  float amax = scale[1] * premul;
   amax = amax > 1e-12f ? amax : 1e-12f;
-  const float s = amax * (1.0f / 448.0f);
-  const float r = 448.0f / amax;
+  float s = amax * (1.0f / 448.0f);
+  if (pow2) {
+    const unsigned b = __float_as_uint(s);
+    s = __uint_as_float(((b & 0x007FFFFFu) ? b + 0x00800000u : b) & 0x7F800000u);
+  }
+  const float r = premul / s;
   if (blockIdx.x == 0 && threadIdx.x == 0) scale[0] = s;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (int64_t)gridDim.x * 256) {
     float f[16];
@@ -151,8 +158,10 @@ extern "C" int mdattn_finalize(void* stream, const float* o_run, void* out_bf16,
   return launch_status();
 }
 
-extern "C" int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, float* scale_out, int64_t n) {
+extern "C" int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, float* scale_out, int64_t n,
+                                 float premul, int pow2_scale) {
   if (!x_bf16 || !x_fp8 || !scale_out || n <= 0) return MDATTN_E_BADARG;
+  if (!(premul > 0.f) || !(premul < 1e30f)) return MDATTN_E_BADARG;
   if (n % 16) return MDATTN_E_UNSUPPORTED;
   if (!aligned16(x_bf16) || !aligned16(x_fp8) || (reinterpret_cast<uintptr_t>(scale_out) & 7u)) return MDATTN_E_ALIGN;
   hipStream_t st = (hipStream_t)stream;
@@ -161,7 +170,8 @@ extern "C" int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, 
   const unsigned g2 = (unsigned)((n16 + 255) / 256 < 16384 ? (n16 + 255) / 256 : 16384);
   hipLaunchKernelGGL(zero2_kernel, dim3(1), dim3(64), 0, st, scale_out);
   hipLaunchKernelGGL(absmax_kernel, dim3(g1), dim3(256), 0, st, (const uint4*)x_bf16, n8, (unsigned*)(scale_out + 1));
-  hipLaunchKernelGGL(quant_kernel, dim3(g2), dim3(256), 0, st, (const uint4*)x_bf16, (uint4*)x_fp8, n16, scale_out);
+  hipLaunchKernelGGL(quant_kernel, dim3(g2), dim3(256), 0, st, (const uint4*)x_bf16, (uint4*)x_fp8, n16, scale_out,
+                     premul, pow2_scale);
   return launch_status();
 }
 

@@ -227,14 +227,18 @@ def flash_attention_backward(q, k, v, out, dout, lse, scale: float | None = None
   return dq, dk, dv
 
 
-def quant_e4m3(x: torch.Tensor):
-  """Per-tensor absmax quantisation of a contiguous bf16 tensor -> (uint8 e4m3 bytes, f32[2] scale buffer)."""
+def quant_e4m3(x: torch.Tensor, premul: float = 1.0, pow2_scale: bool = False):
+  """Per-tensor absmax quantisation of a contiguous bf16 tensor -> (uint8 e4m3 bytes, f32[2] scale buffer).
+
+  `premul` is multiplied into x before the single rounding (x * premul ~= x8 * scale[0]); `pow2_scale` rounds the
+  scale up to a power of two.  q with premul=folded_q_mul(D) and pow2_scale=True, k with pow2_scale=True and
+  flash_attention_fp8(..., scale=FOLDED_SCALE) let the fp8 kernel apply the whole logit scale inside its MFMAs."""
   _check_dev(x)
   if x.dtype != torch.bfloat16 or not x.is_contiguous():
     raise ValueError("quant_e4m3 needs a contiguous bf16 tensor")
   x8 = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
   scale = torch.empty(2, dtype=torch.float32, device=x.device)
-  rc = _lib.load().mdattn_quant_e4m3(_stream(), _ptr(x), _ptr(x8), _ptr(scale), x.numel())
+  rc = _lib.load().mdattn_quant_e4m3(_stream(), _ptr(x), _ptr(x8), _ptr(scale), x.numel(), float(premul), int(bool(pow2_scale)))
   _lib.check(rc, "mdattn_quant_e4m3")
   return x8, scale
 

@@ -425,15 +425,20 @@ def ring_replay(q, k_chunks, v_chunks, scale: float, dtype=np.float64):
 
 
 # --------------------------------------------------------------------------- A7 fp8 variant
-def quant_e4m3(x):
-  """Per-tensor absmax quantisation: s = absmax/448, x8 = e4m3(x / s).  Returns (x8 as f32, s)."""
+def quant_e4m3(x, premul: float = 1.0, pow2_scale: bool = False):
+  """Per-tensor absmax quantisation of x * premul: s = absmax/448 (or the next power of two above it),
+  x8 = e4m3(x * premul / s).  Returns (x8 as f32, s)."""
   x = np.asarray(x, np.float32)
-  s = np.float32(max(float(np.abs(x).max()), 1e-12) / E4M3_MAX)
-  return e4m3_round(x / s), s
+  amax = np.float32(max(float(np.float32(np.abs(x).max()) * np.float32(premul)), 1e-12))
+  s = np.float32(amax * np.float32(1.0 / E4M3_MAX))
+  if pow2_scale:  # the next power of two at or above s
+    m, e = np.frexp(s)
+    s = np.float32(np.ldexp(1.0, int(e) - 1 if m == 0.5 else int(e)))
+  return e4m3_round(x * (np.float32(premul) / s)), s
 
 
 def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: float = 4.0, p_trig: float = 256.0,
-                           rows_per_wave: int = 32):
+                           rows_per_wave: int = 32, pow2_scales: bool = False):
   """Emulation of the fp8 kernel's arithmetic (no reference counterpart).
 
   Q, K, V quantised per tensor; logits from the quantised operands in f32; online softmax per
@@ -444,17 +449,23 @@ def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: f
   every row of that wave takes ref = max(ref, tile max - p_offset).  P then stays within
   [0, p_trig], inside e4m3's range, and probabilities down to 2^-(6+p_offset) of the row max
   stay in e4m3's normal range.  The result does not depend on `ref` except through the e4m3
-  rounding.  q [H,Sq,D], k/v [H,Skv,D].
+  rounding.  q [H,Sq,D], k/v [H,Skv,D].  pow2_scales: q is quantised with scale * log2(e) folded in and with a
+  power-of-two scale, k with a power-of-two scale (the operands of the kernel's path without a multiply per logit).
   """
-  q8, sq = quant_e4m3(q)
-  k8, sk = quant_e4m3(k)
+  log2e = np.float32(np.log2(np.e))
+  if pow2_scales:
+    q8, sq = quant_e4m3(q, premul=np.float32(scale) * log2e, pow2_scale=True)
+    k8, sk = quant_e4m3(k, pow2_scale=True)
+  else:
+    q8, sq = quant_e4m3(q)
+    k8, sk = quant_e4m3(k)
   v8, sv = quant_e4m3(v)
   H, Sq, D = q8.shape
   Skv = k8.shape[1]
   ref = np.full((H, Sq), -1e30, np.float32)
   l = np.zeros((H, Sq), np.float32)
   o = np.zeros((H, Sq, D), np.float32)
-  c = np.float32(np.float32(scale) * np.float32(np.log2(np.e)) * sq * sk)
+  c = np.float32(sq * sk) if pow2_scales else np.float32(np.float32(scale) * log2e * sq * sk)
   nw = -(-Sq // rows_per_wave)
   for t0 in range(0, Skv, kv_tile):
     s = np.einsum("hqd,hkd->hqk", q8, k8[:, t0:t0 + kv_tile])

@@ -94,7 +94,8 @@ def test_bad_arguments_are_rejected_on_the_host(lib):
 
   assert lib.mdattn_finalize(None, fake, fake, 12) == _lib.E_UNSUPPORTED
   assert lib.mdattn_finalize(None, fake, None, 16) == _lib.E_BADARG
-  assert lib.mdattn_quant_e4m3(None, fake, fake, fake, 24) == _lib.E_UNSUPPORTED
-  assert lib.mdattn_quant_e4m3(None, fake, fake, None, 32) == _lib.E_BADARG
+  assert lib.mdattn_quant_e4m3(None, fake, fake, fake, 24, 1.0, 0) == _lib.E_UNSUPPORTED
+  assert lib.mdattn_quant_e4m3(None, fake, fake, None, 32, 1.0, 0) == _lib.E_BADARG
+  assert lib.mdattn_quant_e4m3(None, fake, fake, fake, 32, 0.0, 1) == _lib.E_BADARG
   with pytest.raises(_lib.MdattnError, match="mdattn error -1"):
     _lib.check(_lib.E_BADARG, "unit test")

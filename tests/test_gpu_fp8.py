@@ -17,10 +17,17 @@ pytestmark = pytest.mark.gpu
 COS_BAR = 0.995
 
 
-def _quant_run(q, k, v, dev, scale=None, **kw):
+def _quant_run(q, k, v, dev, scale=None, pow2=False, **kw):
+  """pow2: q quantised with scale * log2(e) folded in and a power-of-two scale, k with a power-of-two scale, the
+  kernel given scale = ln 2 -- the operands of its path that scales the logits inside the MFMAs."""
   qd, kd, vd = (to_dev_bf16(x, dev) for x in (q, k, v))
-  q8, sq = ops.quant_e4m3(qd)
-  k8, sk = ops.quant_e4m3(kd)
+  if pow2:
+    q8, sq = ops.quant_e4m3(qd, premul=ops.folded_q_mul(q.shape[-1], scale), pow2_scale=True)
+    k8, sk = ops.quant_e4m3(kd, pow2_scale=True)
+    scale = ops.FOLDED_SCALE
+  else:
+    q8, sq = ops.quant_e4m3(qd)
+    k8, sk = ops.quant_e4m3(kd)
   v8, sv = ops.quant_e4m3(vd)
   out, lse = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=scale, return_lse=True, **kw)
   return to_np(out), to_np(lse)
@@ -28,16 +35,17 @@ def _quant_run(q, k, v, dev, scale=None, **kw):
 
 @pytest.mark.parametrize("sq,skv,mult", [(1, 1, 1.0), (31, 65, 1.0), (257, 63, 1.0), (300, 333, 1.0), (1000, 77, 1.0),
                                          (64, 4097, 1.0), (513, 512, 1.0), (500, 700, 6.0)])
-def test_fp8_against_emulation_and_bf16_oracle(dev, sq, skv, mult):
+@pytest.mark.parametrize("pow2", [False, True])
+def test_fp8_against_emulation_and_bf16_oracle(dev, sq, skv, mult, pow2):
   H = 3
   q = O.bf16_round(O.normal_bf16((1, sq, H, 128), 0) * np.float32(mult))
   k, v = O.normal_bf16((1, skv, H, 128), 1), O.normal_bf16((1, skv, H, 128), 2)
-  out, lse = _quant_run(q, k, v, dev)
+  out, lse = _quant_run(q, k, v, dev, pow2=pow2)
   exact, lse_exact = O.attention(hsd(q), hsd(k), hsd(v), 128**-0.5)
-  emu, lse_emu = O.attention_fp8_emulated(hsd(q), hsd(k), hsd(v), 128**-0.5)
+  emu, lse_emu = O.attention_fp8_emulated(hsd(q), hsd(k), hsd(v), 128**-0.5, pow2_scales=pow2)
   cos_exact, cos_emu = cosine(hsd(out), exact), cosine(hsd(out), emu)
   lmx = float(np.abs(lse[0] - lse_emu).max())
-  print(f"fp8 Sq={sq} Skv={skv} x{mult}: cos vs f32 oracle {cos_exact:.5f}, vs emulation {cos_emu:.6f}, "
+  print(f"fp8 Sq={sq} Skv={skv} x{mult} pow2={pow2}: cos vs f32 oracle {cos_exact:.5f}, vs emulation {cos_emu:.6f}, "
         f"rel-l2 vs emulation {rel_l2(hsd(out), emu):.3e}, lse vs emulation {lmx:.2e}, vs exact "
         f"{float(np.abs(lse[0] - lse_exact).max()):.2e}", flush=True)
   # the north-star bar is stated for N(0,1) inputs; logits six times sharper amplify the e4m3 noise of
@@ -51,8 +59,9 @@ def test_fp8_against_emulation_and_bf16_oracle(dev, sq, skv, mult):
   assert np.abs(lse[0] - lse_exact).max() <= (0.25 if mult == 1.0 else 1.5)
 
 
+@pytest.mark.parametrize("pow2", [False, True])
 @pytest.mark.parametrize("profile", ["ascending", "descending", "plateau", "late_spike"])
-def test_fp8_reference_point_moves(dev, profile):
+def test_fp8_reference_point_moves(dev, profile, pow2):
   """Logit profiles that make the rows' reference points move often, never, through sums without a single
   large term, and through one exponent far beyond e4m3's range: the kernel has to follow the emulation,
   which applies the same rule (a group of four probabilities above 2^8 moves the wave's rows)."""
@@ -61,11 +70,11 @@ def test_fp8_reference_point_moves(dev, profile):
   qs, ks = zip(*(_structured_logits(sq, skv, 128, profile, seed=5 + h) for h in range(H)))
   q, k = np.stack(qs, 1)[None], np.stack(ks, 1)[None]
   v = O.normal_bf16((1, skv, H, 128), 2)
-  out, lse = _quant_run(q, k, v, dev)
-  emu, lse_emu = O.attention_fp8_emulated(hsd(q), hsd(k), hsd(v), 128**-0.5)
+  out, lse = _quant_run(q, k, v, dev, pow2=pow2)
+  emu, lse_emu = O.attention_fp8_emulated(hsd(q), hsd(k), hsd(v), 128**-0.5, pow2_scales=pow2)
   exact, _ = O.attention(hsd(q), hsd(k), hsd(v), 128**-0.5)
   r, lmx = rel_l2(hsd(out), emu), float(np.abs(lse[0] - lse_emu).max())
-  print(f"fp8 {profile}: rel-l2 vs emulation {r:.3e}, lse vs emulation {lmx:.2e}, cos vs f32 oracle {cosine(hsd(out), exact):.5f} "
+  print(f"fp8 {profile} pow2={pow2}: rel-l2 vs emulation {r:.3e}, lse vs emulation {lmx:.2e}, cos vs f32 oracle {cosine(hsd(out), exact):.5f} "
         f"(emulation {cosine(emu, exact):.5f})", flush=True)
   assert np.isfinite(out).all() and np.isfinite(lse).all()
   # a row whose group sum sits at the threshold may move in one and not in the other: P is then rounded on a
@@ -94,7 +103,12 @@ def test_fp8_layouts_batch_scale_and_dispatcher(dev):
   q3, k3, v3 = (to_dev_bf16(x, dev).reshape(B, S, H * 128) for x in (q, k, v))
   got = op.apply_attention(q3, k3, v3)
   assert got.shape == (B, S, H * 128) and got.dtype == torch.bfloat16
-  np.testing.assert_array_equal(to_np(got).reshape(B, S, H, 128), base)
+  # the registry entry quantises q with the softmax scale folded in and power-of-two scales
+  base2, _ = _quant_run(q, k, v, dev, scale=0.05, pow2=True)
+  np.testing.assert_array_equal(to_np(got).reshape(B, S, H, 128), base2)
+  for b in range(B):
+    exact, _ = O.attention(hsd(q[b:b + 1]), hsd(k[b:b + 1]), hsd(v[b:b + 1]), 0.05)
+    assert cosine(hsd(base2[b:b + 1]), exact) >= COS_BAR
 
 
 def test_fp8_wan14b_full_size_sampled_rows_and_whole_tensor(dev):
@@ -104,10 +118,11 @@ def test_fp8_wan14b_full_size_sampled_rows_and_whole_tensor(dev):
   H, S = w.heads, w.seq
   gen = torch.Generator(device=dev).manual_seed(4)
   q, k, v = (torch.randn((1, S, H, 128), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
-  q8, sq = ops.quant_e4m3(q)
-  k8, sk = ops.quant_e4m3(k)
+  # the operands bench.py uses: q's quantiser carries scale * log2(e), q and k scales are powers of two
+  q8, sq = ops.quant_e4m3(q, premul=ops.folded_q_mul(128, w.scale), pow2_scale=True)
+  k8, sk = ops.quant_e4m3(k, pow2_scale=True)
   v8, sv = ops.quant_e4m3(v)
-  out, lse = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=w.scale, return_lse=True)
+  out, lse = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=ops.FOLDED_SCALE, return_lse=True)
   ref, ref_lse = ops.flash_attention(q, k, v, scale=w.scale, return_lse=True)
   torch.cuda.synchronize()
   of, rf = out.float(), ref.float()
