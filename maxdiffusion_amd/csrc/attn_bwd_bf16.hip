@@ -10,7 +10,8 @@
 // Per tile, with the forward kernel's layouts and fragment reads:
 //   S^T  = stream1 . entity1^T      (A = tile rows by ds_read_b128, B = entity fragments)   lane = entity row
 //   dP^T = stream2 . entity2^T      (not for dv)
-//   W    = exp2(c*S - lse*log2e) [* (dP - delta) * scale]     f32, packed to bf16 in B-operand order
+//   W    = exp2(c*S - lse*log2e) [* (dP - delta)]     f32, packed to bf16 in B-operand order (the factor `scale` of
+//                                                      dS is applied once, to the finished accumulators)
 //   acc^T += stream3^T . W          (A = the tile through the transposing LDS read)
 // lse and delta belong to the q rows: per-lane scalars for dq, sixteen values per lane and tile for dk / dv, read
 // from a workspace that a small kernel fills first (delta, lse in log2 units, both padded to a multiple of 32 rows
@@ -188,7 +189,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
       for (int e = 0; e < 8; ++e) {
         const int i = 8 * hb + e;
         const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(S[i], c, -ls[i]));
-        wv[e] = HAS2 ? p * (dP[i] - dl[i]) * a.scale : p;
+        wv[e] = HAS2 ? p * (dP[i] - dl[i]) : p;  // dS without its factor `scale`: applied once, to the accumulators
       }
       W[hb] = __builtin_bit_cast(bf16x8, pack8(wv));
     }
@@ -201,6 +202,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
   }
 
   const int row = r0 + l32;
+  const float osc = HAS2 ? a.scale : 1.0f;  // dq = scale * dS k, dk = scale * dS^T q
   if (row < a.Se) {
     __bf16* orow = a.out + b * a.o_sb + h * a.o_sh + (int64_t)row * a.o_ss + 4 * hh;
 #pragma unroll
@@ -208,8 +210,8 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         uint2 u;
-        u.x = pack2(acc[db][4 * g], acc[db][4 * g + 1]);
-        u.y = pack2(acc[db][4 * g + 2], acc[db][4 * g + 3]);
+        u.x = pack2(acc[db][4 * g] * osc, acc[db][4 * g + 1] * osc);
+        u.y = pack2(acc[db][4 * g + 2] * osc, acc[db][4 * g + 3] * osc);
         *reinterpret_cast<uint2*>(orow + db * 32 + 8 * g) = u;
       }
   }
