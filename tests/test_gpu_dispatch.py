@@ -79,3 +79,22 @@ def test_fused_prologue_feeds_attention_without_transposes(dev):
   qc, none = A.hip_norm_rope(to_dev_bf16(q, dev), None, to_dev_bf16(wq, dev), None, None, H)  # cross-attention: norm only
   assert none is None
   assert err_stats(to_np(qc), O.norm_rope_fullrow(q, wq, None, None, H))[0] <= 1.6e-2
+
+
+def test_reference_splash_test_shape_head_dim_64(dev):
+  """tests/attention_test.py:90-147 of the reference: B=8, S=4096, H=10, D=64, N(0,1) inputs, criterion
+  ||dot_product - flash||_2 < 1.0 over the whole tensor.  Here: hip_flash through the registry against an f32
+  attention computed by torch on the GPU (test harness only), and the same criterion."""
+  from helpers import torch_attention_f32
+  B, S, H, D = 8, 4096, 10, 64
+  gen = torch.Generator(device=dev).manual_seed(7)
+  q, k, v = (torch.randn((B, S, H * D), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
+  op = A.AttentionOp(mesh=None, attention_kernel="hip_flash", scale=D**-0.5, heads=H, dim_head=D, dtype=torch.bfloat16)
+  got = op.apply_attention(q, k, v)
+  assert got.shape == (B, S, H * D) and got.dtype == torch.bfloat16
+  ref, _ = torch_attention_f32(q.view(B, S, H, D), k.view(B, S, H, D), v.view(B, S, H, D), D**-0.5)
+  diff = got.float().view(B, S, H, D) - ref
+  diff_norm, mx = float(diff.norm()), float(diff.abs().max())
+  print(f"B=8 S=4096 H=10 D=64: ||hip_flash - f32 attention||_2 = {diff_norm:.3f}, max-abs {mx:.2e}", flush=True)
+  assert diff_norm < 1.0 and mx <= 2e-2
+  assert float(diff.norm() / ref.norm()) <= 1.5e-2
