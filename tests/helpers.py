@@ -72,3 +72,24 @@ def torch_attention_f32(q, k, v, scale, q_block=2048):
     out[:, s0:s0 + q_block] = torch.matmul(p, vf).permute(0, 2, 1, 3)
     lse[:, :, s0:s0 + q_block] = l
   return out, lse
+
+
+def structured_logits(sq, skv, d, profile, seed=5):
+  """q, k such that the logit of (row, key j) is gain[row] * beta[j] * 4 (natural units) plus small noise:
+  the shape of beta along the key axis decides when and how often a row's reference point has to move."""
+  import oracle as O
+
+  rng = np.random.default_rng(seed)
+  u = np.ones(d, np.float32)
+  t = np.arange(skv, dtype=np.float32) / max(skv - 1, 1)
+  beta = {
+      "ascending": 2 * t - 1,                                   # the maximum grows with every tile
+      "descending": 1 - 2 * t,                                  # the first key is the maximum
+      "plateau": np.where(t < 0.5, 0.0, 0.3).astype(np.float32),  # many keys a little above the reference
+      "late_spike": np.where(np.arange(skv) == (skv * 3) // 4, 3.0, -0.2 * t).astype(np.float32),
+  }[profile]
+  gain = np.array([0.25, 0.5, 1.0, 2.0, 4.0, 8.0], np.float32)[np.arange(sq) % 6]
+  amp = np.float32(4.0 / (d * d**-0.5))                         # scale * <u, u> * amp == 4
+  q = O.bf16_round(gain[:, None] * u[None] * amp + 0.05 * rng.standard_normal((sq, d)).astype(np.float32))
+  k = O.bf16_round(beta[:, None] * u[None] + 0.05 * rng.standard_normal((skv, d)).astype(np.float32))
+  return q, k

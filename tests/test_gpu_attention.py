@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import oracle as O
-from helpers import bits_to_dev, bits_to_f32, err_stats, golden, hsd, rel_l2, to_dev_bf16, to_np, torch_attention_f32
+from helpers import bits_to_dev, bits_to_f32, err_stats, golden, hsd, rel_l2, structured_logits, to_dev_bf16, to_np, torch_attention_f32
 from maxdiffusion_amd import ops
 
 pytestmark = pytest.mark.gpu
@@ -122,25 +122,6 @@ def test_invariants_on_device(dev):
   assert err_stats(to_np(out[0, 45, 0]), v[0, 123, 0])[0] < 2e-2
 
 
-def _structured_logits(sq, skv, d, profile, seed=5):
-  """q, k such that the logit of (row, key j) is gain[row] * beta[j] * 4 (natural units) plus small noise:
-  the shape of beta along the key axis decides when and how often a row's reference point has to move."""
-  rng = np.random.default_rng(seed)
-  u = np.ones(d, np.float32)
-  t = np.arange(skv, dtype=np.float32) / max(skv - 1, 1)
-  beta = {
-      "ascending": 2 * t - 1,                                   # the maximum grows with every tile
-      "descending": 1 - 2 * t,                                  # the first key is the maximum
-      "plateau": np.where(t < 0.5, 0.0, 0.3).astype(np.float32),  # many keys a little above the reference
-      "late_spike": np.where(np.arange(skv) == (skv * 3) // 4, 3.0, -0.2 * t).astype(np.float32),
-  }[profile]
-  gain = np.array([0.25, 0.5, 1.0, 2.0, 4.0, 8.0], np.float32)[np.arange(sq) % 6]
-  amp = np.float32(4.0 / (d * d**-0.5))                         # scale * <u, u> * amp == 4
-  q = O.bf16_round(gain[:, None] * u[None] * amp + 0.05 * rng.standard_normal((sq, d)).astype(np.float32))
-  k = O.bf16_round(beta[:, None] * u[None] + 0.05 * rng.standard_normal((skv, d)).astype(np.float32))
-  return q, k
-
-
 @pytest.mark.parametrize("var", [1, 2, 3])
 @pytest.mark.parametrize("profile", ["ascending", "descending", "plateau", "late_spike"])
 def test_reference_point_moves(dev, variant, var, profile):
@@ -150,7 +131,7 @@ def test_reference_point_moves(dev, variant, var, profile):
   e^96 above the rest) must all come out like the oracle's exact softmax."""
   variant(var)
   H, sq, skv = 2, 150, 1500
-  qs, ks = zip(*(_structured_logits(sq, skv, 128, profile, seed=5 + h) for h in range(H)))
+  qs, ks = zip(*(structured_logits(sq, skv, 128, profile, seed=5 + h) for h in range(H)))
   q = np.stack(qs, 1)[None]
   k = np.stack(ks, 1)[None]
   v = O.normal_bf16((1, skv, H, 128), 2)
@@ -281,14 +262,14 @@ def test_head_dim_64_masked_and_sharp(dev):
 @pytest.mark.parametrize("profile", ["ascending", "plateau", "late_spike"])
 def test_reference_point_moves_head_dim_64_and_masked(dev, profile):
   H, D, sq, skv = 2, 64, 150, 1500
-  qs, ks = zip(*(_structured_logits(sq, skv, D, profile, seed=9 + h) for h in range(H)))
+  qs, ks = zip(*(structured_logits(sq, skv, D, profile, seed=9 + h) for h in range(H)))
   q, k = np.stack(qs, 1)[None], np.stack(ks, 1)[None]
   v = O.normal_bf16((1, skv, H, D), 2)
   out, lse = _run_np(q, k, v, dev)
   ro, rl = O.attention(hsd(q), hsd(k), hsd(v), D**-0.5)
   _check(hsd(out), lse[0], ro, rl, f"D=64 {profile}", lse_abs=2e-3 if profile == "late_spike" else LSE_ABS)
   # the masked kernel (additive key bias) at head dim 128, a mask that drops every third key
-  qs, ks = zip(*(_structured_logits(sq, skv, 128, profile, seed=9 + h) for h in range(H)))
+  qs, ks = zip(*(structured_logits(sq, skv, 128, profile, seed=9 + h) for h in range(H)))
   q, k = np.stack(qs, 1)[None], np.stack(ks, 1)[None]
   v = O.normal_bf16((1, skv, H, 128), 2)
   keep = (np.arange(skv) % 3 != 1)[None]
@@ -330,7 +311,7 @@ def test_folded_scale_reference_point_moves(dev, variant, profile):
     k[0, :, :, 0] += (np.arange(skv, dtype=np.float32) * 0.01)[:, None]
     k = O.bf16_round(k)
   else:
-    qs, ks = zip(*(_structured_logits(sq, skv, 128, profile, seed=5 + h) for h in range(H)))
+    qs, ks = zip(*(structured_logits(sq, skv, 128, profile, seed=5 + h) for h in range(H)))
     q, k = np.stack(qs, 1)[None], np.stack(ks, 1)[None]
   v = O.normal_bf16((1, skv, H, 128), 2)
   out, lse, ro, rl = _folded_run(q, k, v, dev)

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import oracle as O
-from helpers import cosine, err_stats, hsd, rel_l2, to_dev_bf16, to_np
+from helpers import cosine, err_stats, hsd, rel_l2, structured_logits, to_dev_bf16, to_np
 from maxdiffusion_amd import attention_op, ops
 
 pytestmark = pytest.mark.gpu
@@ -65,9 +65,8 @@ def test_fp8_reference_point_moves(dev, profile, pow2):
   """Logit profiles that make the rows' reference points move often, never, through sums without a single
   large term, and through one exponent far beyond e4m3's range: the kernel has to follow the emulation,
   which applies the same rule (a group of four probabilities above 2^8 moves the wave's rows)."""
-  from test_gpu_attention import _structured_logits
   H, sq, skv = 2, 150, 1500
-  qs, ks = zip(*(_structured_logits(sq, skv, 128, profile, seed=5 + h) for h in range(H)))
+  qs, ks = zip(*(structured_logits(sq, skv, 128, profile, seed=5 + h) for h in range(H)))
   q, k = np.stack(qs, 1)[None], np.stack(ks, 1)[None]
   v = O.normal_bf16((1, skv, H, 128), 2)
   out, lse = _quant_run(q, k, v, dev, pow2=pow2)
