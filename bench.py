@@ -60,6 +60,9 @@ def main():
   ap.add_argument("--traffic-probe", action="store_true",
                   help="also launch one 1 GiB device copy: the plain copy kernel of known size that scales rocprofv3's "
                        "FETCH_SIZE / WRITE_SIZE counters")
+  ap.add_argument("--with-backward", action="store_true",
+                  help="also time the backward pass (dq, dk, dv) of the workload's attention, outside the timed steps; "
+                       "reported as a `backward` object beside the headline")
   args = ap.parse_args()
   if args.gpus != 1:
     print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -181,6 +184,27 @@ def main():
     cross = {"Skv": w.cross_kv, "kernel_ms": cms, "TFLOP/s": cfl / (cms * 1e-3) / 1e12,
              "GB/s": (2 * S * H * D * 2 + 2 * w.cross_kv * H * D * 2 + H * S * 4) / (cms * 1e-3) / 1e9}
 
+  # backward of one attention call of the workload (one KV chunk for the ring shards), with the plain softmax scale
+  backward = None
+  if args.with_backward and not fp8:
+    qb, kb = ops.norm_rope_fullrow(q_in, k_in, wq, wk, cos, sin, H) if w.norm == "fullrow" else ops.norm_rope_perhead(q4, k4, wq, wk, cos, sin)
+    vb = v[:, :Skv]
+    ob, lb = ops.flash_attention(qb, kb, vb, scale=w.scale, return_lse=True)
+    dout = randn(1, S, H, D)
+    for _ in range(2):
+      ops.flash_attention_backward(qb, kb, vb, ob, dout, lb, scale=w.scale)
+    e0, e1 = ev(), ev()
+    e0.record()
+    for _ in range(5):
+      ops.flash_attention_backward(qb, kb, vb, ob, dout, lb, scale=w.scale)
+    e1.record()
+    torch.cuda.synchronize()
+    bms = e0.elapsed_time(e1) / 5
+    # the five matrix products of the backward pass: S, dP, dV, dK, dQ (the three passes execute eight)
+    bfl = 2.5 * O.attention_flops(1, H, S, Skv, D)
+    backward = {"Sq": S, "Skv": Skv, "ms": bms, "TFLOP/s": bfl / (bms * 1e-3) / 1e12,
+                "flop_counted": bfl, "note": "5 matrix products counted, 8 executed (three atomic-free passes)"}
+
   flops = O.attention_flops(1, H, S, Skv * ring, D)
   att_ms = sum(t_att) / len(t_att)
   nr_bytes = O.normrope_bytes(1, S, H, D, with_table=True)
@@ -221,6 +245,8 @@ def main():
     out["quant_ms"] = sum(t_quant) / len(t_quant)
   if cross:
     out["cross_attention"] = cross
+  if backward:
+    out["backward"] = backward
   if args.cpu_rows > 0:
     out["cpu_baseline"] = cpu_baseline(w, args.cpu_rows)
   print(json.dumps(out), flush=True)
