@@ -101,6 +101,13 @@ def main():
     # a ring shard owns the first S tokens of the full latent grid
     cos, sin = (torch.from_numpy(t[:S].copy()).to(dev) for t in O.wan_rope_table(w.grid, D))
     prologue = lambda: ops.norm_rope_fullrow(q_in, k_in, wq, wk, cos, sin, H, q_mul=q_mul)
+  elif w.norm == "rows":  # LTX-2: f32 weights, cos / sin of the size of the tensor (interleaved form), one call per tensor
+    wq, wk = (torch.from_numpy(O.norm_weight(H * D, s_)).to(dev) for s_ in (3, 4))
+    ang = torch.rand((1, S, H * D), generator=gen, device=dev, dtype=torch.float32) * 6.2831853
+    cos, sin = torch.cos(ang), torch.sin(ang)
+    del ang
+    prologue = lambda: (ops.norm_rope_rows(q_in, wq * q_mul, cos, sin, heads=H, mode="interleaved"),
+                        ops.norm_rope_rows(k_in, wk, cos, sin, heads=H, mode="interleaved"))
   else:
     wq, wk = tb(O.norm_weight(D, 3)), tb(O.norm_weight(D, 4))
     cos, sin = (torch.from_numpy(t).to(dev) for t in O.flux_rope_table(O.flux_ids(*w.grid)))
@@ -187,7 +194,14 @@ def main():
   # backward of one attention call of the workload (one KV chunk for the ring shards), with the plain softmax scale
   backward = None
   if args.with_backward and not fp8:
-    qb, kb = ops.norm_rope_fullrow(q_in, k_in, wq, wk, cos, sin, H) if w.norm == "fullrow" else ops.norm_rope_perhead(q4, k4, wq, wk, cos, sin)
+    if D != 128:
+      raise SystemExit("--with-backward: the backward kernels are built for head dim 128")
+    if w.norm == "fullrow":
+      qb, kb = ops.norm_rope_fullrow(q_in, k_in, wq, wk, cos, sin, H)
+    elif w.norm == "rows":
+      qb, kb = ops.norm_rope_rows(q_in, wq, cos, sin, heads=H, mode="interleaved"), ops.norm_rope_rows(k_in, wk, cos, sin, heads=H, mode="interleaved")
+    else:
+      qb, kb = ops.norm_rope_perhead(q4, k4, wq, wk, cos, sin)
     vb = v[:, :Skv]
     ob, lb = ops.flash_attention(qb, kb, vb, scale=w.scale, return_lse=True)
     dout = randn(1, S, H, D)
@@ -207,7 +221,7 @@ def main():
 
   flops = O.attention_flops(1, H, S, Skv * ring, D)
   att_ms = sum(t_att) / len(t_att)
-  nr_bytes = O.normrope_bytes(1, S, H, D, with_table=True)
+  nr_bytes = O.normrope_bytes(1, S, H, D, with_table=True, per_element_table=w.norm == "rows")
   achieved = flops / (att_ms * 1e-3) / 1e12
   traffic = {}
   tpath = os.path.join(ROOT, "profiles", "traffic.json")
@@ -238,7 +252,8 @@ def main():
                    "kernel_ms": att_ms, "flop_per_launch": flops / ring},
       "roofline_norm_rope": {"bound": "hbm", "achieved": nr_bytes / (pro_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                              "frac": nr_bytes / (pro_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "traffic": traffic.get(f"norm_rope_{w.norm}_kernel"),
-                             "kernel": f"norm_rope_{w.norm}_kernel", "kernel_ms": pro_ms, "bytes_per_launch": nr_bytes,
+                             "kernel": f"norm_rope_{w.norm}_kernel" + (" (two launches: q, k)" if w.norm == "rows" else ""),
+                             "kernel_ms": pro_ms, "bytes_per_launch": nr_bytes,
                              "in_step_ms": sum(t_pro) / len(t_pro)},
   }
   if fp8:

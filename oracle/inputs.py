@@ -24,8 +24,8 @@ class Workload:
   head_dim: int
   seq: int  # query tokens
   kv_seq: int  # key/value tokens of the self-attention
-  norm: str  # "fullrow" (Wan) | "perhead" (Flux)
-  rope: str  # "wan" | "flux"
+  norm: str  # "fullrow" (Wan) | "perhead" (Flux) | "rows" (LTX-2)
+  rope: str  # "wan" | "flux" | "ltx2"
   grid: tuple  # wan: (ppf, pph, ppw); flux: (n_txt, rows, cols)
   cross_kv: int = 0  # text tokens of the cross-attention that follows (0: none)
   ring_chunks: int = 0  # >0: Q chunk of `seq` tokens against this many KV chunks of `kv_seq`
@@ -47,6 +47,10 @@ WORKLOADS = {
     # tokens against 4 KV chunks of 18,900
     "wan14b-ulysses": Workload("wan14b-ulysses", 5, 128, 75600, 75600, "fullrow", "wan", (21, 45, 80)),
     "wan14b-usp": Workload("wan14b-usp", 20, 128, 18900, 18900, "fullrow", "wan", (21, 45, 80), ring_chunks=4),
+    # LTX-2 shapes (models/ltx2/transformer_ltx2.py:788-789): 32 heads, head dim 128 for the video stream and 64 for
+    # the audio stream; full-row RMSNorm with f32 weights, interleaved RoPE with per-batch, per-head f32 tables
+    "ltx2-video": Workload("ltx2-video", 32, 128, 13376, 13376, "rows", "ltx2", ()),
+    "ltx2-audio": Workload("ltx2-audio", 32, 64, 13376, 13376, "rows", "ltx2", ()),
 }
 
 
@@ -66,8 +70,11 @@ def attention_flops(batch: int, heads: int, sq: int, skv: int, d: int) -> float:
   return 4.0 * batch * heads * sq * skv * d
 
 
-def normrope_bytes(batch: int, seq: int, heads: int, d: int, with_table: bool = True) -> float:
-  """Q and K each read once and written once in bf16, + weights, + the f32 cos/sin table."""
+def normrope_bytes(batch: int, seq: int, heads: int, d: int, with_table: bool = True, per_element_table: bool = False) -> float:
+  """Q and K each read once and written once in bf16, + weights, + the f32 cos/sin table ([S, D/2] shared by the
+  heads, or, per_element_table, LTX-2's interleaved form: cos and sin of the size of the tensor, for q and for k)."""
+  if per_element_table:
+    return (8.0 + 16.0) * batch * seq * heads * d + 2 * heads * d * 4
   b = 8.0 * batch * seq * heads * d + 2 * heads * d * 2
   if with_table:
     b += seq * (d // 2) * 8
