@@ -56,6 +56,15 @@ def test_masked_attention_against_oracle(dev, sq, skv, kind):
     lmx = float(np.abs(lse[b] - rl).max())
     print(f"mask {kind} Sq={sq} Skv={skv} batch {b}: out max-abs {mx:.3e} mean-abs {mean:.3e} rel-l2 {rel_l2(hsd(out[b:b+1]), ro):.3e} lse {lmx:.3e}", flush=True)
     assert mx <= MAX_ABS and mean <= MEAN_ABS and rel_l2(hsd(out[b:b + 1]), ro) <= REL_L2 and lmx <= LSE_ABS
+  # the same mask with the softmax scale carried by q (scale = ln 2 for the kernel): the masked kernel keeps its
+  # multiply, the result is the one of the plain call on these inputs
+  qf = O.bf16_round((q * np.float32(ops.folded_q_mul(128))).astype(np.float32))
+  out2, lse2 = ops.flash_attention(to_dev_bf16(qf, dev), to_dev_bf16(k, dev), to_dev_bf16(v, dev), scale=ops.FOLDED_SCALE,
+                                   return_lse=True, key_bias=bias)
+  for b in range(B):
+    ro, rl = O.attention(hsd(qf[b:b + 1]), hsd(k[b:b + 1]), hsd(v[b:b + 1]), ops.FOLDED_SCALE, kv_mask=keep[b])
+    mx, mean = err_stats(hsd(to_np(out2)[b:b + 1]), ro)
+    assert mx <= MAX_ABS and mean <= MEAN_ABS and float(np.abs(to_np(lse2)[b] - rl).max()) <= LSE_ABS
 
 
 def test_all_keys_masked_rows_return_zero_and_all_kept_equals_unmasked(dev):
