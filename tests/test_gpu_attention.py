@@ -34,7 +34,10 @@ def variant():
   old = os.environ.get("MDATTN_FWD_VARIANT")
 
   def force(v):
-    os.environ["MDATTN_FWD_VARIANT"] = str(v)
+    if v:
+      os.environ["MDATTN_FWD_VARIANT"] = str(v)
+    else:
+      os.environ.pop("MDATTN_FWD_VARIANT", None)
 
   yield force
   if old is None:
@@ -342,3 +345,42 @@ def test_folded_scale_equals_plain_scale_through_the_prologue(dev):
   out0, lse0 = ops.flash_attention(q0, k0, vd.view(1, S, H, D), scale=w.scale, return_lse=True)
   _check(hsd(to_np(out0)), to_np(lse0)[0], ro, rl, "plain prologue -> attention", lse_abs=3e-3)
   assert float((out.float() - out0.float()).abs().max()) <= 4e-3 and float((lse - lse0).abs().max()) <= 3e-3
+
+
+def test_seeded_sweep_of_shapes_layouts_and_paths(dev, variant):
+  """Sixty seeded draws of (batch, heads, Sq, Skv, head dim, layout, logit sharpness, path: plain / folded scale /
+  key mask / forced schedule) against an f32 attention computed by torch on the GPU (test harness only)."""
+  import random
+  rnd = random.Random(11)
+  gen = torch.Generator(device=dev).manual_seed(11)
+  for it in range(60):
+    D = rnd.choice([128, 128, 128, 64])
+    B, H = rnd.choice([1, 1, 2, 3]), rnd.choice([1, 2, 3, 5])
+    sq = rnd.choice([1, 7, 31, 32, 33, 64, 100, 255, 256, 257, 300, 511, 513, 1000])
+    skv = rnd.choice([1, 5, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 500, 1023, 1025, 3000, 3073, 3500, 4100])
+    layout, mult = rnd.choice(["bshd", "bhsd"]), rnd.choice([1.0, 1.0, 3.0, 8.0])
+    path = rnd.choice(["plain", "folded", "mask", "var1", "var2", "var3"] if D == 128 else ["plain", "folded", "mask"])
+
+    def mk(S):
+      x = torch.randn((B, S, H, D), generator=gen, device=dev)
+      return x.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3) if layout == "bhsd" else x
+
+    qf, k, v = mk(sq) * mult, mk(skv).to(torch.bfloat16), mk(skv).to(torch.bfloat16)
+    q, sc = ((qf * ops.folded_q_mul(D)).to(torch.bfloat16), ops.FOLDED_SCALE) if path == "folded" else (qf.to(torch.bfloat16), D**-0.5)
+    keep = bias = None
+    if path == "mask":
+      keep = torch.rand((B, skv), generator=gen, device=dev) < 0.7
+      keep[:, 0] = True
+      bias = ops.key_mask_bias(keep)
+    variant(int(path[3]) if path.startswith("var") else 0)
+    out, lse = ops.flash_attention(q, k, v, scale=sc, return_lse=True, key_bias=bias, out_layout=layout)
+    if keep is None:
+      ref, rl = torch_attention_f32(q, k, v, sc)
+    else:  # the reference sees only the kept keys of each batch element
+      parts = [torch_attention_f32(q[b:b + 1], k[b:b + 1, keep[b]], v[b:b + 1, keep[b]], sc) for b in range(B)]
+      ref, rl = torch.cat([p[0] for p in parts]), torch.cat([p[1] for p in parts])
+    what = f"draw {it}: B={B} H={H} Sq={sq} Skv={skv} D={D} {layout} x{mult} {path}"
+    d = (out.float() - ref).abs()
+    assert bool(torch.isfinite(out.float()).all()), what
+    assert float(d.max()) <= 2.5e-2 and float((lse - rl).abs().max()) <= 2e-3, what   # x8 logits: |out| up to ~4, one bf16 ulp is 1.6e-2
+    assert float((out.float() - ref).norm() / ref.norm()) <= REL_L2, what

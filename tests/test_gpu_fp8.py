@@ -151,3 +151,32 @@ def test_fp8_cross_attention_shape(dev):
   out, lse = _quant_run(q, k, v, dev)
   exact, _ = O.attention(hsd(q), hsd(k), hsd(v), 128**-0.5)
   assert cosine(hsd(out), exact) >= COS_BAR
+
+
+def test_fp8_seeded_sweep_of_shapes_layouts_and_scale_kinds(dev):
+  """Forty seeded draws of (batch, heads, Sq, Skv, layout, sharpness, power-of-two scales or not) against an f32
+  attention computed by torch on the GPU (test harness only): finite results and the cosine bar."""
+  import random
+  from helpers import torch_attention_f32
+  rnd = random.Random(12)
+  gen = torch.Generator(device=dev).manual_seed(12)
+  for it in range(40):
+    B, H = rnd.choice([1, 1, 2]), rnd.choice([1, 2, 3, 5])
+    sq = rnd.choice([1, 7, 31, 32, 33, 64, 100, 127, 128, 129, 255, 300, 513, 1000])
+    skv = rnd.choice([2, 5, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 500, 1023, 1025, 3000, 4100])
+    layout, mult, pow2 = rnd.choice(["bshd", "bhsd"]), rnd.choice([1.0, 1.0, 2.0, 4.0]), rnd.choice([True, False])
+    q, k, v = ((torch.randn((B, s_, H, 128), generator=gen, device=dev) * m).to(torch.bfloat16) for s_, m in ((sq, mult), (skv, 1.0), (skv, 1.0)))
+    if pow2:
+      (q8, s_q), (k8, s_k), sc = ops.quant_e4m3(q, premul=ops.folded_q_mul(128), pow2_scale=True), ops.quant_e4m3(k, pow2_scale=True), ops.FOLDED_SCALE
+    else:
+      (q8, s_q), (k8, s_k), sc = ops.quant_e4m3(q), ops.quant_e4m3(k), 128**-0.5
+    v8, s_v = ops.quant_e4m3(v)
+    if layout == "bhsd":
+      q8, k8, v8 = (t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3) for t in (q8, k8, v8))
+    out, lse = ops.flash_attention_fp8(q8, k8, v8, s_q, s_k, s_v, scale=sc, return_lse=True, out_layout=layout)
+    ref, rl = torch_attention_f32(q, k, v, 128**-0.5)
+    what = f"draw {it}: B={B} H={H} Sq={sq} Skv={skv} {layout} x{mult} pow2={pow2}"
+    o = out.float()
+    assert bool(torch.isfinite(o).all()) and bool(torch.isfinite(lse).all()), what
+    assert float((o * ref).sum() / (o.norm() * ref.norm())) >= (COS_BAR if mult == 1.0 else 0.985), what
+    assert float((lse - rl).abs().max()) <= (0.3 if mult == 1.0 else 2.0), what
