@@ -112,7 +112,10 @@ int mdattn_norm_rope_rows(void* stream, const void* x_in, int x_is_f32, void* x_
  *   out          bf16 [B,Sq,H,D] by o_strides
  *   lse          f32 [B,H,Sq] contiguous or NULL: natural-log logsumexp of scale*q.k
  *                (kernels/splash_attention/base.py:103-105)
- *   scale        applied to q.k inside the kernel (the reference pre-multiplies k, :1783)
+ *   scale        applied to q.k inside the kernel (the reference pre-multiplies k, :1783).  scale = ln 2, i.e.
+ *                scale * log2(e) == 1, says that q already carries the softmax scale times log2(e)
+ *                (mdattn_norm_rope_*'s q_mul): the kernels then form exp2 of the raw products and save the
+ *                multiply per logit; the result is that of the softmax scale on the plain q.
  * Requires D == 128, or D == 64 (LTX-2's audio stream, models/ltx2/transformer_ltx2.py:788-789).  Any Sq, Skv >= 1
  * (ragged tails handled in-kernel).
  */
@@ -166,6 +169,10 @@ int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, float* scal
  * fp8-e4m3 attention forward: q8/k8/v8 are e4m3 bytes [B,S,H,D] by strides, *_scale device f32[1]
  * de-quantisation factors; P is re-quantised to e4m3 per tile before the PV MFMA; f32 accumulation;
  * bf16 out; lse as above.  Requires D == 128.
+ * When scale * log2(e) * q_scale * k_scale is a power of two (see mdattn_quant_e4m3: premul, pow2_scale, and
+ * scale = ln 2 here) the logit scale is applied inside the MFMAs and the softmax needs no multiply; the scales are
+ * read on the device, so nothing has to be declared: two instances of the kernel are launched and the one whose
+ * case it is not returns at once.
  */
 int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, const void* v8, void* out, float* lse,
                    int B, int H, int Sq, int Skv, int D,
