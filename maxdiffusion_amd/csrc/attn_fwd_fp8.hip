@@ -37,8 +37,9 @@ constexpr int kKS8 = kD8;                                 // K row stride in LDS
 constexpr int kVS8 = kD8;                                 // V row stride in LDS, bytes (chunks permuted, not padded)
 constexpr int kStage8 = kBN8 * kKS8 + kBN8 * kVS8;        // bytes per LDS stage
 constexpr int kSlots8 = 3;                                // LDS ring depth
-constexpr float kPOff = 4.0f;                             // P = exp2(logit - max + kPOff) at a fresh maximum
-constexpr float kPTrig = 256.0f;                          // a 4-key partial row sum above this sends the wave to the rescale branch
+constexpr float kPOff = 3.0f;                             // P = exp2(logit - max + kPOff) at a fresh maximum
+constexpr float kPTrig = 448.0f;                          // a lane's partial row sum over one tile above this (e4m3's largest
+                                                          // value) sends the wave to the rescale branch
 
 typedef __attribute__((ext_vector_type(2))) int i32x2;
 typedef i32x2 __attribute__((address_space(3))) * lds_i32x2_ptr;
@@ -204,30 +205,28 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       }
     };
     // ---- P = exp2(c*S - ref), f32 row sum, e4m3 pack in B-operand order.  The hot path takes no row
-    // maximum: P is formed against the current reference point, and only a group of four probabilities
-    // that sums beyond 2^8 (so possibly one beyond it: e4m3 ends at 448) sends the wave through the branch
-    // that moves every row's reference to its true maximum - kPOff, rescales the accumulators and redoes
-    // the tile's logits and P.  Right after a move a group sums to at most 4 * 2^kPOff, so a row triggers again only
-    // when its maximum has grown by two more log2 units.  The two 32-key blocks of the tile are taken one after
-    // the other, so that only 16 logits per lane are alive at a time.
+    // maximum: P is formed against the current reference point, and only a lane's sum over the tile (32 of the
+    // row's 64 probabilities) beyond e4m3's largest value, so possibly one probability beyond it, sends the wave
+    // through the branch that moves every row's reference to its true maximum - kPOff, rescales the accumulators
+    // and redoes the tile's logits and P.  Right after a move such a sum is at most 32 * 2^kPOff = 256, so even a
+    // row of equal logits triggers again only when its level has grown by 0.8 log2 units.  The two 32-key blocks
+    // of the tile are taken one after the other, so that only 16 logits per lane are alive at a time.
     i32x8 pk;
-    float gmax, ls;
+    float ls;
     auto soft = [&](const f32x16& S, int blk, float rf) __attribute__((always_inline)) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         float p[4];
 #pragma unroll
         for (int x = 0; x < 4; ++x) p[x] = __builtin_amdgcn_exp2f(PRE ? S[4 * g + x] : __builtin_fmaf(S[4 * g + x], c, -rf));
-        const float s4 = (p[0] + p[1]) + (p[2] + p[3]);
-        ls += s4;
-        gmax = fmaxf(gmax, s4);
-        int u = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
+        ls += (p[0] + p[1]) + (p[2] + p[3]);
+        int u = __builtin_bit_cast(int, p[0]);  // any defined value: both halves are written below, in place
+        u = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], u, false);
         u = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], u, true);
         pk[4 * blk + g] = u;
       }
     };
     ls = 0.f;
-    gmax = 0.f;
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
       f32x16 S;
@@ -235,7 +234,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       soft(S, blk, ref);
       if (PRE) __builtin_amdgcn_sched_barrier(0);  // keeps the second block's logits from being hoisted over the first's softmax
     }
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(gmax <= kPTrig)) != 0 || (PRE && t == 0), 0)) {
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(ls <= kPTrig)) != 0 || (PRE && t == 0), 0)) {
       // The logits are recomputed rather than kept: the hot path holds them only while it forms P.
       int zero = 0;
       asm volatile("" : "+s"(zero));  // an address the compiler cannot match with the hot path's: no reuse of its logits
@@ -270,7 +269,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       // once more against the new reference points
       asm volatile("" : "+s"(zero));
       ls = 0.f;
-      gmax = 0.f;
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk) {
         f32x16 S;

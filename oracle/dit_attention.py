@@ -437,14 +437,15 @@ def quant_e4m3(x, premul: float = 1.0, pow2_scale: bool = False):
   return e4m3_round(x * (np.float32(premul) / s)), s
 
 
-def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: float = 4.0, p_trig: float = 256.0,
+def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: float = 3.0, p_trig: float = 448.0,
                            rows_per_wave: int = 32, pow2_scales: bool = False):
   """Emulation of the fp8 kernel's arithmetic (no reference counterpart).
 
   Q, K, V quantised per tensor; logits from the quantised operands in f32; online softmax per
   KV tile in base 2 with P rounded to e4m3 before the PV product; f32 accumulation; the row
   sum uses the un-rounded P.  P = exp2(logit - ref).  The reference point `ref` of a row moves
-  as the kernel moves it: when, in a tile, some aligned group of four keys of some row of the
+  as the kernel moves it: when, in a tile, one of the two interleaved halves of some row's keys (keys
+  whose index mod 8 is below 4, and the others: what one lane of the kernel holds) of some row of the
   same wave (rows_per_wave consecutive query rows) has probabilities summing beyond p_trig,
   every row of that wave takes ref = max(ref, tile max - p_offset).  P then stays within
   [0, p_trig], inside e4m3's range, and probabilities down to 2^-(6+p_offset) of the row max
@@ -472,9 +473,9 @@ def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: f
     with np.errstate(over="ignore"):
       p = np.exp2(s * c - ref[..., None]).astype(np.float32)
     n = p.shape[-1]
-    pg = np.zeros((H, Sq, -(-n // 4) * 4), np.float32)
+    pg = np.zeros((H, Sq, -(-n // 8) * 8), np.float32)
     pg[..., :n] = p
-    row_trig = ~(pg.reshape(H, Sq, -1, 4).sum(axis=-1).max(axis=-1) <= np.float32(p_trig))
+    row_trig = ~(pg.reshape(H, Sq, -1, 2, 4).sum(axis=(-3, -1), dtype=np.float32).max(axis=-1) <= np.float32(p_trig))
     wt = np.zeros((H, nw * rows_per_wave), bool)
     wt[:, :Sq] = row_trig
     wave_trig = np.repeat(wt.reshape(H, nw, rows_per_wave).any(axis=-1), rows_per_wave, axis=1)[:, :Sq]

@@ -64,7 +64,8 @@ def test_fp8_against_emulation_and_bf16_oracle(dev, sq, skv, mult, pow2):
 def test_fp8_reference_point_moves(dev, profile, pow2):
   """Logit profiles that make the rows' reference points move often, never, through sums without a single
   large term, and through one exponent far beyond e4m3's range: the kernel has to follow the emulation,
-  which applies the same rule (a group of four probabilities above 2^8 moves the wave's rows)."""
+  which applies the same rule (a lane's share of a row's probabilities in a tile summing beyond 448 moves the
+  wave's rows)."""
   H, sq, skv = 2, 150, 1500
   qs, ks = zip(*(structured_logits(sq, skv, 128, profile, seed=5 + h) for h in range(H)))
   q, k = np.stack(qs, 1)[None], np.stack(ks, 1)[None]
@@ -76,7 +77,7 @@ def test_fp8_reference_point_moves(dev, profile, pow2):
   print(f"fp8 {profile} pow2={pow2}: rel-l2 vs emulation {r:.3e}, lse vs emulation {lmx:.2e}, cos vs f32 oracle {cosine(hsd(out), exact):.5f} "
         f"(emulation {cosine(emu, exact):.5f})", flush=True)
   assert np.isfinite(out).all() and np.isfinite(lse).all()
-  # a row whose group sum sits at the threshold may move in one and not in the other: P is then rounded on a
+  # a row whose partial sum sits at the threshold may move in one and not in the other: P is then rounded on a
   # grid shifted by a few bits, which stays inside e4m3's own noise
   assert r <= 2e-2 and lmx <= 2e-3
   assert abs(cosine(hsd(out), exact) - cosine(emu, exact)) <= 2e-3
