@@ -60,6 +60,8 @@ def main():
   ap.add_argument("--traffic-probe", action="store_true",
                   help="also launch one 1 GiB device copy: the plain copy kernel of known size that scales rocprofv3's "
                        "FETCH_SIZE / WRITE_SIZE counters")
+  ap.add_argument("--separate-merge", action="store_true",
+                  help="ring workloads: one attention launch and one merge launch per KV chunk instead of the fused step")
   ap.add_argument("--with-backward", action="store_true",
                   help="also time the backward pass (dq, dk, dv) of the workload's attention, outside the timed steps; "
                        "reported as a `backward` object beside the headline")
@@ -135,8 +137,11 @@ def main():
       o_run, l_run = ops.new_merge_state(1, S, H, D, dev)
       for i in range(ring):
         kc = kn if i == 0 else k_extra[:, (i - 1) * Skv:i * Skv]
-        o, l = ops.flash_attention(qn, kc, v[:, i * Skv:(i + 1) * Skv], scale=att_scale, return_lse=True)
-        ops.merge_partial(o_run, l_run, o, l)
+        if args.separate_merge:
+          o, l = ops.flash_attention(qn, kc, v[:, i * Skv:(i + 1) * Skv], scale=att_scale, return_lse=True)
+          ops.merge_partial(o_run, l_run, o, l)
+        else:  # attention and merge in one launch
+          ops.flash_attention_merge(qn, kc, v[:, i * Skv:(i + 1) * Skv], o_run, l_run, scale=att_scale)
       ops.finalize(o_run)
     e2.record()
     if record:

@@ -209,6 +209,21 @@ int mdattn_merge(void* stream, float* o_run, float* lse_run, const void* o_cur, 
                  int cur_is_f32, int B, int H, int S, int D,
                  const mdattn_strides* run_strides, const mdattn_strides* cur_strides);
 
+/*
+ * mdattn_fwd_bf16 and mdattn_merge in one launch: attention of q against one K/V chunk, merged in LSE space into
+ * the running (o_run, lse_run) pair by the attention kernel's own epilogue, so the chunk's (out, lse) never goes
+ * to memory and its merge traffic hides behind the other workgroups' matrix work.  One ring step of the reference:
+ * kernels/splash_attention/ring_attention_kernel.py:1045-1073 (attention on the visiting K/V shard, then the merge),
+ * models/attention_flax.py:736-772.  Same result as the two calls, except that the chunk's output is not rounded to
+ * bf16 before the merge (the reference's ring step merges its f32 numerator too, :1058-1065).  Start from o_run = 0, lse_run = -1e30; mdattn_finalize turns o_run into bf16.
+ *   o_run  f32 [B,Sq,H,D] by run_strides (in floats; multiples of 8, 16-byte aligned base), lse_run f32 [B,H,Sq]
+ *   q, k, v, scale, D as for mdattn_fwd_bf16
+ */
+int mdattn_fwd_bf16_merge(void* stream, const void* q, const void* k, const void* v, float* o_run, float* lse_run,
+                          int B, int H, int Sq, int Skv, int D,
+                          const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                          const mdattn_strides* v_strides, const mdattn_strides* run_strides, float scale);
+
 /* f32 -> bf16 cast of the merged numerator (the `.astype(q.dtype)` of ring_attention_kernel.py:1130).
  * n % 8 == 0, both contiguous. */
 int mdattn_finalize(void* stream, const float* o_run, void* out_bf16, int64_t n);

@@ -73,6 +73,56 @@ __device__ __forceinline__ bf16x8 read_vt(const __bf16* p0, const __bf16* p1) {
   return __builtin_bit_cast(bf16x8, r);
 }
 
+// Epilogue of both schedules for one query row: lane (row, hh) holds, for each 32-wide block db of the head dim, the
+// values d = 32 db + 8 g + 4 hh + 0..3 (g = 0..3) of the un-normalised output, `lt` is the row's sum of P and `mc` its
+// reference point in log2 units.  Either out = O / lt as bf16 and lse = ln 2 * (mc + log2 lt), or, with a running
+// (o_run, lse_run) pair, the LSE-space merge of that result into the pair (ring_attention_kernel.py:1062-1073 of the
+// reference, with (0, -1e30) as the neutral start): the attention result of this call never goes to memory.
+template <int ND>
+__device__ __forceinline__ void store_row(const AttnArgs& a, const f32x16 (&O)[ND], float lt, float mc, int b, int h,
+                                          int row, int hh) {
+  if (row >= a.Sq) return;
+  const int64_t lidx = ((int64_t)b * a.H + h) * a.Sq + row;
+  if (a.o_run) {
+    const float l2 = lt > 0.f ? (mc + __log2f(lt)) * kLn2 : -INFINITY;
+    const float l1 = a.lse_run[lidx];  // both lanes of the row read it before lane hh = 0 writes it back
+    const float L = fmaxf(l1, l2);
+    float w1 = 0.f, w2 = 0.f;
+    if (L > -INFINITY) { w1 = expf(l1 - L); w2 = expf(l2 - L); }
+    const float den = w1 + w2;
+    const float invd = den > 0.f ? 1.0f / den : 0.f;
+    w1 *= invd;
+    w2 = lt > 0.f ? w2 * invd / lt : 0.f;
+    float* orow = a.o_run + b * a.o_sb + h * a.o_sh + (int64_t)row * a.o_ss + 4 * hh;
+#pragma unroll
+    for (int db = 0; db < ND; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float4* p = reinterpret_cast<float4*>(orow + db * 32 + 8 * g);
+        float4 r = *p;
+        r.x = w1 * r.x + w2 * O[db][4 * g];
+        r.y = w1 * r.y + w2 * O[db][4 * g + 1];
+        r.z = w1 * r.z + w2 * O[db][4 * g + 2];
+        r.w = w1 * r.w + w2 * O[db][4 * g + 3];
+        *p = r;
+      }
+    if (hh == 0) a.lse_run[lidx] = den > 0.f ? L + logf(den) : L;
+    return;
+  }
+  const float inv = lt > 0.f ? 1.0f / lt : 0.f;  // rows whose keys are all excluded return 0
+  __bf16* orow = a.out + b * a.o_sb + h * a.o_sh + (int64_t)row * a.o_ss + 4 * hh;
+#pragma unroll
+  for (int db = 0; db < ND; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      uint2 u;
+      u.x = pack2(O[db][4 * g] * inv, O[db][4 * g + 1] * inv);
+      u.y = pack2(O[db][4 * g + 2] * inv, O[db][4 * g + 3] * inv);
+      *reinterpret_cast<uint2*>(orow + db * 32 + 8 * g) = u;
+    }
+  if (a.lse && hh == 0) a.lse[lidx] = (mc + __log2f(lt)) * kLn2;
+}
+
 template <int NW, bool PRE>
 __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
@@ -332,23 +382,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
 #undef MDATTN_ITER
 
   // ---- epilogue: normalise, convert, store; lse = m*scale + ln(l)
-  __bf16* op = a.out + b * a.o_sb + h * a.o_sh;
-  const float lt = xhalf_sum(l);
-  const float inv = 1.0f / lt;
-  const int row = q0 + l32;
-  if (row < a.Sq) {
-    __bf16* orow = op + (int64_t)row * a.o_ss + 4 * hh;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        uint2 u;
-        u.x = pack2(O[db][4 * g] * inv, O[db][4 * g + 1] * inv);
-        u.y = pack2(O[db][4 * g + 2] * inv, O[db][4 * g + 3] * inv);
-        *reinterpret_cast<uint2*>(orow + db * 32 + 8 * g) = u;
-      }
-    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (mc + __log2f(lt)) * kLn2;
-  }
+  store_row<4>(a, O, xhalf_sum(l), mc, b, h, q0 + l32, hh);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -566,23 +600,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   __syncthreads();
   tile(nt - 1, slot, std::true_type{});
 
-  __bf16* op = a.out + b * a.o_sb + h * a.o_sh;
-  const float lt = xhalf_sum(l);
-  const float inv = lt > 0.f ? 1.0f / lt : 0.f;  // rows whose keys are all excluded return 0
-  const int row = q0 + l32;
-  if (row < a.Sq) {
-    __bf16* orow = op + (int64_t)row * a.o_ss + 4 * hh;
-#pragma unroll
-    for (int db = 0; db < ND; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        uint2 u;
-        u.x = pack2(O[db][4 * g] * inv, O[db][4 * g + 1] * inv);
-        u.y = pack2(O[db][4 * g + 2] * inv, O[db][4 * g + 3] * inv);
-        *reinterpret_cast<uint2*>(orow + db * 32 + 8 * g) = u;
-      }
-    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (mc + __log2f(lt)) * kLn2;
-  }
+  store_row<ND>(a, O, xhalf_sum(l), mc, b, h, q0 + l32, hh);
 }
 
 template <int NW, bool BIAS, int HD = 128>
@@ -647,17 +665,11 @@ static int fill_args(AttnArgs& a, const void* q, const void* k, const void* v, v
   a.o_sb = o_strides->batch; a.o_ss = o_strides->seq; a.o_sh = o_strides->head;
   a.c = scale * kLog2e;
   a.bias = nullptr; a.bias_sb = 0;
+  a.o_run = nullptr; a.lse_run = nullptr;
   return MDATTN_OK;
 }
 
-extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* out, float* lse,
-                               int B, int H, int Sq, int Skv, int D,
-                               const mdattn_strides* q_strides, const mdattn_strides* k_strides,
-                               const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
-  AttnArgs a;
-  const int rc = fill_args(a, q, k, v, out, lse, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides, scale);
-  if (rc != MDATTN_OK) return rc;
-  hipStream_t st = (hipStream_t)stream;
+static int dispatch_fwd(hipStream_t st, const AttnArgs& a, int B, int Sq, int Skv, int D) {
   if (D == 64) return launch_flat<4, false, 64>(st, a, B);  // head dim 64: the flat schedule only
 
   // Two schedules.  The software-pipelined kernel (8 waves x 32 query rows, two waves per SIMD) is the faster one
@@ -668,7 +680,7 @@ extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const
   int variant = 0;
   if (const char* e = getenv("MDATTN_FWD_VARIANT")) variant = atoi(e);
   if (variant == 0) {
-    const int64_t wg256 = (int64_t)B * H * ((Sq + 255) / 256);
+    const int64_t wg256 = (int64_t)B * a.H * ((Sq + 255) / 256);
     variant = (Skv <= 3072 || wg256 < 128) ? 3 : 1;
   }
   switch (variant) {
@@ -677,6 +689,32 @@ extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const
     case 3: return launch_flat<4, false>(st, a, B);
     default: return MDATTN_E_BADARG;
   }
+}
+
+extern "C" int mdattn_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* out, float* lse,
+                               int B, int H, int Sq, int Skv, int D,
+                               const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                               const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
+  AttnArgs a;
+  const int rc = fill_args(a, q, k, v, out, lse, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides, scale);
+  if (rc != MDATTN_OK) return rc;
+  return dispatch_fwd((hipStream_t)stream, a, B, Sq, Skv, D);
+}
+
+extern "C" int mdattn_fwd_bf16_merge(void* stream, const void* q, const void* k, const void* v, float* o_run, float* lse_run,
+                                     int B, int H, int Sq, int Skv, int D,
+                                     const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                                     const mdattn_strides* v_strides, const mdattn_strides* run_strides, float scale) {
+  if (!o_run || !lse_run) return MDATTN_E_BADARG;
+  if (reinterpret_cast<uintptr_t>(lse_run) & 3u) return MDATTN_E_ALIGN;
+  AttnArgs a;
+  // o_run stands in for `out` in the checks (16-byte alignment, strides in elements, multiples of 8)
+  const int rc = fill_args(a, q, k, v, o_run, nullptr, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, run_strides, scale);
+  if (rc != MDATTN_OK) return rc;
+  a.out = nullptr;
+  a.o_run = o_run;
+  a.lse_run = lse_run;
+  return dispatch_fwd((hipStream_t)stream, a, B, Sq, Skv, D);
 }
 
 extern "C" int mdattn_fwd_bf16_bias(void* stream, const void* q, const void* k, const void* v, void* out, float* lse,

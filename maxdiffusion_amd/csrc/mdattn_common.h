@@ -108,6 +108,8 @@ struct AttnArgs {
   float c;  // scale * log2(e)
   const float* bias;   // optional additive per-key bias [B, bias_sb] (natural-log units), flat kernel only
   int64_t bias_sb;
+  float* o_run;    // when set: no `out`; the result is merged in LSE space into this f32 carry (strides o_s*, in floats)
+  float* lse_run;  // ... and into its lse [B,H,Sq]
 };
 
 

@@ -287,6 +287,30 @@ def merge_partial(o_run, lse_run, o_cur, lse_cur):
   return o_run, lse_run
 
 
+def flash_attention_merge(q, k, v, o_run, lse_run, scale: float | None = None):
+  """One ring step in one launch: attention of q [B,Sq,H,D] against the chunk k/v [B,Skv,H,D] (bf16 logical views),
+  merged in place into (o_run f32 logical [B,Sq,H,D], lse_run f32 [B,H,Sq]) as `merge_partial` would merge the
+  result of `flash_attention`; the chunk's own output is never stored."""
+  _check_dev(q, k, v, o_run, lse_run)
+  if not (q.dtype == k.dtype == v.dtype == torch.bfloat16):
+    raise ValueError("flash_attention_merge needs bf16 q, k, v")
+  b, sq, h, d = q.shape
+  if k.shape != v.shape or k.shape[0] != b or k.shape[2] != h or k.shape[3] != d:
+    raise ValueError(f"inconsistent shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)}")
+  if o_run.dtype != torch.float32 or tuple(o_run.shape) != (b, sq, h, d):
+    raise ValueError("o_run must be an f32 logical [B,Sq,H,D] view")
+  if lse_run.dtype != torch.float32 or tuple(lse_run.shape) != (b, h, sq) or not lse_run.is_contiguous():
+    raise ValueError("lse_run must be contiguous f32 [B,H,Sq]")
+  if scale is None:
+    scale = 1.0 / math.sqrt(d)
+  sq_, sk_, sv_, sr_ = _strides(q), _strides(k), _strides(v), _strides(o_run)
+  rc = _lib.load().mdattn_fwd_bf16_merge(
+      _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(o_run), _ptr(lse_run), b, h, sq, k.shape[1], d,
+      ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(sr_), float(scale))
+  _lib.check(rc, "mdattn_fwd_bf16_merge")
+  return o_run, lse_run
+
+
 def finalize(o_run: torch.Tensor) -> torch.Tensor:
   """f32 -> bf16 cast of a merged accumulator, same memory layout."""
   _check_dev(o_run)

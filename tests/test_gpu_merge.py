@@ -66,6 +66,54 @@ def test_ring_replay_small_unequal_chunks(dev):
   assert err_stats(to_np(l_run)[0], rl)[0] < 1e-3
 
 
+@pytest.mark.parametrize("layout", ["bshd", "bhsd"])
+@pytest.mark.parametrize("variant", [0, 1, 3])
+def test_fused_ring_step_equals_attention_then_merge(dev, monkeypatch, layout, variant):
+  """mdattn_fwd_bf16_merge (attention + merge in the attention kernel's epilogue) against the two separate calls
+  and against the oracle, with ragged chunks, through both schedules and both layouts of the carry."""
+  if variant:
+    monkeypatch.setenv("MDATTN_FWD_VARIANT", str(variant))
+  H, Sq = 3, 333
+  q = O.normal_bf16((1, Sq, H, 128), 0)
+  sizes = [4200, 1, 63, 777, 3100]
+  ks = [O.normal_bf16((1, n, H, 128), 10 + i) for i, n in enumerate(sizes)]
+  vs = [O.normal_bf16((1, n, H, 128), 20 + i) for i, n in enumerate(sizes)]
+  qd = to_dev_bf16(q, dev)
+  o_f, l_f = ops.new_merge_state(1, Sq, H, 128, dev, layout=layout)
+  o_s, l_s = ops.new_merge_state(1, Sq, H, 128, dev, layout=layout)
+  for kc, vc in zip(ks, vs):
+    kd, vd = to_dev_bf16(kc, dev), to_dev_bf16(vc, dev)
+    ops.flash_attention_merge(qd, kd, vd, o_f, l_f)
+    o, l = ops.flash_attention(qd, kd, vd, return_lse=True)
+    ops.merge_partial(o_s, l_s, o, l)
+  # the separate path rounds each chunk's output to bf16 before the merge, the fused one does not
+  assert float((o_f - o_s).abs().max()) < 8e-3
+  assert float((l_f - l_s).abs().max()) < 1e-5
+  ro, rl = O.attention(hsd(q), hsd(np.concatenate(ks, 1)), hsd(np.concatenate(vs, 1)), 128**-0.5)
+  out = to_np(ops.finalize(o_f))
+  mx, mean = err_stats(hsd(out), ro)
+  mx_s = err_stats(hsd(to_np(ops.finalize(o_s))), ro)[0]
+  print(f"fused ring step ({layout}, variant {variant}): max-abs {mx:.3e} (separate calls {mx_s:.3e}) mean-abs {mean:.3e}")
+  assert mx < 2e-2 and mean < 2e-3 and rel_l2(hsd(out), ro) < 1.5e-2
+  assert err_stats(to_np(l_f)[0], rl)[0] < 1e-3
+
+
+def test_fused_ring_step_neutral_start_and_folded_scale(dev):
+  """A single fused step from the neutral start is the attention itself (f32, unrounded), also with the softmax
+  scale carried by q (scale = ln 2)."""
+  H, Sq, Skv = 2, 100, 5000
+  q, k, v = O.normal_bf16((1, Sq, H, 128), 0), O.normal_bf16((1, Skv, H, 128), 1), O.normal_bf16((1, Skv, H, 128), 2)
+  for folded in (False, True):
+    qd = to_dev_bf16(O.bf16_round(q * np.float32(ops.folded_q_mul(128))) if folded else q, dev)
+    sc = ops.FOLDED_SCALE if folded else None
+    o_run, l_run = ops.new_merge_state(1, Sq, H, 128, dev)
+    ops.flash_attention_merge(qd, to_dev_bf16(k, dev), to_dev_bf16(v, dev), o_run, l_run, scale=sc)
+    out, lse = ops.flash_attention(qd, to_dev_bf16(k, dev), to_dev_bf16(v, dev), scale=sc, return_lse=True)
+    assert float((o_run - out.float()).abs().max()) < 4e-3  # out is the bf16 rounding of what o_run holds
+    assert float((l_run - lse).abs().max()) < 1e-6
+    assert to_np(ops.finalize(o_run)).tobytes() == to_np(out).tobytes()
+
+
 def test_wan14b_ring_shard_replay_full_size(dev):
   """Config 3: a 9 450-token Q chunk x 40 heads against 8 successive 9 450-token KV chunks; the merged
   result must equal full 75 600-token attention for that Q chunk."""
