@@ -150,6 +150,28 @@ ffi::Error MergeImpl(hipStream_t stream, ffi::AnyBuffer o_run_in, ffi::AnyBuffer
                  "mdattn_merge");
 }
 
+// One ring hop: attention of q against the visiting K/V chunk, merged into the donated (o_run, lse_run) in one launch.
+ffi::Error FwdBf16MergeImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v,
+                            ffi::AnyBuffer o_run_in, ffi::AnyBuffer lse_run_in, ffi::Result<ffi::AnyBuffer> o_run,
+                            ffi::Result<ffi::AnyBuffer> lse_run, float scale, int64_t layout) {
+  if (o_run->untyped_data() != o_run_in.untyped_data() || lse_run->untyped_data() != lse_run_in.untyped_data())
+    return ffi::Error::InvalidArgument("mdattn_fwd_bf16_merge: o_run and lse_run must alias their outputs (input_output_aliases={3:0,4:1})");
+  if (q.element_type() != ffi::BF16 || k.element_type() != ffi::BF16 || v.element_type() != ffi::BF16 ||
+      o_run->element_type() != ffi::F32 || lse_run->element_type() != ffi::F32)
+    return ffi::Error::InvalidArgument("mdattn_fwd_bf16_merge: q, k, v must be bf16, o_run and lse_run f32");
+  int64_t B, Sq, H, D, Bk, Skv, Hk, Dk, Bo, So, Ho, Do;
+  mdattn_strides sq, sk, sv, so;
+  if (!Describe(q.dimensions(), layout, &B, &Sq, &H, &D, &sq) || !Describe(k.dimensions(), layout, &Bk, &Skv, &Hk, &Dk, &sk) ||
+      !Describe(v.dimensions(), layout, &Bk, &Skv, &Hk, &Dk, &sv) || !Describe(o_run->dimensions(), 0, &Bo, &So, &Ho, &Do, &so))
+    return ffi::Error::InvalidArgument("mdattn_fwd_bf16_merge: rank-4 buffers expected");
+  if (Bk != B || Hk != H || Dk != D || Bo != B || So != Sq || Ho != H || Do != D)
+    return ffi::Error::InvalidArgument("mdattn_fwd_bf16_merge: inconsistent shapes");
+  return ToError(mdattn_fwd_bf16_merge(stream, q.untyped_data(), k.untyped_data(), v.untyped_data(),
+                                       static_cast<float*>(o_run->untyped_data()), static_cast<float*>(lse_run->untyped_data()),
+                                       (int)B, (int)H, (int)Sq, (int)Skv, (int)D, &sq, &sk, &sv, &so, scale),
+                 "mdattn_fwd_bf16_merge");
+}
+
 }  // namespace
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnFwdBf16, FwdBf16Impl,
@@ -202,3 +224,11 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnMerge, MergeImpl,
                                   .Ctx<ffi::PlatformStream<hipStream_t>>()
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
                                   .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>());
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnFwdBf16Merge, FwdBf16MergeImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
+                                  .Attr<float>("scale").Attr<int64_t>("layout"));

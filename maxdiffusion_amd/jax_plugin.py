@@ -24,6 +24,7 @@ FFI_TARGETS = {
     "mdattn_norm_rope_perhead": "MdattnNormRopePerhead",
     "mdattn_norm_rope_rows": "MdattnNormRopeRows",
     "mdattn_merge": "MdattnMerge",
+    "mdattn_fwd_bf16_merge": "MdattnFwdBf16Merge",
 }
 
 _installed = False
@@ -76,6 +77,22 @@ def hip_flash_attention(q, k, v, scale: float, layout: int, keep_mask=None):
     )
     return call(q, k, v, bias, scale=np.float32(scale), layout=np.int64(layout))
   return call(q, k, v, scale=np.float32(scale), layout=np.int64(layout))
+
+
+def hip_ring_step(q, k_chunk, v_chunk, o_run, lse_run, scale: float, layout: int = 0):
+  """One ring hop in one custom call: attention of q against the visiting K/V chunk merged into the carry
+  (o_run f32 [B,Sq,H,D], lse_run f32 [B,H,Sq]; start from zeros and -1e30).  The body of the scan step in
+  kernels/splash_attention/ring_attention_kernel.py:1045-1073; the carry is donated and updated in place."""
+  jax, jnp = _require_jax()
+  import numpy as np
+
+  call = jax.ffi.ffi_call(
+      "mdattn_fwd_bf16_merge",
+      (jax.ShapeDtypeStruct(o_run.shape, jnp.float32), jax.ShapeDtypeStruct(lse_run.shape, jnp.float32)),
+      input_output_aliases={3: 0, 4: 1},
+      vmap_method="sequential",
+  )
+  return call(q, k_chunk, v_chunk, o_run, lse_run, scale=np.float32(scale), layout=np.int64(layout))
 
 
 def hip_flash_attention_vjp(q, k, v, scale: float):

@@ -17,7 +17,7 @@ from ._lib import Strides
 
 __all__ = [
     "norm_rope_fullrow", "norm_rope_perhead", "norm_rope_rows", "flash_attention", "flash_attention_backward", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
-    "merge_partial", "finalize", "new_merge_state", "LSE_INIT", "FOLDED_SCALE", "folded_q_mul",
+    "merge_partial", "flash_attention_merge", "finalize", "new_merge_state", "LSE_INIT", "FOLDED_SCALE", "folded_q_mul",
 ]
 
 LSE_INIT = -1e30
