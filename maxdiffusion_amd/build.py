@@ -37,12 +37,53 @@ def _hipcc() -> str:
 
 
 def _filter(stderr: str) -> str:
-  return "\n".join(l for l in stderr.splitlines() if "packed-fp32-ops" not in l)
+  """hipcc's stderr without the resource-usage remarks (and their source excerpts) and the host pass's complaint
+  about the target feature it does not know."""
+  import re
+
+  keep, in_remark = [], False
+  for l in stderr.splitlines():
+    if "remark:" in l:
+      in_remark = True
+      continue
+    if in_remark and re.match(r"^\s*(\d+\s*)?\|", l):
+      continue
+    in_remark = False
+    if "packed-fp32-ops" in l or "-Rpass-analysis" in l or re.match(r"^\d+ (warning|remark)s? generated", l):
+      continue
+    keep.append(l)
+  return "\n".join(keep)
+
+
+def _resource_table(stderr: str) -> list[tuple[str, dict]]:
+  """Kernel name -> registers, scratch and occupancy from hipcc's kernel-resource-usage remarks."""
+  import re
+
+  rows, cur = [], None
+  for line in stderr.splitlines():
+    m = re.search(r"remark: Function Name: (\S+)", line)
+    if m:
+      cur = {}
+      rows.append((m.group(1), cur))
+      continue
+    m = re.search(r"remark:\s+(VGPRs|AGPRs|ScratchSize \[bytes/lane\]|Occupancy \[waves/SIMD\]|LDS Size \[bytes/block\]): (\d+)", line)
+    if m and cur is not None:
+      cur[m.group(1).split(" ")[0]] = int(m.group(2))
+  return rows
+
+
+def _demangled(names: list[str]) -> dict[str, str]:
+  exe = shutil.which("llvm-cxxfilt") or shutil.which("c++filt") or "/opt/rocm/lib/llvm/bin/llvm-cxxfilt"
+  if not names or not os.path.exists(exe):
+    return {n: n for n in names}
+  out = subprocess.run([exe, *names], capture_output=True, text=True).stdout.splitlines()
+  return dict(zip(names, out)) if len(out) == len(names) else {n: n for n in names}
 
 
 def build_library(verbose: bool = True) -> str:
   """Compile every HIP source into maxdiffusion_amd/libmdattn.so.  Always recompiles."""
-  cmd = [_hipcc(), *HIPCC_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", "-o", LIB_PATH, *[os.path.join(CSRC, s) for s in SOURCES]]
+  cmd = [_hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", f"-I{INCLUDE}", f"-I{CSRC}", "-o", LIB_PATH,
+         *[os.path.join(CSRC, s) for s in SOURCES]]
   if verbose:
     print("[maxdiffusion_amd.build]", " ".join(cmd), flush=True)
   r = subprocess.run(cmd, capture_output=True, text=True)
@@ -51,6 +92,14 @@ def build_library(verbose: bool = True) -> str:
     raise RuntimeError(f"hipcc failed ({r.returncode}):\n{r.stdout}\n{err}")
   if verbose and err.strip():
     print(err, file=sys.stderr)
+  if verbose:  # registers, spills and occupancy of every kernel: a spill in a hot loop shows here, not in a test
+    rows = _resource_table(r.stderr)
+    names = _demangled([n for n, _ in rows])
+    for n, d in rows:
+      short = names[n].split("(")[0].replace("void ", "").replace("mdattn::", "").replace("(anonymous namespace)::", "")
+      spill = "  <-- spills" if d.get("ScratchSize", 0) else ""
+      print(f"[maxdiffusion_amd.build]   {short:<46} vgpr {d.get('VGPRs', 0):>3} agpr {d.get('AGPRs', 0):>3} "
+            f"scratch {d.get('ScratchSize', 0):>3} B  lds {d.get('LDS', 0):>6} B  waves/SIMD {d.get('Occupancy', 0)}{spill}", flush=True)
   return LIB_PATH
 
 
