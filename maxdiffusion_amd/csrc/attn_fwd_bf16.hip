@@ -18,12 +18,15 @@
 //                point m is not its running maximum: it only keeps P, l and O inside the f32 exponent range and
 //                moves when a logit exceeds it by about 20 log2 units, which the row's partial sum reveals, so
 //                the hot stream computes no maximum at all and the accumulator rescale sits in a cold branch.
+//                When the caller's q already carries scale*log2(e) (scale = ln 2: template flag PRE) the FMA goes
+//                too: the score chains start from minus the reference point and P is one exp2 away.
 //   pipelining = the vector ALU issues through the same port as the MFMAs.  Phases of pure MFMA
 //                followed by phases of pure VALU leave the matrix pipe idle half of the time, so the
 //                keys are walked in blocks of 32, and in iteration b every wave issues, interleaved in
 //                one instruction stream,
 //                    matrix pipe : O^T += V^T(b-1).P^T(b-1)  (8 MFMAs)  and  S^T(b+1) = K(b+1).Q^T  (8 MFMAs)
-//                    vector ALU  : P(b) = exp2(c*S(b) - c*m), row sums, bf16 convert (3.5 instructions per MFMA)
+//                    vector ALU  : P(b) = exp2(c*S(b) - c*m), row sums, bf16 convert (3.5 instructions per MFMA,
+//                                  2.5 with PRE)
 //                    LDS         : the K / V^T fragment of the next MFMA of the same kind
 //                PV and QK MFMAs alternate, so no MFMA depends on the one issued just before it.  The
 //                loop body is the same for every iteration: the iterations before the first and after
