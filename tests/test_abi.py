@@ -93,6 +93,14 @@ def test_bad_arguments_are_rejected_on_the_host(lib):
   assert m(None, fake, fake, fake, fake, 0, 1, 4, 8, 100, st, st) == _lib.E_UNSUPPORTED
   assert m(None, fake, P(0x1002), fake, fake, 0, 1, 4, 8, 128, st, st) == _lib.E_ALIGN
 
+  fm = lib.mdattn_fwd_bf16_merge
+  assert fm(None, fake, fake, fake, None, fake, 1, 4, 8, 8, 128, st, st, st, st, 0.1) == _lib.E_BADARG  # no carry
+  assert fm(None, fake, fake, fake, fake, None, 1, 4, 8, 8, 128, st, st, st, st, 0.1) == _lib.E_BADARG  # no lse carry
+  assert fm(None, fake, fake, fake, odd, fake, 1, 4, 8, 8, 128, st, st, st, st, 0.1) == _lib.E_ALIGN
+  assert fm(None, fake, fake, fake, fake, P(0x1002), 1, 4, 8, 8, 128, st, st, st, st, 0.1) == _lib.E_ALIGN
+  assert fm(None, fake, fake, fake, fake, fake, 1, 4, 8, 8, 32, st, st, st, st, 0.1) == _lib.E_UNSUPPORTED
+  assert fm(None, fake, fake, fake, fake, fake, 1, 4, 8, 0, 128, st, st, st, st, 0.1) == _lib.E_BADARG
+
   assert lib.mdattn_finalize(None, fake, fake, 12) == _lib.E_UNSUPPORTED
   assert lib.mdattn_finalize(None, fake, None, 16) == _lib.E_BADARG
   assert lib.mdattn_quant_e4m3(None, fake, fake, fake, 24, 1.0, 0) == _lib.E_UNSUPPORTED
