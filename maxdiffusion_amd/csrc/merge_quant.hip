@@ -59,8 +59,11 @@ __global__ __launch_bounds__(256) void finalize_kernel(const float4* __restrict_
 
 __global__ void zero2_kernel(float* p) { if (threadIdx.x < 2) p[threadIdx.x] = 0.f; }
 
-// |x| of a non-negative-masked bf16 orders like its bit pattern, so the absmax is an integer max.
+// |x| of a non-negative-masked bf16 orders like its bit pattern, so the absmax is an integer max.  Eight independent
+// 16-byte loads in flight per lane and trip; one atomic per workgroup (thousands of same-address atomics from every
+// wave would cost as much as the read itself).
 __global__ __launch_bounds__(256) void absmax_kernel(const uint4* __restrict__ x, int64_t n8, unsigned* amax_bits) {
+  __shared__ unsigned wmax[4];
   unsigned m = 0;
   auto fold = [&](const uint4& u) {
     const unsigned w[4] = {u.x, u.y, u.z, u.w};
@@ -70,17 +73,24 @@ __global__ __launch_bounds__(256) void absmax_kernel(const uint4* __restrict__ x
       m = max(m, max(lo, hi));
     }
   };
-  // four independent 16-byte loads in flight per lane and trip
   const int64_t stride = (int64_t)gridDim.x * 256;
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  for (; i + 3 * stride < n8; i += 4 * stride) {
-    const uint4 u0 = x[i], u1 = x[i + stride], u2 = x[i + 2 * stride], u3 = x[i + 3 * stride];
-    fold(u0); fold(u1); fold(u2); fold(u3);
+  for (; i + 7 * stride < n8; i += 8 * stride) {
+    uint4 u[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) u[j] = ld_nt(x + i + j * stride);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) fold(u[j]);
   }
   for (; i < n8; i += stride) fold(x[i]);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, o));
-  if ((threadIdx.x & 63) == 0 && m) atomicMax(amax_bits, m);
+  if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    m = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
+    if (m) atomicMax(amax_bits, m);
+  }
 }
 
 // x8 = e4m3(x * premul / s) with s = absmax(x * premul) / 448, or the next power of two above it (pow2): a
@@ -166,7 +176,7 @@ extern "C" int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, 
   if (!aligned16(x_bf16) || !aligned16(x_fp8) || (reinterpret_cast<uintptr_t>(scale_out) & 7u)) return MDATTN_E_ALIGN;
   hipStream_t st = (hipStream_t)stream;
   const int64_t n8 = n / 8, n16 = n / 16;
-  const unsigned g1 = (unsigned)((n8 + 255) / 256 < 4096 ? (n8 + 255) / 256 : 4096);
+  const unsigned g1 = (unsigned)((n8 + 255) / 256 < 2048 ? (n8 + 255) / 256 : 2048);
   const unsigned g2 = (unsigned)((n16 + 255) / 256 < 16384 ? (n16 + 255) / 256 : 16384);
   hipLaunchKernelGGL(zero2_kernel, dim3(1), dim3(64), 0, st, scale_out);
   hipLaunchKernelGGL(absmax_kernel, dim3(g1), dim3(256), 0, st, (const uint4*)x_bf16, n8, (unsigned*)(scale_out + 1));
