@@ -38,6 +38,14 @@ constexpr int kVS8 = kD8;                                 // V row stride in LDS
 constexpr int kStage8 = kBN8 * kKS8 + kBN8 * kVS8;        // bytes per LDS stage
 constexpr int kSlots8 = 3;                                // LDS ring depth
 constexpr float kPOff = 3.0f;                             // P = exp2(logit - max + kPOff) at a fresh maximum
+// Softmax without exponentials (MODE 2).  An e4m3 byte read as an integer is a piecewise-linear log2 of its value:
+// code = 8 * (exponent + 7) + mantissa.  So the QK MFMAs are made to deliver x' = 8 * (logit - ref) + 56 (block scale
+// times 8, start value 56 - 8 ref), and v_cvt_pk_u8_f32 (round to nearest even, saturating at 0) turns x' straight
+// into the operand byte: P~ = e4m3(code), equal to 2^(logit - ref) at every power of two and up to 6 % above it in
+// between (mean ratio 1.0404, against e4m3's own rounding noise of the same size).  The row sum is taken over the
+// decoded bytes, so O / l stays a properly normalised average; the lse carries the mean ratio as a constant.
+constexpr float kCodeOne = 56.0f;                         // the byte of P~ = 1
+constexpr float kCodeBiasLog2 = 0.0570814f;               // log2 of the mean of P~ / 2^x over a binade
 constexpr float kPTrig = 448.0f;                          // a lane's partial row sum over one tile above this (e4m3's largest
                                                           // value) sends the wave to the rescale branch
 
@@ -64,8 +72,10 @@ struct Fp8Args {
 
 // Register budget: three waves per SIMD (<= 168 VGPRs).  The kernel is bound by the vector ALU (softmax)
 // and by latencies a single wave cannot hide, so the third wave per SIMD is worth more than registers.
-template <int NW, bool PRE>
+template <int NW, int MODE>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_fwd_fp8_kernel(Fp8Args a) {
+  constexpr bool PRE = MODE != 0;    // the logit scale is a power of two and rides in the MFMAs' block scale
+  constexpr bool CODE = MODE == 2;   // ... and P is formed without exp2: see kCodeOne
   extern __shared__ __attribute__((aligned(16))) char smem8[];
   constexpr int NT = NW * 64;
   constexpr int BM = NW * 32;
@@ -153,11 +163,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   // scale already inside q), the MFMAs apply it through their block-scale operand and start every logit chain at
   // minus the row's reference point: the logits arrive in log2 units relative to it and the softmax needs no
   // multiply.  The reference then starts at 0 and the first tile always takes the branch that sets it.
-  const int sexp = (int)(__float_as_uint(c) >> 23);  // E8M0 code of c
+  const int sexp = (int)(__float_as_uint(c) >> 23) + (CODE ? 3 : 0);  // E8M0 code of c (of 8 c when the logits come in code units)
   float ref = PRE ? 0.f : -1e30f, l = 0.f;           // reference point of P (log2 units), per-lane partial row sum
   f32x16 negref;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) negref[i] = 0.f;
+  for (int i = 0; i < 16; ++i) negref[i] = CODE ? kCodeOne : 0.f;
 
   // lane-constant LDS offsets (bytes)
   // K fragment (d half j, 16-byte half i) of row l32 is logical chunk 4j + 2hh + i
@@ -213,17 +223,30 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
     // of the tile are taken one after the other, so that only 16 logits per lane are alive at a time.
     i32x8 pk;
     float ls;
+    unsigned hib = 0;  // MODE 2: OR of the operand dwords; a byte above 127 is a logit beyond e4m3's range
     auto soft = [&](const f32x16& S, int blk, float rf) __attribute__((always_inline)) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        float p[4];
+        if constexpr (CODE) {
+          unsigned u = __float_as_uint(S[4 * g]);  // any defined value: all four bytes are written below
+          u = __builtin_amdgcn_cvt_pk_u8_f32(S[4 * g], 0, u);
+          u = __builtin_amdgcn_cvt_pk_u8_f32(S[4 * g + 1], 1, u);
+          u = __builtin_amdgcn_cvt_pk_u8_f32(S[4 * g + 2], 2, u);
+          u = __builtin_amdgcn_cvt_pk_u8_f32(S[4 * g + 3], 3, u);
+          const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)u, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)u, true);
+          ls += (lo[0] + lo[1]) + (hi[0] + hi[1]);
+          hib |= u;
+          pk[4 * blk + g] = (int)u;
+        } else {
+          float p[4];
 #pragma unroll
-        for (int x = 0; x < 4; ++x) p[x] = __builtin_amdgcn_exp2f(PRE ? S[4 * g + x] : __builtin_fmaf(S[4 * g + x], c, -rf));
-        ls += (p[0] + p[1]) + (p[2] + p[3]);
-        int u = __builtin_bit_cast(int, p[0]);  // any defined value: both halves are written below, in place
-        u = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], u, false);
-        u = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], u, true);
-        pk[4 * blk + g] = u;
+          for (int x = 0; x < 4; ++x) p[x] = __builtin_amdgcn_exp2f(PRE ? S[4 * g + x] : __builtin_fmaf(S[4 * g + x], c, -rf));
+          ls += (p[0] + p[1]) + (p[2] + p[3]);
+          int u = __builtin_bit_cast(int, p[0]);  // any defined value: both halves are written below, in place
+          u = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], u, false);
+          u = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], u, true);
+          pk[4 * blk + g] = u;
+        }
       }
     };
     ls = 0.f;
@@ -234,7 +257,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       soft(S, blk, ref);
       if (PRE) __builtin_amdgcn_sched_barrier(0);  // keeps the second block's logits from being hoisted over the first's softmax
     }
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(ls <= kPTrig)) != 0 || (PRE && t == 0), 0)) {
+    // (a byte 0x7F decodes to NaN and poisons the sum; bytes above it are caught by their top bit)
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(ls <= (CODE ? 3.0e38f : kPTrig)) || (hib & 0x80808080u) != 0u) != 0 || (PRE && t == 0), 0)) {
       // The logits are recomputed rather than kept: the hot path holds them only while it forms P.
       int zero = 0;
       asm volatile("" : "+s"(zero));  // an address the compiler cannot match with the hot path's: no reuse of its logits
@@ -247,13 +271,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
         for (int i = 0; i < 16; ++i) mx = fmaxf(mx, S[i]);
       }
       float alpha;
-      if constexpr (PRE) {  // the logits are relative to the old reference
+      if constexpr (PRE) {  // the logits are relative to the old reference (MODE 2: in code units, 56 at the reference)
         mx = xhalf_max(mx);
+        if constexpr (CODE) mx = (mx - kCodeOne) * 0.125f;
         const float dm = t == 0 ? mx - kPOff : fmaxf(mx - kPOff, 0.f);
         alpha = t == 0 ? 0.f : __builtin_amdgcn_exp2f(-dm);
         ref += dm;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) negref[i] = -ref;
+        for (int i = 0; i < 16; ++i) negref[i] = CODE ? kCodeOne - 8.0f * ref : -ref;
       } else {
         mx = xhalf_max(mx) * c;
         const float nref = fmaxf(ref, mx - kPOff);
@@ -269,6 +294,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       // once more against the new reference points
       asm volatile("" : "+s"(zero));
       ls = 0.f;
+      hib = 0u;
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk) {
         f32x16 S;
@@ -323,7 +349,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
         u.y = pack2(O[sl][4 * g + 2] * inv, O[sl][4 * g + 3] * inv);
         *reinterpret_cast<uint2*>(orow + sl * 32 + 8 * g) = u;
       }
-    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (ref + __log2f(lt)) * kLn2;
+    if (a.lse && hh == 0) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (ref + __log2f(lt) - (CODE ? kCodeBiasLog2 : 0.f)) * kLn2;
   }
 }
 
@@ -336,8 +362,11 @@ int launch_fwd8(hipStream_t st, Fp8Args a, int B) {
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
-  hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, false>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
-  hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, true>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 0>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  // Power-of-two logit scale: the exponential-free softmax; MDATTN_FP8_SOFTMAX=1 keeps exp2 there too (experiments).
+  const char* e = getenv("MDATTN_FP8_SOFTMAX");
+  if (e && atoi(e) == 1) hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 1>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  else hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 2>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   return launch_status();
 }
 

@@ -33,8 +33,9 @@ Pinning status of each function (what fixes it besides its own formula):
                                  (2e-2) against `attention`, like the reference's
                                  own tests do (tests/attention_test.py:90-147).
   attention_fp8_emulated         PARITY UNPINNED: no reference counterpart (BASELINE
-                                 configs[4]); it restates the fp8 kernel's rounding points
-                                 and reference-point rule, and is held only to e4m3_round
+                                 configs[4]); it restates the fp8 kernel's rounding points,
+                                 reference-point rule and, for power-of-two scales, its
+                                 exponential-free softmax, and is held only to e4m3_round
                                  and to the cosine bar against `attention`.
 """
 from __future__ import annotations
@@ -438,7 +439,7 @@ def quant_e4m3(x, premul: float = 1.0, pow2_scale: bool = False):
 
 
 def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: float = 3.0, p_trig: float = 448.0,
-                           rows_per_wave: int = 32, pow2_scales: bool = False):
+                           rows_per_wave: int = 32, pow2_scales: bool = False, code_softmax=None):
   """Emulation of the fp8 kernel's arithmetic (no reference counterpart).
 
   Q, K, V quantised per tensor; logits from the quantised operands in f32; online softmax per
@@ -452,6 +453,11 @@ def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: f
   stay in e4m3's normal range.  The result does not depend on `ref` except through the e4m3
   rounding.  q [H,Sq,D], k/v [H,Skv,D].  pow2_scales: q is quantised with scale * log2(e) folded in and with a
   power-of-two scale, k with a power-of-two scale (the operands of the kernel's path without a multiply per logit).
+  code_softmax (default: as pow2_scales, which is when the kernel does it): P is not exp2 but the e4m3 number whose
+  byte is round(8 (logit - ref) + 56), clipped at 0: a piecewise-linear exponential, exact at the powers of two and
+  up to 6 % above between them; the row sum is taken over these P; the lse is lowered by the log of their mean ratio
+  to the exponential (log2 1.0404 = 0.0570814).  The reference moves (to tile max - p_offset) on the first tile and
+  whenever some byte of some row of the wave would pass 126, e4m3's last finite code.
   """
   log2e = np.float32(np.log2(np.e))
   if pow2_scales:
@@ -463,6 +469,12 @@ def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: f
   v8, sv = quant_e4m3(v)
   H, Sq, D = q8.shape
   Skv = k8.shape[1]
+  if code_softmax is None:
+    code_softmax = pow2_scales
+  if code_softmax:
+    if not pow2_scales:
+      raise ValueError("the code softmax needs power-of-two scales")
+    return _attention_fp8_code_softmax(q8, k8, v8, np.float32(sq * sk), sv, kv_tile, p_offset, rows_per_wave)
   ref = np.full((H, Sq), -1e30, np.float32)
   l = np.zeros((H, Sq), np.float32)
   o = np.zeros((H, Sq, D), np.float32)
@@ -487,3 +499,51 @@ def attention_fp8_emulated(q, k, v, scale: float, kv_tile: int = 64, p_offset: f
     l = a * l + p.sum(axis=-1)
     o = a[..., None] * o + np.einsum("hqk,hkd->hqd", e4m3_round(p), v8[:, t0:t0 + kv_tile])
   return o * sv / l[..., None], (ref + np.log2(l)) * np.float32(np.log(2.0))
+
+def _e4m3_decode(code):
+  """Value of the non-negative e4m3 byte `code` (0..126), f32."""
+  code = np.asarray(code, np.int32)
+  e, m = code >> 3, code & 7
+  return np.where(e > 0, np.ldexp(1.0 + m / 8.0, e - 7), np.ldexp(m / 8.0, -6)).astype(np.float32)
+
+
+def _attention_fp8_code_softmax(q8, k8, v8, c, sv, kv_tile, p_offset, rows_per_wave):
+  H, Sq, D = q8.shape
+  Skv = k8.shape[1]
+  ref = np.zeros((H, Sq), np.float32)
+  l = np.zeros((H, Sq), np.float32)
+  o = np.zeros((H, Sq, D), np.float32)
+  nw = -(-Sq // rows_per_wave)
+  c8 = np.float32(8.0) * np.float32(c)
+  q64, k64 = q8.astype(np.float64), k8.astype(np.float64)
+  half = D // 2
+
+  def code_logits(s_lo, s_hi, ref):
+    # as the two chained MFMAs form them: f32(start + first half of d), then f32(that + second half)
+    start = (np.float32(56.0) - np.float32(8.0) * ref).astype(np.float32)[..., None]
+    x1 = (start.astype(np.float64) + s_lo * float(c8)).astype(np.float32)
+    return (x1.astype(np.float64) + s_hi * float(c8)).astype(np.float32)
+
+  for it, t0 in enumerate(range(0, Skv, kv_tile)):
+    s_lo = np.einsum("hqd,hkd->hqk", q64[..., :half], k64[:, t0:t0 + kv_tile, :half])
+    s_hi = np.einsum("hqd,hkd->hqk", q64[..., half:], k64[:, t0:t0 + kv_tile, half:])
+    xp = code_logits(s_lo, s_hi, ref)
+    row_trig = np.rint(xp).max(axis=-1) >= 127.0
+    wt = np.zeros((H, nw * rows_per_wave), bool)
+    wt[:, :Sq] = row_trig
+    wave_trig = np.repeat(wt.reshape(H, nw, rows_per_wave).any(axis=-1), rows_per_wave, axis=1)[:, :Sq]
+    mx = (xp.max(axis=-1) - np.float32(56.0)) * np.float32(0.125)  # tile max relative to the old reference, log2 units
+    if it == 0:
+      dm = mx - np.float32(p_offset)
+      a = np.zeros_like(l)
+    else:
+      dm = np.where(wave_trig, np.maximum(mx - np.float32(p_offset), np.float32(0.0)), np.float32(0.0)).astype(np.float32)
+      a = np.exp2(-dm).astype(np.float32)
+    ref = (ref + dm).astype(np.float32)
+    xp = code_logits(s_lo, s_hi, ref)
+    p = _e4m3_decode(np.clip(np.rint(xp), 0, 126))
+    l = a * l + p.sum(axis=-1, dtype=np.float32)
+    o = a[..., None] * o + np.einsum("hqk,hkd->hqd", p, v8[:, t0:t0 + kv_tile])
+  lse = (ref + np.log2(l) - np.float32(0.0570814)) * np.float32(np.log(2.0))
+  return o * sv / l[..., None], lse
+

@@ -393,6 +393,29 @@ def test_fp8_emulation_meets_cosine_bar():
   assert np.abs(l8 - lse).max() < 0.1
   x8, s = O.quant_e4m3(q)
   assert np.abs(x8).max() == 448.0 and abs(s - np.abs(q).max() / 448.0) < 1e-9
+  # power-of-two scales: with exp2, and with the exponential-free softmax (P from the e4m3 byte grid)
+  oe, le = O.attention_fp8_emulated(q, k, v, 128**-0.5, pow2_scales=True, code_softmax=False)
+  oc, lc = O.attention_fp8_emulated(q, k, v, 128**-0.5, pow2_scales=True)
+  for o_, l_ in ((oe, le), (oc, lc)):
+    assert (o_.ravel() @ exact.ravel()) / (np.linalg.norm(o_) * np.linalg.norm(exact)) >= 0.995
+    assert np.abs(l_ - lse).max() < 0.1
+  assert np.abs(lc - le).max() < 0.08 and abs(float(np.mean(lc - le))) < 0.01  # the constant correction centres it
+
+
+def test_code_softmax_byte_grid():
+  """The byte of P~ is round(8 x + 56): exact at the powers of two, never below 0.957 nor above 1.108 of 2^x, mean
+  ratio over a binade 1.0404 (the constant the lse is corrected by)."""
+  x = np.linspace(-3.0, 5.0, 800001)
+  code = np.clip(np.rint(8 * x + 56), 0, 126)
+  val = O.dit_attention._e4m3_decode(code).astype(np.float64)
+  # the decode agrees with torch's float8_e4m3fn
+  bytes_ = torch.arange(0, 127, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+  np.testing.assert_array_equal(O.dit_attention._e4m3_decode(np.arange(127)), bytes_)
+  r = val / 2.0**x
+  assert 0.957 < r.min() and r.max() < 1.108
+  assert abs(np.log2(r.mean()) - 0.0570814) < 2e-4
+  for n in range(-3, 6):
+    assert O.dit_attention._e4m3_decode(np.rint(8 * n + 56)) == 2.0**n
 
 
 # ----------------------------------------------------------------------------- workloads
