@@ -110,7 +110,8 @@ def hip_flash_fp8_kernel(q, k, v, context):
   heads = context["heads"]
   qv, kv, vv = (_as_bshd(t, heads).to(torch.bfloat16).contiguous() for t in (q, k, v))
   # the softmax scale rides on q's quantisation (one rounding either way) and the q and k scales are powers of two:
-  # the kernel then applies the whole logit scale inside its MFMAs
+  # the kernel then applies the whole logit scale inside its MFMAs and forms P without exponentials (P's e4m3 byte
+  # straight from the logit: a piecewise-linear exponential within e4m3's own rounding noise)
   q8, sq = ops.quant_e4m3(qv, premul=context["scale"] * math.log2(math.e), pow2_scale=True)
   k8, sk = ops.quant_e4m3(kv, pow2_scale=True)
   v8, sv = ops.quant_e4m3(vv)
