@@ -11,6 +11,7 @@ struct MergeArgs {
   const float* lse_cur;
   int H, S;
   int64_t rows;  // B*H*S
+  int h_fast;    // rows are walked with the head index fastest (what [B,S,H,D] storage wants) instead of the token index
   int64_t r_sb, r_ss, r_sh, c_sb, c_ss, c_sh;
 };
 
@@ -21,11 +22,21 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
   const int tid = threadIdx.x, lane = tid % LPR;
   const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + tid / LPR;
   if (row >= a.rows) return;
-  const int s = (int)(row % a.S);
-  const int64_t bh = row / a.S;
-  const int h = (int)(bh % a.H);
-  const int64_t b = bh / a.H;
-  const float l1 = a.lse_run[row], l2 = a.lse_cur[row];
+  int s, h;
+  int64_t b;
+  if (a.h_fast) {  // consecutive rows of a workgroup are consecutive in memory
+    h = (int)(row % a.H);
+    const int64_t bs = row / a.H;
+    s = (int)(bs % a.S);
+    b = bs / a.S;
+  } else {
+    s = (int)(row % a.S);
+    const int64_t bh = row / a.S;
+    h = (int)(bh % a.H);
+    b = bh / a.H;
+  }
+  const int64_t lidx = (b * a.H + h) * a.S + s;
+  const float l1 = a.lse_run[lidx], l2 = a.lse_cur[lidx];
   float4* pr = reinterpret_cast<float4*>(a.o_run + b * a.r_sb + s * a.r_ss + h * a.r_sh) + 2 * lane;
   float4 r0 = pr[0], r1 = pr[1];
   float cur[8];
@@ -46,7 +57,7 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
   r0.x = w1 * r0.x + w2 * cur[0]; r0.y = w1 * r0.y + w2 * cur[1]; r0.z = w1 * r0.z + w2 * cur[2]; r0.w = w1 * r0.w + w2 * cur[3];
   r1.x = w1 * r1.x + w2 * cur[4]; r1.y = w1 * r1.y + w2 * cur[5]; r1.z = w1 * r1.z + w2 * cur[6]; r1.w = w1 * r1.w + w2 * cur[7];
   pr[0] = r0; pr[1] = r1;
-  if (lane == 0) a.lse_run[row] = den > 0.f ? L + logf(den) : L;
+  if (lane == 0) a.lse_run[lidx] = den > 0.f ? L + logf(den) : L;
 }
 
 __global__ __launch_bounds__(256) void finalize_kernel(const float4* __restrict__ in, uint4* __restrict__ out, int64_t n8) {
@@ -141,6 +152,7 @@ extern "C" int mdattn_merge(void* stream, float* o_run, float* lse_run, const vo
   MergeArgs a;
   a.o_run = o_run; a.lse_run = lse_run; a.o_cur = o_cur; a.lse_cur = lse_cur;
   a.H = H; a.S = S; a.rows = (int64_t)B * H * S;
+  a.h_fast = run_strides->head < run_strides->seq;
   a.r_sb = run_strides->batch; a.r_ss = run_strides->seq; a.r_sh = run_strides->head;
   a.c_sb = cur_strides->batch; a.c_ss = cur_strides->seq; a.c_sh = cur_strides->head;
   const int lpr = D / 8;
