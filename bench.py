@@ -249,7 +249,7 @@ def main():
       "dtype": "fp8-e4m3" if fp8 else "bf16",
       "data": "synthetic",
       "config": {"workload": f"{args.workload}: B=1 H={H} D={D} Sq={S} Skv={Skv * ring} norm={w.norm} rope={w.rope}"
-                             + (f" ring_chunks={ring} (merge per chunk)" if ring > 1 else ""),
+                             + (f" ring_chunks={ring} ({'attention and merge launched separately' if args.separate_merge else 'merged in the attention launch'})" if ring > 1 else ""),
                  "step": "fused q/k RMSNorm+RoPE -> " + ("per-tensor e4m3 quantisation of q, k, v -> fp8 flash-attention forward with LSE"
                                                              if fp8 else "bf16 flash-attention forward with LSE (softmax scale * log2 e carried by the prologue's q output)")},
       "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
