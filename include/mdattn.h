@@ -31,7 +31,8 @@ enum {
   MDATTN_E_BADARG = -1,      /* null pointer, non-positive size, inconsistent shape   */
   MDATTN_E_UNSUPPORTED = -2, /* well-formed request this build has no kernel for      */
   MDATTN_E_ALIGN = -3,       /* pointer or stride not aligned as the kernels require  */
-  MDATTN_E_LAUNCH = -4       /* the HIP runtime rejected the launch                   */
+  MDATTN_E_LAUNCH = -4,      /* the HIP runtime rejected the launch                   */
+  MDATTN_E_TOOBIG = -5       /* larger than the static scratch of a no-allocation entry point */
 };
 
 /* Element strides of one rank-4 tensor [batch, seq, head, dim] with dim contiguous. */
@@ -203,6 +204,25 @@ int mdattn_bwd_bf16(void* stream, const void* q, const void* k, const void* v, c
                     int B, int H, int Sq, int Skv, int D,
                     const mdattn_strides* q_strides, const mdattn_strides* k_strides,
                     const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale);
+
+/*
+ * mdattn_bwd_bf16 for callers that cannot allocate device memory and have no workspace to hand over: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+ * Same arguments and results as mdattn_bwd_bf16 without `workspace`: the lse / delta scratch lives in a device array
+ * that is part of the library image (MDATTN_BWD_STATIC_MAX_FLOATS floats = 32 MiB, held by every GPU the library runs
+ * on until the process ends).  Requests with mdattn_bwd_workspace_floats(B,H,Sq) above that limit (more than
+ * 4,194,304 padded query rows over all batches and heads) return MDATTN_E_TOOBIG and launch nothing.  The call
+ * allocates nothing and frees nothing.  All calls on one GPU share the array: calls that may overlap on one GPU (two
+ * streams, two threads) race on it and must be serialised by the caller; calls on different GPUs are independent.
+ * The device that `stream` belongs to must be the current device.
+ */
+#define MDATTN_BWD_STATIC_MAX_FLOATS (8 * 1024 * 1024)
+int64_t mdattn_bwd_static_max_floats(void);
+int mdattn_bwd_bf16_static(void* stream, const void* q, const void* k, const void* v, const void* out, const void* dout,
+                           const float* lse, void* dq, void* dk, void* dv,
+                           int B, int H, int Sq, int Skv, int D,
+                           const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                           const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale);
 
 /*
  * In-place LSE-space merge of a normalised partial (o_cur, lse_cur) into the running

@@ -9,7 +9,7 @@ import os
 
 from .build import LIB_PATH
 
-E_OK, E_BADARG, E_UNSUPPORTED, E_ALIGN, E_LAUNCH = 0, -1, -2, -3, -4
+E_OK, E_BADARG, E_UNSUPPORTED, E_ALIGN, E_LAUNCH, E_TOOBIG = 0, -1, -2, -3, -4, -5
 
 
 class Strides(ctypes.Structure):
@@ -41,6 +41,8 @@ SIGNATURES = {
     "mdattn_key_mask_bias": ([_P, _P, _P, _I, _I, _L, _F], _I),
     "mdattn_bwd_workspace_floats": ([_I, _I, _I], _L),
     "mdattn_bwd_bf16": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),
+    "mdattn_bwd_static_max_floats": ([], _L),
+    "mdattn_bwd_bf16_static": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),
     "mdattn_quant_e4m3": ([_P, _P, _P, _P, _L, _F, _I], _I),
     "mdattn_fwd_fp8": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F, _P, _P, _P], _I),
     "mdattn_merge": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S], _I),

@@ -16,6 +16,9 @@
 // lse and delta belong to the q rows: per-lane scalars for dq, sixteen values per lane and tile for dk / dv, read
 // from a workspace that a small kernel fills first (delta, lse in log2 units, both padded to a multiple of 32 rows
 // with lse = +inf so that padded q rows get p = 0).
+#include <atomic>
+#include <mutex>
+
 #include "mdattn_common.h"
 
 namespace mdattn {
@@ -269,11 +272,12 @@ extern "C" int64_t mdattn_bwd_workspace_floats(int B, int H, int Sq) {
   return 2 * (int64_t)B * H * (((int64_t)Sq + 31) / 32 * 32);
 }
 
-extern "C" int mdattn_bwd_bf16(void* stream, const void* q, const void* k, const void* v, const void* out, const void* dout,
-                               const float* lse, void* dq, void* dk, void* dv, float* workspace, int64_t workspace_floats,
-                               int B, int H, int Sq, int Skv, int D,
-                               const mdattn_strides* q_strides, const mdattn_strides* k_strides,
-                               const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
+// Shared body of mdattn_bwd_bf16 and mdattn_bwd_bf16_static: validation, the preparation kernel and the three passes.
+static int bwd_run(hipStream_t st, const void* q, const void* k, const void* v, const void* out, const void* dout,
+                   const float* lse, void* dq, void* dk, void* dv, float* workspace, int64_t workspace_floats,
+                   int B, int H, int Sq, int Skv, int D,
+                   const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                   const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
   if (!q || !k || !v || !out || !dout || !lse || !dq || !dk || !dv || !workspace) return MDATTN_E_BADARG;
   if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return MDATTN_E_BADARG;
   if (!q_strides || !k_strides || !v_strides || !o_strides) return MDATTN_E_BADARG;
@@ -287,7 +291,6 @@ extern "C" int mdattn_bwd_bf16(void* stream, const void* q, const void* k, const
     return MDATTN_E_ALIGN;
   if (q_strides->seq < D || k_strides->seq < D || v_strides->seq < D || o_strides->seq < D) return MDATTN_E_BADARG;
 
-  hipStream_t st = (hipStream_t)stream;
   const int Sp = (Sq + 31) / 32 * 32;
   float* lse2 = workspace;
   float* delta = workspace + (int64_t)B * H * Sp;
@@ -322,4 +325,64 @@ extern "C" int mdattn_bwd_bf16(void* stream, const void* q, const void* k, const
   set(a.s3_sb, a.s3_ss, a.s3_sh, o_strides);
   set(a.o_sb, a.o_ss, a.o_sh, v_strides);
   return launch_bwd<2>(st, a, B);
+}
+
+
+extern "C" int mdattn_bwd_bf16(void* stream, const void* q, const void* k, const void* v, const void* out, const void* dout,
+                               const float* lse, void* dq, void* dk, void* dv, float* workspace, int64_t workspace_floats,
+                               int B, int H, int Sq, int Skv, int D,
+                               const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                               const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
+  return bwd_run((hipStream_t)stream, q, k, v, out, dout, lse, dq, dk, dv, workspace, workspace_floats, B, H, Sq, Skv, D,
+                 q_strides, k_strides, v_strides, o_strides, scale);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// mdattn_bwd_bf16_static: the same backward for callers that cannot allocate (HIP graph capture, serving loops that
+// forbid hipMalloc).  The workspace (lse in log2 units and delta, one float each per padded query row) lives in a
+// file-scope device array instead of a caller's buffer.  Every GPU holds its own copy of the array at its own
+// address: that address is looked up once per device with hipGetSymbolAddress and kept; host code never uses the
+// array's name as a pointer.  bwd_prep_kernel writes every element the passes read, so nothing has to be cleared
+// between calls; calls that overlap on one GPU share the array and race.
+static __device__ __align__(256) float scratch[MDATTN_BWD_STATIC_MAX_FLOATS];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+std::atomic<float*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up on the first call per device), or nullptr.
+float* scratch_on_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  float* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+  if (p) return p;
+  void* sym = nullptr;
+  if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || !sym) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  p = static_cast<float*>(sym);
+  g_scratch_ptr[dev].store(p, std::memory_order_release);
+  return p;
+}
+}  // namespace
+
+extern "C" int64_t mdattn_bwd_static_max_floats(void) { return MDATTN_BWD_STATIC_MAX_FLOATS; }
+
+extern "C" int mdattn_bwd_bf16_static(void* stream, const void* q, const void* k, const void* v, const void* out,
+                                      const void* dout, const float* lse, void* dq, void* dk, void* dv,
+                                      int B, int H, int Sq, int Skv, int D,
+                                      const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                                      const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
+  if (B <= 0 || H <= 0 || Sq <= 0) return MDATTN_E_BADARG;
+  const int64_t need = mdattn_bwd_workspace_floats(B, H, Sq);
+  if (need > (int64_t)MDATTN_BWD_STATIC_MAX_FLOATS) return MDATTN_E_TOOBIG;
+  float* ws = scratch_on_current_device();
+  if (!ws) return MDATTN_E_LAUNCH;
+  return bwd_run((hipStream_t)stream, q, k, v, out, dout, lse, dq, dk, dv, ws, need, B, H, Sq, Skv, D,
+                 q_strides, k_strides, v_strides, o_strides, scale);
 }

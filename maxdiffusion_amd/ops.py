@@ -16,7 +16,7 @@ from . import _lib
 from ._lib import Strides
 
 __all__ = [
-    "norm_rope_fullrow", "norm_rope_perhead", "norm_rope_rows", "flash_attention", "flash_attention_backward", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
+    "norm_rope_fullrow", "norm_rope_perhead", "norm_rope_rows", "flash_attention", "flash_attention_backward", "flash_attention_backward_static", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
     "merge_partial", "flash_attention_merge", "finalize", "new_merge_state", "LSE_INIT", "FOLDED_SCALE", "folded_q_mul",
 ]
 
@@ -224,6 +224,31 @@ def flash_attention_backward(q, k, v, out, dout, lse, scale: float | None = None
       _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), nws,
       b, h, sq, skv, d, ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale))
   _lib.check(rc, "mdattn_bwd_bf16")
+  return dq, dk, dv
+
+
+def flash_attention_backward_static(q, k, v, out, dout, lse, dq, dk, dv, scale: float | None = None):
+  """`flash_attention_backward` into caller-provided dq, dk, dv (strides of q, k, v) through the entry point that
+  allocates nothing: its lse / delta scratch is a static device array of the library (32 MiB per GPU), so the call can
+  sit in code that must not allocate (HIP graph capture).  Raises MdattnError (code E_TOOBIG) when B*H*ceil32(Sq)
+  exceeds 4,194,304 rows.  Calls that overlap on one GPU share the scratch and race."""
+  _check_dev(q, k, v, out, dout, lse, dq, dk, dv)
+  if not all(t.dtype == torch.bfloat16 for t in (q, k, v, out, dout, dq, dk, dv)):
+    raise ValueError("flash_attention_backward_static needs bf16 tensors")
+  b, sq, h, d = q.shape
+  if out.shape != q.shape or dout.shape != q.shape or k.shape != v.shape or tuple(lse.shape) != (b, h, sq) or not lse.is_contiguous():
+    raise ValueError("inconsistent shapes")
+  if dout.stride() != out.stride() or dq.stride() != q.stride() or dk.stride() != k.stride() or dv.stride() != v.stride():
+    raise ValueError("dout must share out's strides and dq, dk, dv those of q, k, v")
+  if dq.shape != q.shape or dk.shape != k.shape or dv.shape != v.shape:
+    raise ValueError("dq, dk, dv must be shaped like q, k, v")
+  if scale is None:
+    scale = 1.0 / math.sqrt(d)
+  sq_, sk_, sv_, so_ = _strides(q), _strides(k), _strides(v), _strides(out)
+  rc = _lib.load().mdattn_bwd_bf16_static(
+      _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv),
+      b, h, sq, k.shape[1], d, ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale))
+  _lib.check(rc, "mdattn_bwd_bf16_static")
   return dq, dk, dv
 
 

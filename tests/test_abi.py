@@ -20,7 +20,7 @@ def test_header_declares_the_expected_entry_points():
   assert declared_symbols() == sorted([
       "mdattn_version", "mdattn_strerror", "mdattn_norm_rope_fullrow", "mdattn_norm_rope_perhead", "mdattn_fwd_bf16",
       "mdattn_quant_e4m3", "mdattn_fwd_fp8", "mdattn_merge", "mdattn_finalize", "mdattn_fwd_bf16_bias", "mdattn_key_mask_bias", "mdattn_norm_rope_rows", "mdattn_bwd_bf16", "mdattn_bwd_workspace_floats",
-      "mdattn_fwd_bf16_merge",
+      "mdattn_fwd_bf16_merge", "mdattn_bwd_bf16_static", "mdattn_bwd_static_max_floats",
   ])
 
 
@@ -37,7 +37,7 @@ def test_version_and_strerror(lib):
   text = open(HEADER).read()
   want = int(re.search(r"#define MDATTN_VERSION (\d+)", text).group(1))
   assert lib.mdattn_version() == want
-  for code in (0, -1, -2, -3, -4, -99):
+  for code in (0, -1, -2, -3, -4, -5, -99):
     assert len(lib.mdattn_strerror(code)) > 0
   assert lib.mdattn_strerror(0) == b"ok"
 
