@@ -44,6 +44,22 @@ typedef struct mdattn_strides {
 
 int mdattn_version(void);
 const char* mdattn_strerror(int code);
+/* Hash of the sources and compiler flags the library was built from (the build script passes it in): lets the
+ * host side refuse a library that was not built from the sources next to it. */
+const char* mdattn_build_id(void);
+
+/*
+ * Test and tuning hook, no counterpart in the reference: forces the schedule that mdattn_fwd_bf16 and
+ * mdattn_fwd_bf16_merge use at head dim 128, for the whole process, until set again.  0 restores the choice by shape.
+ * Returns the previous value (>= 0) or MDATTN_E_BADARG.  The parity tests use it to run every schedule on every shape;
+ * nothing else should: it is the one piece of mutable state in the library, read once per call.
+ */
+#define MDATTN_FWD_SCHEDULE_AUTO 0
+#define MDATTN_FWD_SCHEDULE_PIPELINED8 1 /* 8 waves x 32 rows, software-pipelined, 64-key tiles */
+#define MDATTN_FWD_SCHEDULE_PIPELINED4 2 /* 4 waves x 32 rows, same loop                        */
+#define MDATTN_FWD_SCHEDULE_FLAT 3       /* 4 waves x 32 rows, 32-key tiles, 3 workgroups per CU */
+#define MDATTN_FWD_SCHEDULE_LAST 3
+int mdattn_set_fwd_schedule(int schedule);
 
 /*
  * Fused RMSNorm over the FULL inner dimension H*D + 3-axis RoPE, for q and k in one pass.
@@ -158,8 +174,8 @@ int mdattn_key_mask_bias(void* stream, const void* keep, float* bias, int B, int
  *   pow2_scale   non-zero: the scale is rounded up to a power of two (e4m3 is a floating-point format: no
  *                precision is lost, at most one binade of range).  With power-of-two q and k scales and the
  *                softmax scale carried by premul, mdattn_fwd_fp8 applies the whole logit scale through the
- *                MFMA's block-scale operand, saves its multiply per logit and forms P without exponentials
- *                (see mdattn_fwd_fp8).
+ *                MFMA's block-scale operand, saves its multiply per logit and can form P without exponentials
+ *                (see mdattn_fwd_fp8's softmax_mode).
  *   scale_out f32[2] device: [0] = s with x * premul ~= x_fp8 * s (absmax(x * premul) / 448, or the next
  *                power of two), [1] = absmax(x) (scratch of the reduction)
  * n % 16 == 0.
@@ -175,18 +191,23 @@ int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, float* scal
  * scale = ln 2 here) the logit scale is applied inside the MFMAs and the softmax needs no multiply; the scales are
  * read on the device, so nothing has to be declared: two instances of the kernel are launched and the one whose
  * case it is not returns at once.
- * In that power-of-two case P is formed without exponentials: the e4m3 byte of a probability is the integer
- * round(8 * (log2-logit - reference) + 56), i.e. P is a piecewise-linear exponential, exact at the powers of two and
- * up to 6 % above them in between (comparable to e4m3's own rounding); the row sum is taken over those P, so out is a
- * properly normalised average, and lse is corrected by the mean of the difference (log2 1.0404) and so exact to
- * about +-0.08 for a row that a single key dominates, much closer otherwise.  With any other scales P = e4m3(exp2(.))
- * and the lse is that of the quantised logits.
+ *   softmax_mode  MDATTN_FP8_SOFTMAX_EXP2: P = e4m3(exp2(.)), the row sum over the unrounded P; lse is the exact
+ *                 logsumexp of the quantised logits (usable as a partial for mdattn_merge).
+ *                 MDATTN_FP8_SOFTMAX_BYTE_GRID: in the power-of-two case only (otherwise as EXP2), P is formed without
+ *                 exponentials: the e4m3 byte of a probability is the integer round(8 * (log2-logit - reference) + 56),
+ *                 i.e. P is a piecewise-linear exponential, exact at the powers of two and up to 6 % above them in
+ *                 between (comparable to e4m3's own rounding); the row sum is taken over those P, so out is a properly
+ *                 normalised average, and lse is corrected by the mean of the difference (log2 1.0404): within 0.08 of
+ *                 the EXP2 lse for a row that a single key dominates, much closer otherwise.  12 % faster; meant for
+ *                 callers that use `out` only.
  */
+#define MDATTN_FP8_SOFTMAX_EXP2 0
+#define MDATTN_FP8_SOFTMAX_BYTE_GRID 1
 int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, const void* v8, void* out, float* lse,
                    int B, int H, int Sq, int Skv, int D,
                    const mdattn_strides* q_strides, const mdattn_strides* k_strides,
                    const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
-                   const float* q_scale, const float* k_scale, const float* v_scale);
+                   const float* q_scale, const float* k_scale, const float* v_scale, int softmax_mode);
 
 /*
  * Backward of mdattn_fwd_bf16: dq, dk, dv from (q, k, v, out, dout, lse), non-causal, no mask.  Replaces: the

@@ -33,6 +33,8 @@ _S = ctypes.POINTER(Strides)
 SIGNATURES = {
     "mdattn_version": ([], _I),
     "mdattn_strerror": ([_I], ctypes.c_char_p),
+    "mdattn_build_id": ([], ctypes.c_char_p),
+    "mdattn_set_fwd_schedule": ([_I], _I),
     "mdattn_norm_rope_fullrow": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _L, _L, _S], _I),
     "mdattn_norm_rope_perhead": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _F, _F, _S, _S], _I),
     "mdattn_norm_rope_rows": ([_P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _L, _L, _S], _I),
@@ -44,7 +46,7 @@ SIGNATURES = {
     "mdattn_bwd_static_max_floats": ([], _L),
     "mdattn_bwd_bf16_static": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),
     "mdattn_quant_e4m3": ([_P, _P, _P, _P, _L, _F, _I], _I),
-    "mdattn_fwd_fp8": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F, _P, _P, _P], _I),
+    "mdattn_fwd_fp8": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F, _P, _P, _P, _I], _I),
     "mdattn_merge": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S], _I),
     "mdattn_fwd_bf16_merge": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),
     "mdattn_finalize": ([_P, _P, _P, _L], _I),
@@ -66,6 +68,12 @@ def load() -> ctypes.CDLL:
       fn = getattr(lib, name)
       fn.argtypes = argtypes
       fn.restype = restype
+    from . import build
+
+    if os.path.isdir(build.CSRC) and lib.mdattn_build_id().decode() != build.source_id():
+      raise RuntimeError(
+          f"{LIB_PATH} was built from other sources than the ones in {build.CSRC} (build id "
+          f"{lib.mdattn_build_id().decode()}, sources {build.source_id()}): rebuild with `python -m maxdiffusion_amd.build`")
     _lib = lib
   return _lib
 

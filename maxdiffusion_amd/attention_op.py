@@ -96,6 +96,9 @@ def hip_flash_kernel(q, k, v, context):
   # [B,Skv] keep-mask (attention_flax.py:1926-1939): masked keys are excluded, as the flash wrappers do with
   # segment ids (:390-438); rows without a kept key return 0 (:1552-1554)
   mask = context.get("attention_mask")
+  if mask is not None and tuple(mask.shape) != (qv.shape[0], kv.shape[1]):
+    # the reference's additive bias would fail to broadcast against the [B,H,Sq,Skv] scores (:1550)
+    raise ValueError(f"attention_mask must have shape [batch, kv_length] = {(qv.shape[0], kv.shape[1])}, got {tuple(mask.shape)}.")
   bias = ops.key_mask_bias(mask) if mask is not None else None
   out = ops.flash_attention(qv, kv, vv, scale=context["scale"], key_bias=bias)
   b, s, h, d = out.shape
@@ -110,12 +113,13 @@ def hip_flash_fp8_kernel(q, k, v, context):
   heads = context["heads"]
   qv, kv, vv = (_as_bshd(t, heads).to(torch.bfloat16).contiguous() for t in (q, k, v))
   # the softmax scale rides on q's quantisation (one rounding either way) and the q and k scales are powers of two:
-  # the kernel then applies the whole logit scale inside its MFMAs and forms P without exponentials (P's e4m3 byte
-  # straight from the logit: a piecewise-linear exponential within e4m3's own rounding noise)
+  # the kernel then applies the whole logit scale inside its MFMAs; the registry entry returns `out` only, so it asks
+  # for the softmax without exponentials (P's e4m3 byte straight from the logit: a piecewise-linear exponential
+  # within e4m3's own rounding noise).  Callers that need an lse to merge use ops.flash_attention_fp8(softmax="exp2").
   q8, sq = ops.quant_e4m3(qv, premul=context["scale"] * math.log2(math.e), pow2_scale=True)
   k8, sk = ops.quant_e4m3(kv, pow2_scale=True)
   v8, sv = ops.quant_e4m3(vv)
-  out = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=ops.FOLDED_SCALE)
+  out = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=ops.FOLDED_SCALE, softmax="byte_grid")
   b, s, h, d = out.shape
   return out.reshape(b, s, h * d).to(q.dtype)
 

@@ -26,6 +26,9 @@ HIPCC_FLAGS = [
     # instead of bouncing through AGPRs with v_accvgpr_read/write
     "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
+    # the direct global->LDS loads are inline assembly that writes M0 and lists it as clobbered; clang remarks that
+    # M0 is a reserved register.  The statement really does overwrite it, so the compiler is told.
+    "-Wno-inline-asm",
 ]
 
 
@@ -80,10 +83,46 @@ def _demangled(names: list[str]) -> dict[str, str]:
   return dict(zip(names, out)) if len(out) == len(names) else {n: n for n in names}
 
 
+def source_id() -> str:
+  """Hash of everything libmdattn.so is compiled from (sources, headers, flags); compiled into the library as
+  mdattn_build_id() so that a library built from other sources than the ones beside it is recognised."""
+  import hashlib
+
+  h = hashlib.sha256(" ".join(HIPCC_FLAGS).encode())
+  files = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC)) if f.endswith((".hip", ".h"))]
+  for path in files + [os.path.join(INCLUDE, "mdattn.h")]:
+    h.update(os.path.basename(path).encode())
+    with open(path, "rb") as f:
+      h.update(f.read())
+  return h.hexdigest()[:16]
+
+
+def library_is_current() -> bool:
+  """True when libmdattn.so exists and was built from the sources in this tree."""
+  if not os.path.exists(LIB_PATH):
+    return False
+  import ctypes
+
+  try:
+    fn = ctypes.CDLL(LIB_PATH).mdattn_build_id
+  except (OSError, AttributeError):
+    return False
+  fn.restype = ctypes.c_char_p
+  return fn().decode() == source_id()
+
+
+def ensure_built(verbose: bool = True) -> str:
+  """What tests, smoke() and bench.py call: loads what is built, builds only when nothing is built or the library
+  was compiled from other sources than the ones in the tree."""
+  if not library_is_current():
+    build_library(verbose)
+  return LIB_PATH
+
+
 def build_library(verbose: bool = True) -> str:
   """Compile every HIP source into maxdiffusion_amd/libmdattn.so.  Always recompiles."""
-  cmd = [_hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", f"-I{INCLUDE}", f"-I{CSRC}", "-o", LIB_PATH,
-         *[os.path.join(CSRC, s) for s in SOURCES]]
+  cmd = [_hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", f'-DMDATTN_BUILD_ID="{source_id()}"',
+         f"-I{INCLUDE}", f"-I{CSRC}", "-o", LIB_PATH, *[os.path.join(CSRC, s) for s in SOURCES]]
   if verbose:
     print("[maxdiffusion_amd.build]", " ".join(cmd), flush=True)
   r = subprocess.run(cmd, capture_output=True, text=True)
@@ -96,7 +135,7 @@ def build_library(verbose: bool = True) -> str:
     rows = _resource_table(r.stderr)
     names = _demangled([n for n, _ in rows])
     for n, d in rows:
-      short = names[n].split("(")[0].replace("void ", "").replace("mdattn::", "").replace("(anonymous namespace)::", "")
+      short = names[n].replace("(anonymous namespace)::", "").split("(")[0].replace("void ", "").replace("mdattn::", "")
       spill = "  <-- spills" if d.get("ScratchSize", 0) else ""
       print(f"[maxdiffusion_amd.build]   {short:<46} vgpr {d.get('VGPRs', 0):>3} agpr {d.get('AGPRs', 0):>3} "
             f"scratch {d.get('ScratchSize', 0):>3} B  lds {d.get('LDS', 0):>6} B  waves/SIMD {d.get('Occupancy', 0)}{spill}", flush=True)

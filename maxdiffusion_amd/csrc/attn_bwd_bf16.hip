@@ -256,8 +256,8 @@ int launch_bwd(hipStream_t st, BwdArgs a, int B) {
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
   auto kern = attn_bwd_kernel<MODE>;
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-    return MDATTN_E_LAUNCH;
+  static LdsOptIn opted;
+  if (lds_opt_in(opted, reinterpret_cast<const void*>(kern), lds_bytes) != MDATTN_OK) return MDATTN_E_LAUNCH;
   hipLaunchKernelGGL(kern, dim3(a.chunk * 8), dim3(256), lds_bytes, st, a);
   return launch_status();
 }

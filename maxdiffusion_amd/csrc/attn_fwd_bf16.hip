@@ -34,8 +34,6 @@
 //   grid       = 1-D, remapped so that each XCD (workgroup id mod 8) walks a contiguous range of
 //                (head, q-tile) pairs: the workgroups resident on one XCD stream the same K/V and
 //                share it through that XCD's L2.
-#include <stdlib.h>
-
 #include <type_traits>
 
 #include "mdattn_common.h"
@@ -635,8 +633,8 @@ static int launch_fwd(hipStream_t st, AttnArgs a, int B) {
   // scale * log2(e) == 1 (to f32 round-off): the caller folded the factor into q; the logits need no multiply
   const bool pre = a.c > 1.0f - 1e-6f && a.c < 1.0f + 1e-6f;
   auto kern = pre ? attn_fwd_bf16_kernel<NW, true> : attn_fwd_bf16_kernel<NW, false>;
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-    return MDATTN_E_LAUNCH;
+  static LdsOptIn opted[2];
+  if (lds_opt_in(opted[pre], reinterpret_cast<const void*>(kern), lds_bytes) != MDATTN_OK) return MDATTN_E_LAUNCH;
   hipLaunchKernelGGL(kern, dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   return launch_status();
 }
@@ -679,9 +677,8 @@ static int dispatch_fwd(hipStream_t st, const AttnArgs& a, int B, int Sq, int Sk
   // on long key sequences; its prologue and epilogue (three tiles of look-ahead, one virtual block at each end)
   // weigh on short ones, where the flat kernel (4 waves x 32 rows, three workgroups per CU) wins: measured
   // cross-over between 2048 and 4608 keys.  The flat kernel also yields twice the workgroups on tiny grids.
-  // MDATTN_FWD_VARIANT (1: pipelined 8 waves, 2: pipelined 4 waves, 3: flat) overrides the choice.
-  int variant = 0;
-  if (const char* e = getenv("MDATTN_FWD_VARIANT")) variant = atoi(e);
+  // mdattn_set_fwd_schedule (1: pipelined 8 waves, 2: pipelined 4 waves, 3: flat) overrides the choice, for tests.
+  int variant = forced_fwd_schedule();
   if (variant == 0) {
     const int64_t wg256 = (int64_t)B * a.H * ((Sq + 255) / 256);
     variant = (Skv <= 3072 || wg256 < 128) ? 3 : 1;

@@ -22,8 +22,6 @@
 //                padding (128 B rows); its 8-byte chunks are XOR-swizzled by row bits 1 and 3, which
 //                makes the 8 rows x 32 B a half-wave reads hit 64 distinct banks.
 //   epilogue     O * v_scale / l, bf16; lse = ln2 * (reference + log2 l).
-#include <stdlib.h>
-
 #include <type_traits>
 
 #include "mdattn_common.h"
@@ -354,7 +352,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
 }
 
 template <int NW>
-int launch_fwd8(hipStream_t st, Fp8Args a, int B) {
+int launch_fwd8(hipStream_t st, Fp8Args a, int B, int softmax_mode) {
   constexpr int BM = NW * 32;
   constexpr int lds_bytes = kSlots8 * kStage8;
   a.nqt = (a.Sq + BM - 1) / BM;
@@ -363,10 +361,12 @@ int launch_fwd8(hipStream_t st, Fp8Args a, int B) {
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
   hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 0>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
-  // Power-of-two logit scale: the exponential-free softmax; MDATTN_FP8_SOFTMAX=1 keeps exp2 there too (experiments).
-  const char* e = getenv("MDATTN_FP8_SOFTMAX");
-  if (e && atoi(e) == 1) hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 1>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
-  else hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 2>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  // Power-of-two logit scale (the instance above then returns at once, this one otherwise): exp2, or the
+  // exponential-free softmax when the caller asked for it.
+  if (softmax_mode == MDATTN_FP8_SOFTMAX_BYTE_GRID)
+    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 2>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  else
+    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 1>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   return launch_status();
 }
 
@@ -379,7 +379,8 @@ extern "C" int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, cons
                               int B, int H, int Sq, int Skv, int D,
                               const mdattn_strides* q_strides, const mdattn_strides* k_strides,
                               const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
-                              const float* q_scale, const float* k_scale, const float* v_scale) {
+                              const float* q_scale, const float* k_scale, const float* v_scale, int softmax_mode) {
+  if (softmax_mode != MDATTN_FP8_SOFTMAX_EXP2 && softmax_mode != MDATTN_FP8_SOFTMAX_BYTE_GRID) return MDATTN_E_BADARG;
   if (!q8 || !k8 || !v8 || !out || !q_scale || !k_scale || !v_scale) return MDATTN_E_BADARG;
   if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return MDATTN_E_BADARG;
   if (!q_strides || !k_strides || !v_strides || !o_strides) return MDATTN_E_BADARG;
@@ -407,13 +408,6 @@ extern "C" int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, cons
   a.c = scale * kLog2e;
   if (a.c > 1.0f - 1e-6f && a.c < 1.0f + 1e-6f) a.c = 1.0f;  // scale = ln 2: the caller's q carries the softmax scale
   hipStream_t st = (hipStream_t)stream;
-  // Four waves per workgroup (three workgroups per CU) measured faster than eight at every shape tried;
-  // MDATTN_FP8_VARIANT (1: 8 waves, 2: 4 waves per workgroup) overrides the choice for experiments.
-  int variant = 2;
-  if (const char* e = getenv("MDATTN_FP8_VARIANT")) variant = atoi(e);
-  switch (variant) {
-    case 1: return launch_fwd8<8>(st, a, B);
-    case 2: return launch_fwd8<4>(st, a, B);
-    default: return MDATTN_E_BADARG;
-  }
+  // Four waves per workgroup (three workgroups per CU) measured faster than eight at every shape tried.
+  return launch_fwd8<4>(st, a, B, softmax_mode);
 }

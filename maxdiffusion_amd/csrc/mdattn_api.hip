@@ -1,6 +1,23 @@
 // Version / error-string entry points of the C ABI.
 #include "mdattn_common.h"
 
+namespace mdattn {
+namespace {
+std::atomic<int> g_fwd_schedule{0};
+}
+int forced_fwd_schedule() { return g_fwd_schedule.load(std::memory_order_relaxed); }
+}  // namespace mdattn
+
+extern "C" int mdattn_set_fwd_schedule(int schedule) {
+  if (schedule < 0 || schedule > MDATTN_FWD_SCHEDULE_LAST) return MDATTN_E_BADARG;
+  return mdattn::g_fwd_schedule.exchange(schedule, std::memory_order_relaxed);
+}
+
+#ifndef MDATTN_BUILD_ID
+#define MDATTN_BUILD_ID "unknown"
+#endif
+extern "C" const char* mdattn_build_id(void) { return MDATTN_BUILD_ID; }
+
 extern "C" int mdattn_version(void) { return MDATTN_VERSION; }
 
 extern "C" const char* mdattn_strerror(int code) {

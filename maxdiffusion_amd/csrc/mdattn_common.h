@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "mdattn.h"
 
 namespace mdattn {
@@ -80,13 +82,13 @@ __device__ __forceinline__ void st_nt(uint4* p, const uint4& u) {
 // Direct global -> LDS load of 16 bytes per lane: lane i's bytes land at lds_addr + 16*i (the LDS base
 // travels in M0).  Written as inline assembly so that the loads stay asynchronous: the compiler cannot
 // tell which LDS bytes such a load writes and would otherwise wait for it before the next LDS read.
-// M0 is never live across statements in compiled code (the compiler sets it right before each use).
+// The statement writes M0 and says so, so the compiler never keeps a value of its own in M0 across it.
 // The kernels track these loads themselves with s_waitcnt vmcnt.
 __device__ __forceinline__ void lds_dma16(const void* base, unsigned byte_off, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(byte_off), "s"(base) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(byte_off), "s"(base) : "memory", "m0");
 }
 __device__ __forceinline__ void lds_dma16(const void* addr, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(addr) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(addr) : "memory", "m0");
 }
 __device__ __forceinline__ unsigned lds_addr_of(const void* p) {
   return (unsigned)(uintptr_t)(const void __attribute__((address_space(3)))*)p;
@@ -119,5 +121,23 @@ inline bool strides_ok(const mdattn_strides* s, int64_t mult) {
   return s && s->batch % mult == 0 && s->seq % mult == 0 && s->head % mult == 0 && s->seq > 0 && s->head > 0 && s->batch >= 0;
 }
 inline int launch_status() { return hipGetLastError() == hipSuccess ? MDATTN_OK : MDATTN_E_LAUNCH; }
+
+// A kernel that needs more dynamic LDS than the default limit has to opt in with hipFuncSetAttribute, once per
+// kernel and device: one LdsOptIn per kernel instance remembers the devices that have been told.
+struct LdsOptIn {
+  std::atomic<uint64_t> devices{0};
+};
+inline int lds_opt_in(LdsOptIn& flag, const void* kernel, int lds_bytes) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MDATTN_E_LAUNCH;
+  const uint64_t bit = 1ull << dev;
+  if (flag.devices.load(std::memory_order_acquire) & bit) return MDATTN_OK;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) return MDATTN_E_LAUNCH;
+  flag.devices.fetch_or(bit, std::memory_order_release);
+  return MDATTN_OK;
+}
+
+// Schedule forced by mdattn_set_fwd_schedule (0: chosen by shape).
+int forced_fwd_schedule();
 
 }  // namespace mdattn

@@ -17,10 +17,21 @@ from ._lib import Strides
 
 __all__ = [
     "norm_rope_fullrow", "norm_rope_perhead", "norm_rope_rows", "flash_attention", "flash_attention_backward", "flash_attention_backward_static", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
-    "merge_partial", "flash_attention_merge", "finalize", "new_merge_state", "LSE_INIT", "FOLDED_SCALE", "folded_q_mul",
+    "merge_partial", "flash_attention_merge", "finalize", "new_merge_state", "LSE_INIT", "FOLDED_SCALE", "folded_q_mul", "set_fwd_schedule", "FWD_SCHEDULES", "FP8_SOFTMAX_MODES",
 ]
 
 LSE_INIT = -1e30
+
+FWD_SCHEDULES = {"auto": 0, "pipelined8": 1, "pipelined4": 2, "flat": 3}
+
+
+def set_fwd_schedule(schedule) -> int:
+  """Test and tuning hook: forces the schedule of the bf16 forward at head dim 128 for the whole process ("auto"
+  restores the choice by shape).  Returns the previous setting."""
+  rc = _lib.load().mdattn_set_fwd_schedule(FWD_SCHEDULES.get(schedule, schedule))
+  if rc < 0:
+    _lib.check(rc, "mdattn_set_fwd_schedule")
+  return rc
 
 # Folding the softmax scale into the prologue: norm_rope_*(..., q_mul=folded_q_mul(D)) emits q * D^-1/2 * log2(e)
 # (still one rounding), and the attention entry points, given scale=FOLDED_SCALE = ln 2, see scale * log2(e) == 1:
@@ -188,6 +199,10 @@ def flash_attention(q, k, v, scale: float | None = None, return_lse: bool = Fals
     _check_dev(key_bias)
     if key_bias.dtype != torch.float32 or key_bias.dim() != 2 or key_bias.shape[0] != b or key_bias.stride(1) != 1:
       raise ValueError("key_bias must be an f32 [batch, padded kv_length] tensor with a contiguous last axis")
+    if key_bias.shape[1] != (skv + 31) // 32 * 32:
+      # a shorter bias whose padding still covers Skv would silently exclude the trailing keys
+      raise ValueError(f"key_bias must have kv_length rounded up to 32 = {(skv + 31) // 32 * 32} columns (padding filled with "
+                       f"the masked value), got {key_bias.shape[1]}")
     rc = _lib.load().mdattn_fwd_bf16_bias(
         _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), b, h, sq, skv, d,
         ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale),
@@ -206,10 +221,8 @@ def flash_attention_backward(q, k, v, out, dout, lse, scale: float | None = None
   skv = k.shape[1]
   if out.shape != q.shape or dout.shape != q.shape or k.shape != v.shape or tuple(lse.shape) != (b, h, sq):
     raise ValueError("inconsistent shapes")
-  if dout.stride() != out.stride():
-    dout = dout.contiguous() if out.is_contiguous() else dout.clone(memory_format=torch.preserve_format).as_strided(out.shape, out.stride())
-  if dout.stride() != out.stride():
-    raise ValueError("out and dout must share strides")
+  if dout.stride() != out.stride():  # the kernels walk out and dout with one set of strides: re-lay dout like out
+    dout = torch.empty_strided(out.shape, out.stride(), dtype=dout.dtype, device=dout.device).copy_(dout)
   if scale is None:
     scale = 1.0 / math.sqrt(d)
   lse = lse.contiguous()
@@ -268,9 +281,19 @@ def quant_e4m3(x: torch.Tensor, premul: float = 1.0, pow2_scale: bool = False):
   return x8, scale
 
 
+FP8_SOFTMAX_MODES = {"exp2": 0, "byte_grid": 1}
+
+
 def flash_attention_fp8(q8, k8, v8, q_scale, k_scale, v_scale, scale: float | None = None, return_lse: bool = False,
-                        out_layout: str = "bshd"):
-  """fp8-e4m3 variant: q8/k8/v8 uint8 logical [B,S,H,D] views, *_scale device f32 tensors (element 0 is used)."""
+                        out_layout: str = "bshd", softmax: str = "exp2"):
+  """fp8-e4m3 variant: q8/k8/v8 uint8 logical [B,S,H,D] views, *_scale device f32 tensors (element 0 is used).
+
+  softmax="exp2": exact exponentials; the lse is the logsumexp of the quantised logits and the pair (out, lse) can be
+  merged like a bf16 partial.  softmax="byte_grid": with power-of-two q and k scales and the softmax scale carried by
+  q (see `quant_e4m3`) P is a piecewise-linear exponential read off the e4m3 byte grid (12 % faster; out keeps its
+  accuracy, the lse is only good to about 0.08); with any other scales it is the same as "exp2"."""
+  if softmax not in FP8_SOFTMAX_MODES:
+    raise ValueError(f"softmax={softmax!r} not supported. Choose between 'exp2' and 'byte_grid'.")
   _check_dev(q8, k8, v8, q_scale, k_scale, v_scale)
   b, sq, h, d = q8.shape
   skv = k8.shape[1]
@@ -282,7 +305,7 @@ def flash_attention_fp8(q8, k8, v8, q_scale, k_scale, v_scale, scale: float | No
   rc = _lib.load().mdattn_fwd_fp8(
       _stream(), _ptr(q8), _ptr(k8), _ptr(v8), _ptr(out), _ptr(lse), b, h, sq, skv, d,
       ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale),
-      _ptr(q_scale), _ptr(k_scale), _ptr(v_scale))
+      _ptr(q_scale), _ptr(k_scale), _ptr(v_scale), FP8_SOFTMAX_MODES[softmax])
   _lib.check(rc, "mdattn_fwd_fp8")
   return (out, lse) if return_lse else out
 

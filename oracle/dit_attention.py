@@ -27,16 +27,21 @@ Pinning status of each function (what fixes it besides its own formula):
   attention_bwd                  torch autograd through torch SDPA (fp64, CPU), finite differences
   merge_lse / merge_mlo /        attention over a union of KV chunks equals the
   merge_scan_ring                merge of per-chunk results (brute force)
-  attention_dot_product_bf16     PARITY UNPINNED at bit level: the rounding points
-                                 of XLA-CPU's bf16 einsum/softmax are not fixed by
-                                 any reference test; it is pinned only to tolerance
-                                 (2e-2) against `attention`, like the reference's
-                                 own tests do (tests/attention_test.py:90-147).
-  attention_fp8_emulated         PARITY UNPINNED: no reference counterpart (BASELINE
-                                 configs[4]); it restates the fp8 kernel's rounding points,
-                                 reference-point rule and, for power-of-two scales, its
-                                 exponential-free softmax, and is held only to e4m3_round
-                                 and to the cosine bar against `attention`.
+  attention_dot_product_bf16     torch's CPU bf16 kernels (matmul with bf16 result, bf16 scale multiply,
+                                 softmax, matmul) on the same inputs: >= 99.5 % of the outputs bit-identical,
+                                 the rest one bf16 step of one probability apart, while moving any single
+                                 rounding point or the scale drops the agreement below 85 %; and inputs on
+                                 which every rounding is exact (uniform and one-hot probabilities), where it
+                                 equals `attention` bit for bit.  (What XLA-CPU does inside einsum / softmax
+                                 is fixed by no reference test or fixture; the flow restated is the one the
+                                 source's dtypes prescribe, attention_flax.py:1546-1564.)
+  attention_fp8_emulated         no reference counterpart (BASELINE configs[4]).  Pinned by a scalar brute-force
+                                 loop over rows, tiles and keys with torch.float8_e4m3fn casts (both scale
+                                 kinds, both softmax forms, profiles that move the reference points), and by
+                                 what the mathematics fixes: with exp2 the lse equals the f64 lse of the
+                                 de-quantised q and k, and out equals f64 attention on the de-quantised
+                                 operands up to e4m3's rounding of P; the byte-grid softmax within 0.08 of
+                                 that lse.
 """
 from __future__ import annotations
 

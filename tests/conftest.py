@@ -34,11 +34,10 @@ def pytest_collection_modifyitems(config, items):
 
 @pytest.fixture(scope="session")
 def lib():
-  """The built C-ABI library; built once here only if nothing is built yet."""
+  """The built C-ABI library; built here only if nothing is built yet or what is built comes from other sources."""
   from maxdiffusion_amd import _lib, build
 
-  if not os.path.exists(build.LIB_PATH):
-    build.build_library()
+  build.ensure_built()
   return _lib.load()
 
 

@@ -21,6 +21,7 @@ def test_header_declares_the_expected_entry_points():
       "mdattn_version", "mdattn_strerror", "mdattn_norm_rope_fullrow", "mdattn_norm_rope_perhead", "mdattn_fwd_bf16",
       "mdattn_quant_e4m3", "mdattn_fwd_fp8", "mdattn_merge", "mdattn_finalize", "mdattn_fwd_bf16_bias", "mdattn_key_mask_bias", "mdattn_norm_rope_rows", "mdattn_bwd_bf16", "mdattn_bwd_workspace_floats",
       "mdattn_fwd_bf16_merge", "mdattn_bwd_bf16_static", "mdattn_bwd_static_max_floats",
+      "mdattn_build_id", "mdattn_set_fwd_schedule",
   ])
 
 
@@ -40,6 +41,25 @@ def test_version_and_strerror(lib):
   for code in (0, -1, -2, -3, -4, -5, -99):
     assert len(lib.mdattn_strerror(code)) > 0
   assert lib.mdattn_strerror(0) == b"ok"
+
+
+def test_build_id_and_schedule_hook(lib):
+  from maxdiffusion_amd import _lib, build
+
+  assert lib.mdattn_build_id().decode() == build.source_id()  # the library in the tree was built from the tree
+  assert lib.mdattn_set_fwd_schedule(3) == 0 and lib.mdattn_set_fwd_schedule(0) == 3
+  assert lib.mdattn_set_fwd_schedule(99) == _lib.E_BADARG and lib.mdattn_set_fwd_schedule(-1) == _lib.E_BADARG
+  assert lib.mdattn_set_fwd_schedule(0) == 0
+
+
+def test_stale_library_is_refused(monkeypatch):
+  from maxdiffusion_amd import _lib, build
+
+  monkeypatch.setattr(_lib, "_lib", None)
+  monkeypatch.setattr(build, "source_id", lambda: "0123456789abcdef")
+  with pytest.raises(RuntimeError, match="built from other sources"):
+    _lib.load()
+  assert not build.library_is_current()
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

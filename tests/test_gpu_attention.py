@@ -4,7 +4,6 @@ Bars (BASELINE north star): out max-abs <= 2e-2 and mean-abs <= 2e-3 against an 
 LSE within 1e-3.  With N(0,1) inputs |out| is ~1e-2, so those absolute bars alone would pass an
 all-zero output: every case also checks the relative L2 error, and sharpened inputs are included."""
 import math
-import os
 
 import numpy as np
 import pytest
@@ -30,20 +29,9 @@ def _check(out, lse, ref_o, ref_l, what, lse_abs=LSE_ABS):
 
 @pytest.fixture
 def variant():
-  """Lets a test force one of the kernel's tile variants; restores automatic choice afterwards."""
-  old = os.environ.get("MDATTN_FWD_VARIANT")
-
-  def force(v):
-    if v:
-      os.environ["MDATTN_FWD_VARIANT"] = str(v)
-    else:
-      os.environ.pop("MDATTN_FWD_VARIANT", None)
-
-  yield force
-  if old is None:
-    os.environ.pop("MDATTN_FWD_VARIANT", None)
-  else:
-    os.environ["MDATTN_FWD_VARIANT"] = old
+  """Lets a test force one of the kernel's schedules (mdattn_set_fwd_schedule); restores the choice by shape afterwards."""
+  yield lambda v: ops.set_fwd_schedule(int(v or 0))
+  ops.set_fwd_schedule(0)
 
 
 def _run_np(q, k, v, dev, **kw):
@@ -183,14 +171,28 @@ def _wan14b_inputs(dev, sq, skv, seed):
   return mk(sq), mk(skv), mk(skv)
 
 
-def test_wan14b_self_attention_full_size(dev):
+@pytest.mark.parametrize("folded", [False, True])
+def test_wan14b_self_attention_full_size(dev, folded):
   """Config 2 at full size (75 600 tokens, 40 heads): CPU oracle on a deterministic sample of rows of
   every head (tile boundaries and the ragged tail included) + the whole tensor against a plain torch
-  f32 reference computed on the GPU."""
+  f32 reference computed on the GPU.  folded: the path the benchmark times -- the prologue kernel emits
+  q * D^-1/2 * log2(e) and the attention kernel is given scale = ln 2, which selects its instance without a
+  multiply per logit; the references see the prologue's bf16 output and scale = ln 2."""
   w = O.WORKLOADS["wan14b"]
-  S = w.seq
-  q, k, v = _wan14b_inputs(dev, S, S, 0)
-  out, lse = ops.flash_attention(q, k, v, scale=w.scale, return_lse=True)
+  S, H, D = w.seq, w.heads, 128
+  if folded:
+    gen = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda: torch.randn((1, S, H * D), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    q_in, k_in, v = mk(), mk(), mk().view(1, S, H, D)
+    cos, sin = (torch.from_numpy(t).to(dev) for t in O.wan_rope_table(w.grid, D))
+    q, k = ops.norm_rope_fullrow(q_in, k_in, to_dev_bf16(O.norm_weight(H * D, 3), dev), to_dev_bf16(O.norm_weight(H * D, 4), dev),
+                                 cos, sin, H, q_mul=ops.folded_q_mul(D, w.scale))
+    scale = ops.FOLDED_SCALE
+    del q_in, k_in
+  else:
+    q, k, v = _wan14b_inputs(dev, S, S, 0)
+    scale = w.scale
+  out, lse = ops.flash_attention(q, k, v, scale=scale, return_lse=True)
   torch.cuda.synchronize()
   rows = O.sample_rows(S, n_random=48)
   idx = torch.from_numpy(rows).to(dev)
@@ -198,14 +200,15 @@ def test_wan14b_self_attention_full_size(dev):
   kc, vc = k[0].float().cpu().numpy(), v[0].float().cpu().numpy()
   worst = [0.0, 0.0, 0.0, 0.0]
   for h in range(w.heads):
-    ro, rl = O.attention_rows(qs[:, h], kc[:, h], vc[:, h], w.scale, dtype=np.float32)
+    ro, rl = O.attention_rows(qs[:, h], kc[:, h], vc[:, h], scale, dtype=np.float32)
     mx, mean = err_stats(os_[:, h], ro)
     worst = [max(worst[0], mx), max(worst[1], mean), max(worst[2], rel_l2(os_[:, h], ro)), max(worst[3], float(np.abs(ls[h] - rl).max()))]
-  print(f"wan14b sampled rows ({len(rows)} x 40 heads): max-abs {worst[0]:.3e} mean-abs {worst[1]:.3e} rel-l2 {worst[2]:.3e} lse {worst[3]:.3e}", flush=True)
+  print(f"wan14b{' (scale carried by the prologue)' if folded else ''} sampled rows ({len(rows)} x 40 heads): max-abs {worst[0]:.3e} "
+        f"mean-abs {worst[1]:.3e} rel-l2 {worst[2]:.3e} lse {worst[3]:.3e}", flush=True)
   assert worst[0] <= MAX_ABS and worst[1] <= MEAN_ABS and worst[2] <= REL_L2 and worst[3] <= LSE_ABS
   # whole tensor, 8 heads at a time to bound the f32 score buffer
   for h0 in range(0, 40, 8):
-    ro, rl = torch_attention_f32(q[:, :, h0:h0 + 8], k[:, :, h0:h0 + 8], v[:, :, h0:h0 + 8], w.scale, q_block=1024)
+    ro, rl = torch_attention_f32(q[:, :, h0:h0 + 8], k[:, :, h0:h0 + 8], v[:, :, h0:h0 + 8], scale, q_block=1024)
     d = (out[:, :, h0:h0 + 8].float() - ro).abs()
     assert float(d.max()) <= MAX_ABS and float(d.mean()) <= MEAN_ABS
     assert float((lse[:, h0:h0 + 8] - rl).abs().max()) <= LSE_ABS
@@ -235,6 +238,16 @@ def test_host_side_validation_raises(dev):
     ops.flash_attention(q, q[:, :, :1], q[:, :, :1])
   from maxdiffusion_amd._lib import MdattnError
 
+  # a key bias that is shorter than the padded key count would silently drop the trailing keys
+  q60 = torch.zeros((1, 60, 2, 128), dtype=torch.bfloat16, device=dev)
+  with pytest.raises(ValueError, match="rounded up to 32"):
+    ops.flash_attention(q, q60, q60, key_bias=torch.zeros((1, 32), device=dev))
+  from maxdiffusion_amd import attention_op
+
+  op = attention_op.AttentionOp(attention_kernel="hip_flash", heads=2, dim_head=128, scale=0.1)
+  with pytest.raises(ValueError, match=r"attention_mask must have shape \[batch, kv_length\]"):
+    op.apply_attention(q.reshape(1, 8, 256), q60.reshape(1, 60, 256), q60.reshape(1, 60, 256),
+                       attention_mask=torch.ones((1, 40), dtype=torch.bool, device=dev))
   q32 = torch.zeros((1, 8, 2, 32), dtype=torch.bfloat16, device=dev)  # head dims other than 128 and 64
   with pytest.raises(MdattnError, match="unsupported"):
     ops.flash_attention(q32, q32, q32)

@@ -65,6 +65,21 @@ def test_backward_layout_scale_and_sharp_logits(dev):
     _check(hsd(dv), rv, f"dv {layout} sharp")
 
 
+def test_backward_accepts_dout_in_another_layout_than_out(dev):
+  """out stored [B,H,S,D], dout contiguous [B,S,H,D] (what autograd hands over): the wrapper has to re-lay dout like
+  out, element by element."""
+  H, sq, skv = 3, 130, 200
+  q, k, v, do = (O.normal_bf16((1, s_, H, 128), i) for i, s_ in enumerate((sq, skv, skv, sq)))
+  qd, kd, vd, dod = (to_dev_bf16(x, dev) for x in (q, k, v, do))
+  out, lse = ops.flash_attention(qd, kd, vd, return_lse=True, out_layout="bhsd")
+  assert out.stride() != dod.stride()
+  dq, dk, dv = ops.flash_attention_backward(qd, kd, vd, out, dod, lse)
+  rq, rk, rv = O.attention_bwd(hsd(q), hsd(k), hsd(v), hsd(do), 128**-0.5)
+  _check(hsd(to_np(dq)), rq, "dq, dout bshd / out bhsd")
+  _check(hsd(to_np(dk)), rk, "dk, dout bshd / out bhsd")
+  _check(hsd(to_np(dv)), rv, "dv, dout bshd / out bhsd")
+
+
 def test_backward_wan13b_shape_against_torch_autograd_on_gpu(dev):
   """configs[0] size (12 heads x 4680 tokens): whole tensors against torch's f32 autograd (test harness only)."""
   w = O.WORKLOADS["wan1.3b"]

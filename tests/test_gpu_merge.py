@@ -68,11 +68,11 @@ def test_ring_replay_small_unequal_chunks(dev):
 
 @pytest.mark.parametrize("layout", ["bshd", "bhsd"])
 @pytest.mark.parametrize("variant", [0, 1, 3])
-def test_fused_ring_step_equals_attention_then_merge(dev, monkeypatch, layout, variant):
+def test_fused_ring_step_equals_attention_then_merge(dev, request, layout, variant):
   """mdattn_fwd_bf16_merge (attention + merge in the attention kernel's epilogue) against the two separate calls
   and against the oracle, with ragged chunks, through both schedules and both layouts of the carry."""
-  if variant:
-    monkeypatch.setenv("MDATTN_FWD_VARIANT", str(variant))
+  ops.set_fwd_schedule(variant)
+  request.addfinalizer(lambda: ops.set_fwd_schedule(0))
   H, Sq = 3, 333
   q = O.normal_bf16((1, Sq, H, 128), 0)
   sizes = [4200, 1, 63, 777, 3100]
@@ -140,5 +140,39 @@ def test_wan14b_ring_shard_replay_full_size(dev):
   idx = torch.from_numpy(rows).to(dev)
   for h in (0, 21, 39):  # CPU oracle on sampled rows
     co, cl = O.attention_rows(to_np(q[0, idx, h]), to_np(k[0, :, h]), to_np(v[0, :, h]), w.scale)
+    assert err_stats(to_np(merged[0, idx, h]), co)[0] <= 2e-2 and rel_l2(to_np(merged[0, idx, h]), co) <= 1.5e-2
+    assert err_stats(to_np(l_run[0, h, idx]), cl)[0] <= 1e-3
+
+
+def test_wan14b_ring_shard_fused_hops_full_size(dev):
+  """Config 3 the way the benchmark runs it: the prologue carries the softmax scale (q * D^-1/2 * log2 e, kernel
+  given scale = ln 2) and each of the 8 hops is ONE launch of mdattn_fwd_bf16_merge (attention and merge in the
+  attention kernel's epilogue).  The merged result must equal the one-pass attention over all 75 600 keys, the torch
+  f32 reference on the whole chunk and the CPU oracle on sampled rows."""
+  w = O.WORKLOADS["wan14b-ring"]
+  C, n, H, D = w.seq, w.ring_chunks, w.heads, 128
+  gen = torch.Generator(device=dev).manual_seed(3)
+  mk = lambda s: torch.randn((1, s, H, D), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+  q = (mk(C).float() * ops.folded_q_mul(D, w.scale)).to(torch.bfloat16)  # what the prologue hands over
+  k, v = mk(C * n), mk(C * n)
+  sc = ops.FOLDED_SCALE
+  o_run, l_run = ops.new_merge_state(1, C, H, D, dev)
+  for i in range(n):
+    ops.flash_attention_merge(q, k[:, i * C:(i + 1) * C], v[:, i * C:(i + 1) * C], o_run, l_run, scale=sc)
+  merged = ops.finalize(o_run)
+  full, full_l = ops.flash_attention(q, k, v, scale=sc, return_lse=True)  # one pass over all 75 600 keys
+  d_o, d_l = float((merged.float() - full.float()).abs().max()), float((l_run - full_l).abs().max())
+  print(f"fused ring hops vs one pass: out {d_o:.3e} lse {d_l:.3e}", flush=True)
+  assert d_o < 2e-3 and d_l < 1e-4
+  for h0 in range(0, H, 8):
+    ro, rl = torch_attention_f32(q[:, :, h0:h0 + 8], k[:, :, h0:h0 + 8], v[:, :, h0:h0 + 8], sc, q_block=1024)
+    d = (merged[:, :, h0:h0 + 8].float() - ro).abs()
+    assert float(d.max()) <= 2e-2 and float(d.mean()) <= 2e-3
+    assert float((merged[:, :, h0:h0 + 8].float() - ro).norm() / ro.norm()) <= 1.5e-2
+    assert float((l_run[:, h0:h0 + 8] - rl).abs().max()) <= 1e-3
+  rows = O.sample_rows(C, n_random=24)
+  idx = torch.from_numpy(rows).to(dev)
+  for h in (0, 21, 39):
+    co, cl = O.attention_rows(to_np(q[0, idx, h]), to_np(k[0, :, h]), to_np(v[0, :, h]), sc)
     assert err_stats(to_np(merged[0, idx, h]), co)[0] <= 2e-2 and rel_l2(to_np(merged[0, idx, h]), co) <= 1.5e-2
     assert err_stats(to_np(l_run[0, h, idx]), cl)[0] <= 1e-3
