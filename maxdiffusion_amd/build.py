@@ -16,7 +16,9 @@ INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "libmdattn.so")
 FFI_LIB_PATH = os.path.join(PKG_DIR, "libmdattn_ffi.so")
 
-SOURCES = ["mdattn_api.hip", "norm_rope.hip", "attn_fwd_bf16.hip", "attn_fwd_fp8.hip", "attn_bwd_bf16.hip", "merge_quant.hip"]
+SOURCES = ["mdattn_api.hip", "norm_rope.hip", "attn_fwd_bf16.hip", "attn_fwd_fp8.hip", "attn_bwd_bf16.hip", "merge_quant.hip",
+           # the bodies of the XLA custom-call handlers on plain structs (no XLA header): part of the library
+           os.path.join("ffi", "mdattn_marshal.cc")]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32 out of scalar float code.
 HIPCC_FLAGS = [
@@ -90,7 +92,7 @@ def source_id() -> str:
 
   h = hashlib.sha256(" ".join(HIPCC_FLAGS).encode())
   files = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC)) if f.endswith((".hip", ".h"))]
-  for path in files + [os.path.join(INCLUDE, "mdattn.h")]:
+  for path in files + [os.path.join(CSRC, "ffi", "mdattn_marshal.cc"), os.path.join(INCLUDE, "mdattn.h"), os.path.join(INCLUDE, "mdattn_marshal.h")]:
     h.update(os.path.basename(path).encode())
     with open(path, "rb") as f:
       h.update(f.read())

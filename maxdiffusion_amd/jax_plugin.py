@@ -1,31 +1,46 @@
 """Registers the HIP kernels with a live maxdiffusion + JAX (ROCm) install.
 
 `install()` (1) registers the XLA-FFI targets exported by libmdattn_ffi.so with
-``jax.ffi.register_ffi_target(..., platform="ROCM")`` and (2) adds ``hip_flash`` to
+``jax.ffi.register_ffi_target(..., platform="ROCM")`` and (2) adds ``hip_flash`` and ``hip_flash_fp8`` to
 maxdiffusion's own KERNEL_REGISTRY (models/attention_flax.py:1589-1597), after which
 ``attention: hip_flash`` in any Wan / Flux / LTX config reaches the MI355X kernel through
 the unchanged `_apply_attention` (models/attention_flax.py:1965-1966).
 
-Nothing here runs at import time: jax, jaxlib's FFI headers and maxdiffusion are absent from
-the build image, so this module is exercised only where they exist.
+Every compute entry point of include/mdattn.h has one custom-call target here (FFI_TARGETS) and one wrapper below;
+the operands, results and attributes of each `jax.ffi.ffi_call` follow the bind line of the same target in
+csrc/ffi/mdattn_ffi.cc, in order.  Nothing here runs at import time: jax, jaxlib's FFI headers and maxdiffusion are
+absent from the build image, so this module is exercised with them only where they exist
+(tests/test_ffi_shim.py drives every wrapper through a recording stand-in for `jax.ffi`).
 """
 from __future__ import annotations
 
 import ctypes
+import math
 import os
 
 from .build import FFI_LIB_PATH, build_ffi_library
 
+# custom-call target (= the C-ABI entry point it ends in) -> handler symbol exported by libmdattn_ffi.so
 FFI_TARGETS = {
     "mdattn_fwd_bf16": "MdattnFwdBf16",
     "mdattn_fwd_bf16_bias": "MdattnFwdBf16Bias",
-    "mdattn_bwd_bf16": "MdattnBwdBf16",
+    "mdattn_key_mask_bias": "MdattnKeyMaskBias",
+    "mdattn_fwd_bf16_merge": "MdattnFwdBf16Merge",
+    "mdattn_merge": "MdattnMerge",
+    "mdattn_finalize": "MdattnFinalize",
     "mdattn_norm_rope_fullrow": "MdattnNormRopeFullrow",
     "mdattn_norm_rope_perhead": "MdattnNormRopePerhead",
     "mdattn_norm_rope_rows": "MdattnNormRopeRows",
-    "mdattn_merge": "MdattnMerge",
-    "mdattn_fwd_bf16_merge": "MdattnFwdBf16Merge",
+    "mdattn_quant_e4m3": "MdattnQuantE4m3",
+    "mdattn_fwd_fp8": "MdattnFwdFp8",
+    "mdattn_bwd_bf16": "MdattnBwdBf16",
+    "mdattn_bwd_bf16_static": "MdattnBwdBf16Static",
 }
+# entry points of mdattn.h that are host-side helpers, not kernels: no custom call
+HOST_ONLY = ("mdattn_version", "mdattn_strerror", "mdattn_build_id", "mdattn_set_fwd_schedule",
+             "mdattn_bwd_workspace_floats", "mdattn_bwd_static_max_floats")
+
+FOLDED_SCALE = math.log(2.0)  # see ops.FOLDED_SCALE: scale * log2(e) == 1, the softmax scale rides on q
 
 _installed = False
 
@@ -49,34 +64,78 @@ def register_ffi_targets():
     jax.ffi.register_ffi_target(target, jax.ffi.pycapsule(getattr(lib, symbol)), platform="ROCM")
 
 
+def _f32(x):
+  import numpy as np
+
+  return np.float32(x)
+
+
+def _i64(x):
+  import numpy as np
+
+  return np.int64(x)
+
+
+def _bshd_dims(x, layout: int):
+  if layout == 0:
+    b, s, h, d = x.shape
+  else:
+    b, h, s, d = x.shape
+  return b, s, h, d
+
+
+def hip_key_mask_bias(keep_mask, masked_value: float = -math.inf):
+  """[B,Skv] bool keep-mask -> additive key bias f32 [B, Skv rounded up to 32] (masked keys and the padding get
+  `masked_value`): the mask canonicalisation of models/attention_flax.py:1931-1939 for the flash-type kernels."""
+  jax, jnp = _require_jax()
+  if keep_mask.ndim != 2:
+    raise ValueError(f"attention_mask must have shape [batch, kv_length], got {tuple(keep_mask.shape)}.")
+  b, skv = keep_mask.shape
+  call = jax.ffi.ffi_call("mdattn_key_mask_bias", jax.ShapeDtypeStruct((b, (skv + 31) // 32 * 32), jnp.float32), vmap_method="sequential")
+  return call(keep_mask.astype(jnp.bool_), masked_value=_f32(masked_value))
+
+
 def hip_flash_attention(q, k, v, scale: float, layout: int, keep_mask=None):
   """q [B,Sq,H,D] (layout 0) or [B,H,Sq,D] (layout 1) bf16 -> (out [B,Sq,H,D] bf16, lse [B,H,Sq] f32).
 
-  keep_mask: optional [B,Skv] bool; masked keys are excluded (the bias is built with jnp: a [B,Skv] select)."""
+  keep_mask: optional [B,Skv] bool; masked keys are excluded, rows without a kept key return 0."""
   jax, jnp = _require_jax()
-  if layout == 0:
-    b, sq, h, d = q.shape
-  else:
-    b, h, sq, d = q.shape
-  call = jax.ffi.ffi_call(
-      "mdattn_fwd_bf16",
-      (jax.ShapeDtypeStruct((b, sq, h, d), jnp.bfloat16), jax.ShapeDtypeStruct((b, h, sq), jnp.float32)),
-      vmap_method="sequential",
-  )
-  import numpy as np
-
+  b, sq, h, d = _bshd_dims(q, layout)
+  results = (jax.ShapeDtypeStruct((b, sq, h, d), jnp.bfloat16), jax.ShapeDtypeStruct((b, h, sq), jnp.float32))
   if keep_mask is not None:
-    skv = k.shape[1] if layout == 0 else k.shape[2]
-    pad = (-skv) % 32
-    bias = jnp.where(keep_mask, 0.0, -jnp.inf).astype(jnp.float32)
-    bias = jnp.pad(bias, ((0, 0), (0, pad)), constant_values=-jnp.inf)
-    call = jax.ffi.ffi_call(
-        "mdattn_fwd_bf16_bias",
-        (jax.ShapeDtypeStruct((b, sq, h, d), jnp.bfloat16), jax.ShapeDtypeStruct((b, h, sq), jnp.float32)),
-        vmap_method="sequential",
-    )
-    return call(q, k, v, bias, scale=np.float32(scale), layout=np.int64(layout))
-  return call(q, k, v, scale=np.float32(scale), layout=np.int64(layout))
+    skv = _bshd_dims(k, layout)[1]
+    if tuple(keep_mask.shape) != (b, skv):
+      raise ValueError(f"attention_mask must have shape [batch, kv_length] = {(b, skv)}, got {tuple(keep_mask.shape)}.")
+    call = jax.ffi.ffi_call("mdattn_fwd_bf16_bias", results, vmap_method="sequential")
+    return call(q, k, v, hip_key_mask_bias(keep_mask), scale=_f32(scale), layout=_i64(layout))
+  call = jax.ffi.ffi_call("mdattn_fwd_bf16", results, vmap_method="sequential")
+  return call(q, k, v, scale=_f32(scale), layout=_i64(layout))
+
+
+def hip_quant_e4m3(x, premul: float = 1.0, pow2_scale: bool = False):
+  """Per-tensor absmax quantisation of a bf16 array -> (float8_e4m3fn array of the same shape, f32[2]: [0] the
+  de-quantisation scale of x * premul, [1] absmax(x))."""
+  jax, jnp = _require_jax()
+  call = jax.ffi.ffi_call("mdattn_quant_e4m3", (jax.ShapeDtypeStruct(x.shape, jnp.float8_e4m3fn), jax.ShapeDtypeStruct((2,), jnp.float32)),
+                          vmap_method="sequential")
+  return call(x.astype(jnp.bfloat16), premul=_f32(premul), pow2_scale=_i64(bool(pow2_scale)))
+
+
+def hip_flash_attention_fp8(q, k, v, scale: float, layout: int, softmax: str = "byte_grid"):
+  """BASELINE configs[4]: quantises bf16 q, k, v per tensor (q carries scale * log2(e), q and k scales are powers of
+  two) and runs the fp8-e4m3 kernel.  softmax "byte_grid" (fastest; use `out`) or "exp2" (exact lse, mergeable).
+  Returns (out [B,Sq,H,D] bf16, lse [B,H,Sq] f32)."""
+  jax, jnp = _require_jax()
+  modes = {"exp2": 0, "byte_grid": 1}
+  if softmax not in modes:
+    raise ValueError(f"softmax={softmax!r} not supported. Choose between 'exp2' and 'byte_grid'.")
+  b, sq, h, d = _bshd_dims(q, layout)
+  q8, qs = hip_quant_e4m3(q, premul=scale * math.log2(math.e), pow2_scale=True)
+  k8, ks = hip_quant_e4m3(k, pow2_scale=True)
+  v8, vs = hip_quant_e4m3(v)
+  call = jax.ffi.ffi_call("mdattn_fwd_fp8", (jax.ShapeDtypeStruct((b, sq, h, d), jnp.bfloat16), jax.ShapeDtypeStruct((b, h, sq), jnp.float32)),
+                          vmap_method="sequential")
+  return call(q8, k8, v8, qs, ks, vs, scale=_f32(FOLDED_SCALE), layout=_i64(layout), softmax_mode=_i64(modes[softmax]))
 
 
 def hip_ring_step(q, k_chunk, v_chunk, o_run, lse_run, scale: float, layout: int = 0):
@@ -84,22 +143,40 @@ def hip_ring_step(q, k_chunk, v_chunk, o_run, lse_run, scale: float, layout: int
   (o_run f32 [B,Sq,H,D], lse_run f32 [B,H,Sq]; start from zeros and -1e30).  The body of the scan step in
   kernels/splash_attention/ring_attention_kernel.py:1045-1073; the carry is donated and updated in place."""
   jax, jnp = _require_jax()
-  import numpy as np
-
   call = jax.ffi.ffi_call(
       "mdattn_fwd_bf16_merge",
       (jax.ShapeDtypeStruct(o_run.shape, jnp.float32), jax.ShapeDtypeStruct(lse_run.shape, jnp.float32)),
       input_output_aliases={3: 0, 4: 1},
       vmap_method="sequential",
   )
-  return call(q, k_chunk, v_chunk, o_run, lse_run, scale=np.float32(scale), layout=np.int64(layout))
+  return call(q, k_chunk, v_chunk, o_run, lse_run, scale=_f32(scale), layout=_i64(layout))
 
 
-def hip_flash_attention_vjp(q, k, v, scale: float):
-  """Differentiable attention on [B,S,H,D] bf16 arrays: jax.custom_vjp around the forward and backward custom calls
-  (what kernels/splash_attention/splash_attention_kernel.py:1277-1600 does for the Pallas kernel)."""
+def hip_merge(o_run, lse_run, o_cur, lse_cur):
+  """LSE-space merge of a normalised partial (o_cur bf16|f32 [B,S,H,D], lse_cur) into the donated carry
+  (kernels/splash_attention/ring_attention_kernel.py:1062-1073)."""
   jax, jnp = _require_jax()
-  import numpy as np
+  call = jax.ffi.ffi_call(
+      "mdattn_merge",
+      (jax.ShapeDtypeStruct(o_run.shape, jnp.float32), jax.ShapeDtypeStruct(lse_run.shape, jnp.float32)),
+      input_output_aliases={0: 0, 1: 1},
+      vmap_method="sequential",
+  )
+  return call(o_run, lse_run, o_cur, lse_cur)
+
+
+def hip_finalize(o_run):
+  """f32 carry -> bf16 (the `.astype(q.dtype)` of ring_attention_kernel.py:1130)."""
+  jax, jnp = _require_jax()
+  call = jax.ffi.ffi_call("mdattn_finalize", jax.ShapeDtypeStruct(o_run.shape, jnp.bfloat16), vmap_method="sequential")
+  return call(o_run)
+
+
+def hip_flash_attention_vjp(q, k, v, scale: float, static_scratch: bool = False):
+  """Differentiable attention on [B,S,H,D] bf16 arrays: jax.custom_vjp around the forward and backward custom calls
+  (what kernels/splash_attention/splash_attention_kernel.py:1277-1600 does for the Pallas kernel).  static_scratch:
+  the backward that needs no workspace result (its scratch is a static device array of the library)."""
+  jax, jnp = _require_jax()
 
   @jax.custom_vjp
   def attn(q, k, v):
@@ -112,14 +189,13 @@ def hip_flash_attention_vjp(q, k, v, scale: float):
   def bwd(res, dout):
     q, k, v, out, lse = res
     b, sq, h, d = q.shape
+    grads = (jax.ShapeDtypeStruct(q.shape, jnp.bfloat16), jax.ShapeDtypeStruct(k.shape, jnp.bfloat16), jax.ShapeDtypeStruct(v.shape, jnp.bfloat16))
+    if static_scratch:
+      call = jax.ffi.ffi_call("mdattn_bwd_bf16_static", grads, vmap_method="sequential")
+      return tuple(call(q, k, v, out, dout.astype(jnp.bfloat16), lse, scale=_f32(scale)))
     nws = 2 * b * h * ((sq + 31) // 32 * 32)  # mdattn_bwd_workspace_floats
-    call = jax.ffi.ffi_call(
-        "mdattn_bwd_bf16",
-        (jax.ShapeDtypeStruct(q.shape, jnp.bfloat16), jax.ShapeDtypeStruct(k.shape, jnp.bfloat16),
-         jax.ShapeDtypeStruct(v.shape, jnp.bfloat16), jax.ShapeDtypeStruct((nws,), jnp.float32)),
-        vmap_method="sequential",
-    )
-    dq, dk, dv, _ = call(q, k, v, out, dout.astype(jnp.bfloat16), lse, scale=np.float32(scale))
+    call = jax.ffi.ffi_call("mdattn_bwd_bf16", grads + (jax.ShapeDtypeStruct((nws,), jnp.float32),), vmap_method="sequential")
+    dq, dk, dv, _ = call(q, k, v, out, dout.astype(jnp.bfloat16), lse, scale=_f32(scale))
     return dq, dk, dv
 
   attn.defvjp(fwd, bwd)
@@ -127,36 +203,53 @@ def hip_flash_attention_vjp(q, k, v, scale: float):
 
 
 def hip_norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6, q_mul: float = 1.0):
-  """q, k [B,S,H*D] bf16; cos/sin f32 [S,D/2] or None -> (q_out, k_out) [B,S,H,D] bf16.  `q_mul` is multiplied into
-  q_out before its rounding: D**-0.5 * log2(e) here and scale = ln 2 in hip_flash_attention carry the softmax scale
-  in the prologue."""
+  """q, k [B,S,H*D] bf16 (k may be None: cached text K/V); cos/sin f32 [S,D/2] or None (norm only) -> (q_out, k_out)
+  [B,S,H,D] bf16.  `q_mul` is multiplied into q_out before its rounding: D**-0.5 * log2(e) here and scale = ln 2 in
+  hip_flash_attention carry the softmax scale in the prologue.  FlaxWanAttention.__call__, attention_flax.py:2655-2677."""
   jax, jnp = _require_jax()
-  import numpy as np
-
   b, s, n = q.shape
   d = n // heads
-  rope = cos is not None
-  if not rope:
-    cos = sin = jnp.zeros((1, 1), jnp.float32)
+  rope, has_k = cos is not None, k is not None
+  dummy = jnp.zeros((8,), jnp.float32)
   out = jax.ShapeDtypeStruct((b, s, heads, d), jnp.bfloat16)
-  call = jax.ffi.ffi_call("mdattn_norm_rope_fullrow", (out, out), vmap_method="sequential")
-  return call(q, k, wq, wk, cos, sin, eps=np.float32(eps), q_mul=np.float32(q_mul), heads=np.int64(heads), rope=np.int64(rope))
+  k_out = out if has_k else jax.ShapeDtypeStruct((8,), jnp.bfloat16)
+  call = jax.ffi.ffi_call("mdattn_norm_rope_fullrow", (out, k_out), vmap_method="sequential")
+  q_out, k_res = call(q, k if has_k else q, wq, wk if has_k else wq, cos if rope else dummy, sin if rope else dummy,
+                      eps=_f32(eps), q_mul=_f32(q_mul), heads=_i64(heads), rope=_i64(rope), has_k=_i64(has_k))
+  return q_out, (k_res if has_k else None)
+
+
+def hip_norm_rope_perhead(q, k, wq, wk, cos, sin, eps: float = 1e-6, wq_txt=None, wk_txt=None, n_txt: int = 0, q_mul: float = 1.0):
+  """q, k [B,S,H,D] bf16 (k may be None); per-head RMSNorm with weights [D]; tokens [0, n_txt) take wq_txt / wk_txt
+  (FlaxFluxAttention's encoder_*_norm on the text tokens of the joint sequence, attention_flax.py:3002-3003);
+  cos/sin f32 [S,D/2] or None -> (q_out, k_out) [B,S,H,D] bf16.  FlaxFluxAttention.__call__, :2989-3020."""
+  jax, jnp = _require_jax()
+  rope, has_k = cos is not None, k is not None
+  if n_txt and (wq_txt is None or (has_k and wk_txt is None)):
+    raise ValueError("n_txt > 0 needs the text-token norm weights wq_txt (and wk_txt with k)")
+  dummy = jnp.zeros((8,), jnp.float32)
+  out = jax.ShapeDtypeStruct(q.shape, jnp.bfloat16)
+  k_out = out if has_k else jax.ShapeDtypeStruct((8,), jnp.bfloat16)
+  call = jax.ffi.ffi_call("mdattn_norm_rope_perhead", (out, k_out), vmap_method="sequential")
+  q_out, k_res = call(q, k if has_k else q, wq, wk if has_k else wq, wq_txt if n_txt else wq, wk_txt if (n_txt and has_k) else wq,
+                      cos if rope else dummy, sin if rope else dummy,
+                      eps=_f32(eps), q_mul=_f32(q_mul), n_txt=_i64(n_txt), rope=_i64(rope), has_k=_i64(has_k))
+  return q_out, (k_res if has_k else None)
 
 
 def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotary_emb=None, k_rotary_emb=None,
-                       rope_type: str = "interleaved", is_self_attention: bool = True, eps: float = 1e-6):
+                       rope_type: str = "interleaved", is_self_attention: bool = True, eps: float = 1e-6, q_mul: float = 1.0):
   """Fused prologue of LTX2Attention.__call__ (models/ltx2/attention_ltx2.py:556-585): see attention_op.hip_norm_rope_ltx2.
-  query/key [B,S,H*D] -> bf16 [B,S,H,D]; tables (cos, sin) as LTX2RotaryPosEmbed returns them."""
+  query/key [B,S,H*D] -> bf16 [B,S,H,D]; tables (cos, sin) as LTX2RotaryPosEmbed returns them; `q_mul` is folded into
+  the f32 query scale."""
   jax, jnp = _require_jax()
-  import numpy as np
-
   if rope_type not in ("interleaved", "split"):
     raise ValueError(f"{rope_type=} not supported. Choose between 'interleaved' and 'split'.")
   q_tab = rotary_emb
   k_tab = k_rotary_emb if k_rotary_emb is not None else (rotary_emb if is_self_attention else None)
   if rotary_emb is None:
     q_tab = k_tab = None
-  dummy = jnp.zeros((1,), jnp.float32)
+  dummy = jnp.zeros((8,), jnp.float32)
 
   def run(x, scale, tab):
     b, s, n = x.shape
@@ -164,26 +257,27 @@ def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotar
     mode = 0 if tab is None else (1 if rope_type == "interleaved" else 2)
     cos, sin = (dummy, dummy) if tab is None else (tab[0].astype(jnp.float32), tab[1].astype(jnp.float32))
     call = jax.ffi.ffi_call("mdattn_norm_rope_rows", out, vmap_method="sequential")
-    return call(x, scale.astype(jnp.float32), cos, sin, eps=np.float32(eps), heads=np.int64(heads), mode=np.int64(mode))
+    return call(x, scale.astype(jnp.float32), cos, sin, eps=_f32(eps), heads=_i64(heads), mode=_i64(mode))
 
-  return run(query, norm_q_scale, q_tab), (run(key, norm_k_scale, k_tab) if key is not None else None)
+  q_scale = norm_q_scale if q_mul == 1.0 else norm_q_scale * q_mul
+  return run(query, q_scale, q_tab), (run(key, norm_k_scale, k_tab) if key is not None else None)
 
 
-def hip_flash_kernel(q, k, v, context):
-  """The KERNEL_REGISTRY entry: fn(q, k, v, context) -> [B, Sq, H*D] in q's dtype."""
-  _, jnp = _require_jax()
-  if context.get("is_causal"):
-    raise NotImplementedError("hip_flash is non-causal")
-  heads = context["heads"]
+def _as_rank4(q, k, v, heads: int):
+  """Registry inputs are rank 3 [B,S,H*D] (a free reshape to [B,S,H,D]: layout 0) or rank 4 [B,H,S,D] (layout 1)."""
   if q.ndim == 3:
     b, sq, n = q.shape
     d = n // heads
-    q4 = q.reshape(b, sq, heads, d)
-    k4 = k.reshape(b, k.shape[1], heads, d)
-    v4 = v.reshape(b, v.shape[1], heads, d)
-    layout = 0
-  else:
-    q4, k4, v4, layout = q, k, v, 1
+    return q.reshape(b, sq, heads, d), k.reshape(b, k.shape[1], heads, d), v.reshape(b, v.shape[1], heads, d), 0
+  return q, k, v, 1
+
+
+def hip_flash_kernel(q, k, v, context):
+  """The KERNEL_REGISTRY entry `hip_flash`: fn(q, k, v, context) -> [B, Sq, H*D] in q's dtype."""
+  _, jnp = _require_jax()
+  if context.get("is_causal"):
+    raise NotImplementedError("hip_flash is non-causal")
+  q4, k4, v4, layout = _as_rank4(q, k, v, context["heads"])
   dt = q.dtype
   out, _ = hip_flash_attention(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"], layout,
                                keep_mask=context.get("attention_mask"))
@@ -191,8 +285,23 @@ def hip_flash_kernel(q, k, v, context):
   return out.reshape(b, sq, h * d).astype(dt)
 
 
+def hip_flash_fp8_kernel(q, k, v, context):
+  """The KERNEL_REGISTRY entry `hip_flash_fp8` (BASELINE configs[4]): per-tensor e4m3 q, k, v on the device, then the
+  fp8 kernel.  Masks are not supported (the custom kernels of the reference raise the same way, attention_flax.py:850-854)."""
+  _, jnp = _require_jax()
+  if context.get("attention_mask") is not None:
+    raise NotImplementedError("hip_flash_fp8 does not take an attention_mask")
+  if context.get("is_causal"):
+    raise NotImplementedError("hip_flash is non-causal")
+  q4, k4, v4, layout = _as_rank4(q, k, v, context["heads"])
+  dt = q.dtype
+  out, _ = hip_flash_attention_fp8(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"], layout)
+  b, sq, h, d = out.shape
+  return out.reshape(b, sq, h * d).astype(dt)
+
+
 def install():
-  """Idempotent: FFI targets + maxdiffusion KERNEL_REGISTRY['hip_flash']."""
+  """Idempotent: FFI targets + maxdiffusion KERNEL_REGISTRY['hip_flash'] and ['hip_flash_fp8']."""
   global _installed
   if _installed:
     return
@@ -200,4 +309,5 @@ def install():
   from maxdiffusion.models import attention_flax  # type: ignore
 
   attention_flax.register_kernel("hip_flash")(hip_flash_kernel)
+  attention_flax.register_kernel("hip_flash_fp8")(hip_flash_fp8_kernel)
   _installed = True
