@@ -124,6 +124,44 @@ __device__ __forceinline__ void store_row(const AttnArgs& a, const f32x16 (&O)[N
   if (a.lse && hh == 0) a.lse[lidx] = (mc + __log2f(lt)) * kLn2;
 }
 
+// The same epilogue with whole-row stores, for a wave that may use `stage` (32 rows of HD * 2 + 16 bytes of LDS that
+// nobody else touches any more).  store_row writes, per instruction, 16 bytes of each of 32 rows that lie a whole
+// token apart; at short key sequences, where the output is a large part of the launch's work, that costs as much as
+// the attention itself (75,600 x 40 x 128 outputs: 0.27 ms).  Here the wave's 32 x HD tile is normalised, rounded to
+// bf16 and transposed through LDS, and every store instruction then writes 1 KB of whole rows (4 rows of 256 bytes
+// at head dim 128).  Same values, same rounding as store_row.
+template <int ND>
+__device__ __forceinline__ void store_rows_through_lds(const AttnArgs& a, const f32x16 (&O)[ND], float lt, float mc, int b,
+                                                       int h, int row0, int lane, char* stage) {
+  constexpr int HD = ND * 32;
+  constexpr int ROWB = HD * 2 + 16;      // padded row: the 32 lanes of a column write land on 16 different bank groups
+  constexpr int LPR = HD * 2 / 16;       // lanes that share a row in the read-back
+  constexpr int RPI = 64 / LPR;          // rows per store instruction
+  const int l32 = lane & 31, hh = lane >> 5;
+  const float inv = lt > 0.f ? 1.0f / lt : 0.f;  // rows whose keys are all excluded return 0
+  char* wrow = stage + l32 * ROWB + hh * 8;
+#pragma unroll
+  for (int db = 0; db < ND; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      uint2 u;
+      u.x = pack2(O[db][4 * g] * inv, O[db][4 * g + 1] * inv);
+      u.y = pack2(O[db][4 * g + 2] * inv, O[db][4 * g + 3] * inv);
+      *reinterpret_cast<uint2*>(wrow + (db * 32 + g * 8) * 2) = u;
+    }
+  const int row = row0 + l32;
+  if (a.lse && hh == 0 && row < a.Sq) a.lse[((int64_t)b * a.H + h) * a.Sq + row] = (mc + __log2f(lt)) * kLn2;
+  // LDS accesses of one wave execute in order: the reads below see the writes above
+  __bf16* obase = a.out + b * a.o_sb + h * a.o_sh;
+  const int rr = lane / LPR, cc = lane % LPR;
+#pragma unroll
+  for (int j = 0; j < 32 / RPI; ++j) {
+    const int r = j * RPI + rr;
+    const uint4 v = *reinterpret_cast<const uint4*>(stage + r * ROWB + cc * 16);
+    if (row0 + r < a.Sq) *reinterpret_cast<uint4*>(obase + (int64_t)(row0 + r) * a.o_ss + cc * 8) = v;
+  }
+}
+
 template <int NW, bool PRE>
 __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
@@ -431,14 +469,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   const float cs = BIAS ? 1.0f : c;
   const float* bias_row = BIAS ? a.bias + b * a.bias_sb + 4 * hh : nullptr;
 
-  bf16x8 qf[NJ];
-  {
-    int row = q0 + l32;
-    row = row < a.Sq ? row : a.Sq - 1;
-    const __bf16* p = qp + (int64_t)row * a.q_ss + hh * 8;
-#pragma unroll
-    for (int s = 0; s < NJ; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(p + s * 16);
-  }
+  bf16x8 qf[NJ];  // filled from LDS below: the wave's 32 Q rows arrive like a K tile, by whole-row loads
 
   // lane -> (row of the group, logical 16-byte chunk stored at this lane's position)
   const int grow = HD == 128 ? lane >> 4 : lane >> 3;
@@ -586,7 +617,27 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
     }
   };
 
+  // ---- Q fragments.  A lane's registers hold 16-byte pieces of ONE row, so loading them straight from global memory
+  // makes every load instruction touch 32 rows, 32 bytes of each (75,600 x 40 rows: 0.1-0.17 ms per launch).  Instead
+  // the wave fetches its 32 rows as a K-shaped tile with the same direct global->LDS loads (whole 256-byte rows per
+  // 16 lanes), into a staging area behind ring slot 0 (which receives key tile 0 meanwhile), and reads the fragments
+  // with the K fragment offsets.  Each wave stages and reads only its own rows.
   dma(0, 0);
+  {
+    const unsigned Qs = smem_addr + (unsigned)(STAGE + wave * KTILE) * 2u;
+#pragma unroll
+    for (int g = 0; g < kTS / RPI; ++g) {
+      int row = q0 + RPI * g + grow;
+      row = row < a.Sq ? row : a.Sq - 1;
+      const int qcol = HD == 128 ? kcol : ((lane & 7) ^ ((4 * (g & 1) + (grow >> 1)) & 7)) * 8;
+      lds_dma16(qp + (int64_t)row * a.q_ss + qcol, Qs + (unsigned)(g * KGS) * 2u);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the wave's own Q rows (and its share of tile 0) are in LDS
+    const __bf16* qs = smem + STAGE + wave * KTILE;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) qf[j] = *reinterpret_cast<const bf16x8*>(qs + k_off[j]);
+  }
+  __syncthreads();  // every wave holds its fragments: the staging area is ring slots 1 and 2 again
   dma(1, 1);
   int slot = 0, fill = 2;
   for (int t = 0; t < nt - 1; ++t) {
@@ -601,13 +652,21 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   __syncthreads();
   tile(nt - 1, slot, std::true_type{});
 
-  store_row<ND>(a, O, xhalf_sum(l), mc, b, h, q0 + l32, hh);
+  if (a.o_run) {  // ring step: merged into the f32 carry, row by row
+    store_row<ND>(a, O, xhalf_sum(l), mc, b, h, q0 + l32, hh);
+  } else {
+    static_assert(NW * 32 * (HD * 2 + 16) <= kSlotsS * STAGE * 2, "the output staging tiles must fit the ring's LDS");
+    __syncthreads();  // every wave has finished reading the ring: its LDS now stages the output tiles
+    store_rows_through_lds<ND>(a, O, xhalf_sum(l), mc, b, h, q0, lane, smem_raw + wave * 32 * (HD * 2 + 16));
+  }
 }
 
 template <int NW, bool BIAS, int HD = 128>
 static int launch_flat(hipStream_t st, AttnArgs a, int B) {
   constexpr int BM = NW * 32;
-  constexpr int lds_bytes = kSlotsS * (HD == 128 ? kStageS : 2 * kTS * 64) * 2;
+  // the ring, or ring slot 0 plus one K-shaped Q staging tile per wave, whichever is larger
+  constexpr int stage_el = HD == 128 ? kStageS : 2 * kTS * 64, ktile_el = HD == 128 ? kKTileS : kTS * 64;
+  constexpr int lds_bytes = (kSlotsS * stage_el > stage_el + NW * ktile_el ? kSlotsS * stage_el : stage_el + NW * ktile_el) * 2;
   a.nqt = (a.Sq + BM - 1) / BM;
   const int64_t total = (int64_t)B * a.H * a.nqt;
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
