@@ -62,6 +62,9 @@ def main():
                        "FETCH_SIZE / WRITE_SIZE counters")
   ap.add_argument("--separate-merge", action="store_true",
                   help="ring workloads: one attention launch and one merge launch per KV chunk instead of the fused step")
+  ap.add_argument("--fused-qkv", action="store_true",
+                  help="also time the prologue over a fused q|k|v projection output [1,S,3*H*D] with the three Linear biases "
+                       "(mdattn_norm_rope_qkv, in place), outside the timed steps; reported as `roofline_norm_rope_qkv`")
   ap.add_argument("--with-backward", action="store_true",
                   help="also time the backward pass (dq, dk, dv) of the workload's attention, outside the timed steps; "
                        "reported as a `backward` object beside the headline")
@@ -177,6 +180,27 @@ def main():
   torch.cuda.synchronize()
   pro_ms = e0.elapsed_time(e1) / reps
 
+  # the prologue over one fused q|k|v projection output, biases folded in, written back in place
+  fused_qkv = None
+  if args.fused_qkv and w.norm == "fullrow":
+    qkv = randn(1, S, 3 * H * D)
+    b3 = (randn(3 * H * D).float() * 0.5).to(torch.bfloat16)
+    run = lambda: ops.norm_rope_qkv(qkv, wq, wk, cos, sin, H, bias=b3, q_mul=q_mul, inplace=True)
+    run()
+    e0, e1 = ev(), ev()
+    e0.record()
+    for _ in range(reps):
+      run()
+    e1.record()
+    torch.cuda.synchronize()
+    fms = e0.elapsed_time(e1) / reps
+    fbytes = 2 * 3 * S * H * D * 2 + 2 * S * (D // 2) * 4 + 2 * 2 * H * D * 2 + 3 * H * D * 2  # q, k, v read and written; tables; weights; bias
+    fused_qkv = {"bound": "hbm", "achieved": fbytes / (fms * 1e-3) / 1e9, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                 "frac": fbytes / (fms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "traffic": None,
+                 "kernel": "norm_rope_fullrow_kernel<., true> (fused q|k|v projection, biases added, in place)",
+                 "kernel_ms": fms, "bytes_per_launch": fbytes}
+    del qkv
+
   # fp8: the same attention with exact exponentials (mdattn_fwd_fp8's other softmax mode: the lse is then the exact
   # logsumexp of the quantised logits), outside the timed steps
   fp8_exp2 = None
@@ -288,6 +312,8 @@ def main():
   if fp8:
     out["quant_ms"] = sum(t_quant) / len(t_quant)
     out["roofline_exp2"] = fp8_exp2
+  if fused_qkv:
+    out["roofline_norm_rope_qkv"] = fused_qkv
   if cross:
     out["cross_attention"] = cross
   if backward:

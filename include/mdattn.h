@@ -88,6 +88,30 @@ int mdattn_norm_rope_fullrow(void* stream, const void* q_in, const void* k_in, v
                              const mdattn_strides* out_strides);
 
 /*
+ * The same prologue over the output of ONE fused q|k|v projection, with the projections' bias adds folded in: one
+ * launch reads the GEMM output once and leaves q, k (and v) ready for the attention entry points.
+ * Replaces: the bias adds of FlaxWanAttention's query / key / value Linear layers (models/attention_flax.py:2471-2510,
+ * called :2653-2663), norm_q / norm_k (:2657, :2669), _unflatten_heads of q, k and v (:2673-2675) and _apply_rope
+ * (:2677).  (The reference runs three GEMMs; fusing them into one [hidden, 3*H*D] GEMM is the maintainer's choice:
+ * this entry point only asks that the three outputs sit side by side in one row.)
+ *   qkv          bf16 [B,S,3*H*D]: column blocks q | k | v of each token row; row stride qkv_stride_seq >= 3*H*D
+ *   bias         bf16 [3*H*D] (q | k | v) or NULL.  Given: the GEMM ran without its bias epilogue, and the biases
+ *                are added here in f32 before the statistics (one rounding fewer than the reference's bf16 Linear
+ *                output).  NULL: qkv already holds the biased projections.
+ *   q_out,k_out  bf16 by out_strides ([B,S,H,D] or [B,H,S,D]); v_out likewise, or NULL
+ *   v_out        NULL (only without bias): v is not touched; the attention entry points read it in place from the
+ *                fused buffer (pointer qkv + 2*H*D, strides {qkv_stride_batch, qkv_stride_seq, D}).
+ *   In place: with out_strides = {qkv_stride_batch, qkv_stride_seq, D}, q_out = qkv, k_out = qkv + H*D (and
+ *   v_out = qkv + 2*H*D) the fused buffer itself becomes the attention operands; outputs may alias the input only
+ *   like this, element for element.
+ *   wq, wk, cos, sin, eps, q_mul and the arithmetic as for mdattn_norm_rope_fullrow.
+ */
+int mdattn_norm_rope_qkv(void* stream, const void* qkv, const void* bias, void* q_out, void* k_out, void* v_out,
+                         const void* wq, const void* wk, const float* cos, const float* sin,
+                         int B, int S, int H, int D, float eps, float q_mul,
+                         int64_t qkv_stride_batch, int64_t qkv_stride_seq, const mdattn_strides* out_strides);
+
+/*
  * Fused per-head RMSNorm (over D) + 3-axis RoPE, for q and k in one pass.
  * Replaces: FlaxFluxAttention's query_norm / key_norm / encoder_*_norm
  * (models/attention_flax.py:2947-2967, applied :2989-2990 and :3002-3003; single blocks

@@ -82,6 +82,15 @@ int mdattn_xla_norm_rope_fullrow(void* stream, const mdattn_buffer* q, const mda
                                  const mdattn_buffer* q_out, const mdattn_buffer* k_out, float eps, float q_mul,
                                  int64_t heads, int64_t rope, int64_t has_k, char* err, int err_len);
 
+/* "mdattn_norm_rope_qkv": (qkv bf16 [B,S,3*H*D], bias bf16 [3*H*D], wq, wk bf16 [H*D], cos, sin f32 [S,D/2]) -> (q_out,
+ * k_out, v_out bf16 [B,S,H,D]).  has_bias == 0: bias is ignored; has_v == 0 (only without bias): v_out is ignored and v
+ * stays in the fused buffer (the caller slices it).  XLA cannot alias a result to a slice of an operand, so the
+ * custom call always writes dense results; the in-place form is for callers of the C ABI. */
+int mdattn_xla_norm_rope_qkv(void* stream, const mdattn_buffer* qkv, const mdattn_buffer* bias, const mdattn_buffer* wq,
+                             const mdattn_buffer* wk, const mdattn_buffer* cos, const mdattn_buffer* sin,
+                             const mdattn_buffer* q_out, const mdattn_buffer* k_out, const mdattn_buffer* v_out, float eps,
+                             float q_mul, int64_t heads, int64_t rope, int64_t has_bias, int64_t has_v, char* err, int err_len);
+
 /* "mdattn_norm_rope_perhead": (q, k bf16 [B,S,H,D], wq, wk, wq_txt, wk_txt bf16 [D], cos, sin f32 [S,D/2]) ->
  * (q_out, k_out bf16 [B,S,H,D]).  Tokens [0, n_txt) take the text weights (FlaxFluxAttention's encoder_*_norm,
  * attention_flax.py:3002-3003); n_txt == 0: wq_txt / wk_txt are ignored. */

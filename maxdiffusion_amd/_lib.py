@@ -36,6 +36,7 @@ SIGNATURES = {
     "mdattn_build_id": ([], ctypes.c_char_p),
     "mdattn_set_fwd_schedule": ([_I], _I),
     "mdattn_norm_rope_fullrow": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _L, _L, _S], _I),
+    "mdattn_norm_rope_qkv": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _L, _L, _S], _I),
     "mdattn_norm_rope_perhead": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _F, _F, _S, _S], _I),
     "mdattn_norm_rope_rows": ([_P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _L, _L, _S], _I),
     "mdattn_fwd_bf16": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),

@@ -82,6 +82,14 @@ ffi::Error NormRopeFullrow(hipStream_t s, Buf q, Buf k, Buf wq, Buf wk, Buf cos,
   const mdattn_buffer a = In(q), b = In(k), c = In(wq), d = In(wk), e = In(cos), f = In(sin), qo = Out(q_out), ko = Out(k_out);
   return m.done(mdattn_xla_norm_rope_fullrow(s, &a, &b, &c, &d, &e, &f, &qo, &ko, eps, q_mul, heads, rope, has_k, m.text, sizeof m.text));
 }
+ffi::Error NormRopeQkv(hipStream_t s, Buf qkv, Buf bias, Buf wq, Buf wk, Buf cos, Buf sin, Res q_out, Res k_out, Res v_out, float eps,
+                       float q_mul, int64_t heads, int64_t rope, int64_t has_bias, int64_t has_v) {
+  Msg m;
+  const mdattn_buffer a = In(qkv), b = In(bias), c = In(wq), d = In(wk), e = In(cos), f = In(sin), qo = Out(q_out), ko = Out(k_out),
+                      vo = Out(v_out);
+  return m.done(mdattn_xla_norm_rope_qkv(s, &a, &b, &c, &d, &e, &f, &qo, &ko, &vo, eps, q_mul, heads, rope, has_bias, has_v, m.text,
+                                         sizeof m.text));
+}
 ffi::Error NormRopePerhead(hipStream_t s, Buf q, Buf k, Buf wq, Buf wk, Buf wq_txt, Buf wk_txt, Buf cos, Buf sin, Res q_out, Res k_out,
                            float eps, float q_mul, int64_t n_txt, int64_t rope, int64_t has_k) {
   Msg m;
@@ -140,6 +148,11 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopeFullrow, NormRopeFullrow,
                               MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Ret<Buf>().Ret<Buf>()
                                   .Attr<float>("eps").Attr<float>("q_mul").Attr<int64_t>("heads").Attr<int64_t>("rope")
                                   .Attr<int64_t>("has_k"));
+XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopeQkv, NormRopeQkv,
+                              MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>()
+                                  .Ret<Buf>().Ret<Buf>().Ret<Buf>()
+                                  .Attr<float>("eps").Attr<float>("q_mul").Attr<int64_t>("heads").Attr<int64_t>("rope")
+                                  .Attr<int64_t>("has_bias").Attr<int64_t>("has_v"));
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopePerhead, NormRopePerhead,
                               MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>()
                                   .Ret<Buf>().Ret<Buf>()

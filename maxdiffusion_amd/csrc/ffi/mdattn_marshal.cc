@@ -266,6 +266,45 @@ extern "C" int mdattn_xla_norm_rope_fullrow(void* stream, const mdattn_buffer* q
                                          q_mul, S * N, N, &so));
 }
 
+extern "C" int mdattn_xla_norm_rope_qkv(void* stream, const mdattn_buffer* qkv, const mdattn_buffer* bias, const mdattn_buffer* wq,
+                                        const mdattn_buffer* wk, const mdattn_buffer* cos, const mdattn_buffer* sin,
+                                        const mdattn_buffer* q_out, const mdattn_buffer* k_out, const mdattn_buffer* v_out, float eps,
+                                        float q_mul, int64_t heads, int64_t rope, int64_t has_bias, int64_t has_v, char* err,
+                                        int err_len) {
+  const Err e{err, err_len, "mdattn_norm_rope_qkv"};
+  CHECK_BUF(e, qkv, "qkv");
+  CHECK_DT(e, qkv, "qkv", MDATTN_DT_BF16);
+  if (qkv->rank != 3 || heads <= 0 || qkv->dims[2] % (3 * heads))
+    return e.fail(MDATTN_E_BADARG, "qkv must be [B,S,3*H*D] with H = heads = %lld", (long long)heads);
+  const int64_t B = qkv->dims[0], S = qkv->dims[1], N = qkv->dims[2] / 3, D = N / heads;
+  if (!fits_int(B) || !fits_int(S) || !fits_int(3 * N)) return e.fail(MDATTN_E_UNSUPPORTED, "dimensions beyond 2^31");
+  if (has_bias && !has_v) return e.fail(MDATTN_E_BADARG, "with a bias the value block needs its bias too: has_v must be set");
+  auto is_bshd = [&](const mdattn_buffer* b) {
+    return b->rank == 4 && b->dims[0] == B && b->dims[1] == S && b->dims[2] == heads && b->dims[3] == D;
+  };
+  const mdattn_buffer* outs[3] = {q_out, k_out, v_out};
+  const char* names[3] = {"q_out", "k_out", "v_out"};
+  for (int i = 0; i < (has_v ? 3 : 2); ++i) {
+    CHECK_BUF(e, outs[i], names[i]);
+    CHECK_DT(e, outs[i], names[i], MDATTN_DT_BF16);
+    if (!is_bshd(outs[i]))
+      return e.fail(MDATTN_E_BADARG, "%s must be [B,S,H,D] = [%lld,%lld,%lld,%lld]", names[i], (long long)B, (long long)S, (long long)heads, (long long)D);
+  }
+  TRY(check_vec(e, wq, "wq", MDATTN_DT_BF16, N));
+  TRY(check_vec(e, wk, "wk", MDATTN_DT_BF16, N));
+  if (has_bias) TRY(check_vec(e, bias, "bias", MDATTN_DT_BF16, 3 * N));
+  if (rope) {
+    TRY(check_vec(e, cos, "cos", MDATTN_DT_F32, S * (D / 2)));
+    TRY(check_vec(e, sin, "sin", MDATTN_DT_F32, S * (D / 2)));
+  }
+  const mdattn_strides so{S * N, N, D};
+  return e.from(mdattn_norm_rope_qkv(stream, qkv->data, has_bias ? bias->data : nullptr, q_out->data, k_out->data,
+                                     has_v ? v_out->data : nullptr, wq->data, wk->data,
+                                     rope ? static_cast<const float*>(cos->data) : nullptr,
+                                     rope ? static_cast<const float*>(sin->data) : nullptr, (int)B, (int)S, (int)heads, (int)D, eps,
+                                     q_mul, S * 3 * N, 3 * N, &so));
+}
+
 extern "C" int mdattn_xla_norm_rope_perhead(void* stream, const mdattn_buffer* q, const mdattn_buffer* k, const mdattn_buffer* wq,
                                             const mdattn_buffer* wk, const mdattn_buffer* wq_txt, const mdattn_buffer* wk_txt,
                                             const mdattn_buffer* cos, const mdattn_buffer* sin, const mdattn_buffer* q_out,

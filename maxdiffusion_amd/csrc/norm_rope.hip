@@ -16,10 +16,16 @@ struct NormRopeFullArgs {
   float q_mul;            // constant folded into the q output before its rounding
   int64_t in_sb, in_ss;
   int64_t out_sb, out_ss, out_sh;
+  // FUSED (mdattn_norm_rope_qkv): the projection biases still to be added (null: none), and the value block
+  const uint4* bias[3];   // q, k, v
+  const uint4* v_in;
+  uint4* v_out;           // null: v is left where it is
 };
 
 // One workgroup (256 lanes) per token row; lane t owns 16-byte chunks t, t+256, ... (<= MAXC).
-template <int MAXC>
+// FUSED: the row is the output of a fused q|k|v projection; the projection biases are added in f32 before the
+// statistics, and the value block is passed through (bias added, laid out like q and k) in the same launch.
+template <int MAXC, bool FUSED = false>
 __global__ __launch_bounds__(256) void norm_rope_fullrow_kernel(NormRopeFullArgs a) {
   const int tid = threadIdx.x;
   const int s = blockIdx.x, b = blockIdx.y;
@@ -40,6 +46,29 @@ __global__ __launch_bounds__(256) void norm_rope_fullrow_kernel(NormRopeFullArgs
       }
     }
   }
+  [[maybe_unused]] uint4 vraw[MAXC];
+  if constexpr (FUSED) {
+    if (a.v_out) {
+      const uint4* row = a.v_in + ((b * a.in_sb + s * a.in_ss) >> 3);
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = tid + i * 256;
+        if (c < nchunks) vraw[i] = ld_nt(row + c);
+      }
+    }
+  }
+  // value of chunk c of tensor t as the statistics and the output see it: the projection plus its bias
+  auto chunk_f32 = [&](int t, int i, int c, float* f) __attribute__((always_inline)) {
+    unpack8(raw[t][i], f);
+    if constexpr (FUSED) {
+      if (a.bias[t]) {
+        float bb[8];
+        unpack8(a.bias[t][c], bb);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] += bb[j];
+      }
+    }
+  };
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     if (t < ntens) {
@@ -48,7 +77,7 @@ __global__ __launch_bounds__(256) void norm_rope_fullrow_kernel(NormRopeFullArgs
         const int c = tid + i * 256;
         if (c < nchunks) {
           float f[8];
-          unpack8(raw[t][i], f);
+          chunk_f32(t, i, c, f);
 #pragma unroll
           for (int j = 0; j < 8; ++j) ss[t] = __builtin_fmaf(f[j], f[j], ss[t]);
         }
@@ -91,7 +120,7 @@ __global__ __launch_bounds__(256) void norm_rope_fullrow_kernel(NormRopeFullArgs
       for (int t = 0; t < 2; ++t) {
         if (t < ntens) {
           float f[8], w[8], o[8];
-          unpack8(raw[t][i], f);
+          chunk_f32(t, i, c, f);
           unpack8(a.w[t][c], w);
 #pragma unroll
           for (int j = 0; j < 8; ++j) f[j] = f[j] * inv[t] * w[j];
@@ -102,6 +131,20 @@ __global__ __launch_bounds__(256) void norm_rope_fullrow_kernel(NormRopeFullArgs
           }
           uint4* dst = a.x_out[t] + ((b * a.out_sb + s * a.out_ss + h * a.out_sh + d) >> 3);
           st_nt(dst, pack8(o));
+        }
+      }
+      if constexpr (FUSED) {
+        if (a.v_out) {
+          uint4 u = vraw[i];
+          if (a.bias[2]) {
+            float f[8], bb[8];
+            unpack8(u, f);
+            unpack8(a.bias[2][c], bb);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) f[j] += bb[j];
+            u = pack8(f);
+          }
+          st_nt(a.v_out + ((b * a.out_sb + s * a.out_ss + h * a.out_sh + d) >> 3), u);
         }
       }
     }
@@ -337,6 +380,7 @@ extern "C" int mdattn_norm_rope_fullrow(void* stream, const void* q_in, const vo
   a.S = S; a.H = H; a.D = D; a.N = (int)N; a.eps = eps; a.inv_n = 1.0f / (float)N; a.q_mul = q_mul;
   a.in_sb = in_stride_batch; a.in_ss = in_stride_seq;
   a.out_sb = out_strides->batch; a.out_ss = out_strides->seq; a.out_sh = out_strides->head;
+  a.bias[0] = a.bias[1] = a.bias[2] = nullptr; a.v_in = nullptr; a.v_out = nullptr;
   dim3 grid(S, B), block(256);
   hipStream_t st = (hipStream_t)stream;
   const int nchunks = (int)(N / 8);
@@ -344,6 +388,44 @@ extern "C" int mdattn_norm_rope_fullrow(void* stream, const void* q_in, const vo
   else if (nchunks <= 512) hipLaunchKernelGGL(norm_rope_fullrow_kernel<2>, grid, block, 0, st, a);
   else if (nchunks <= 768) hipLaunchKernelGGL(norm_rope_fullrow_kernel<3>, grid, block, 0, st, a);
   else hipLaunchKernelGGL(norm_rope_fullrow_kernel<4>, grid, block, 0, st, a);
+  return launch_status();
+}
+
+extern "C" int mdattn_norm_rope_qkv(void* stream, const void* qkv, const void* bias, void* q_out, void* k_out, void* v_out,
+                                    const void* wq, const void* wk, const float* cos, const float* sin,
+                                    int B, int S, int H, int D, float eps, float q_mul,
+                                    int64_t qkv_stride_batch, int64_t qkv_stride_seq, const mdattn_strides* out_strides) {
+  if (!qkv || !q_out || !k_out || !wq || !wk || B <= 0 || S <= 0 || H <= 0 || D <= 0 || !out_strides) return MDATTN_E_BADARG;
+  if ((cos == nullptr) != (sin == nullptr)) return MDATTN_E_BADARG;
+  if (bias && !v_out) return MDATTN_E_BADARG;  // the value block needs its bias too: it cannot stay where it is
+  if (!(eps >= 0.f) || !(q_mul > 0.f) || !(q_mul < 1e30f)) return MDATTN_E_BADARG;
+  const int64_t N = (int64_t)H * D;
+  if (D % 8 != 0 || N > 8192) return MDATTN_E_UNSUPPORTED;
+  if (B > 65535) return MDATTN_E_UNSUPPORTED;
+  if (qkv_stride_seq < 3 * N || qkv_stride_batch < 0) return MDATTN_E_BADARG;
+  if (!aligned16(qkv) || !aligned16(bias) || !aligned16(q_out) || !aligned16(k_out) || !aligned16(v_out) || !aligned16(wq) ||
+      !aligned16(wk) || !aligned16(cos) || !aligned16(sin))
+    return MDATTN_E_ALIGN;
+  if (qkv_stride_batch % 8 || qkv_stride_seq % 8 || !strides_ok(out_strides, 8)) return MDATTN_E_ALIGN;
+
+  NormRopeFullArgs a;
+  const uint4* base = (const uint4*)qkv;
+  a.x_in[0] = base; a.x_in[1] = base + N / 8; a.v_in = base + 2 * N / 8;
+  a.x_out[0] = (uint4*)q_out; a.x_out[1] = (uint4*)k_out; a.v_out = (uint4*)v_out;
+  a.w[0] = (const uint4*)wq; a.w[1] = (const uint4*)wk;
+  const uint4* bb = (const uint4*)bias;
+  a.bias[0] = bb; a.bias[1] = bb ? bb + N / 8 : nullptr; a.bias[2] = bb ? bb + 2 * N / 8 : nullptr;
+  a.cos = (const float4*)cos; a.sin = (const float4*)sin;
+  a.S = S; a.H = H; a.D = D; a.N = (int)N; a.eps = eps; a.inv_n = 1.0f / (float)N; a.q_mul = q_mul;
+  a.in_sb = qkv_stride_batch; a.in_ss = qkv_stride_seq;
+  a.out_sb = out_strides->batch; a.out_ss = out_strides->seq; a.out_sh = out_strides->head;
+  dim3 grid(S, B), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  const int nchunks = (int)(N / 8);
+  if (nchunks <= 256) hipLaunchKernelGGL((norm_rope_fullrow_kernel<1, true>), grid, block, 0, st, a);
+  else if (nchunks <= 512) hipLaunchKernelGGL((norm_rope_fullrow_kernel<2, true>), grid, block, 0, st, a);
+  else if (nchunks <= 768) hipLaunchKernelGGL((norm_rope_fullrow_kernel<3, true>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((norm_rope_fullrow_kernel<4, true>), grid, block, 0, st, a);
   return launch_status();
 }
 

@@ -29,6 +29,7 @@ FFI_TARGETS = {
     "mdattn_merge": "MdattnMerge",
     "mdattn_finalize": "MdattnFinalize",
     "mdattn_norm_rope_fullrow": "MdattnNormRopeFullrow",
+    "mdattn_norm_rope_qkv": "MdattnNormRopeQkv",
     "mdattn_norm_rope_perhead": "MdattnNormRopePerhead",
     "mdattn_norm_rope_rows": "MdattnNormRopeRows",
     "mdattn_quant_e4m3": "MdattnQuantE4m3",
@@ -217,6 +218,26 @@ def hip_norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6,
   q_out, k_res = call(q, k if has_k else q, wq, wk if has_k else wq, cos if rope else dummy, sin if rope else dummy,
                       eps=_f32(eps), q_mul=_f32(q_mul), heads=_i64(heads), rope=_i64(rope), has_k=_i64(has_k))
   return q_out, (k_res if has_k else None)
+
+
+def hip_norm_rope_qkv(qkv, wq, wk, cos, sin, heads: int, bias=None, eps: float = 1e-6, q_mul: float = 1.0):
+  """The prologue over the output of one fused q|k|v projection: qkv bf16 [B,S,3*H*D] (column blocks q | k | v);
+  bias bf16 [3*H*D] or None (the Linear biases, when the GEMM ran without them) -> (q, k, v) [B,S,H,D] bf16.  Without
+  a bias v is a slice of the fused buffer (XLA fuses the reshape; nothing is copied by the custom call).  One launch in
+  place of the three bias adds, norm_q / norm_k, _unflatten_heads and _apply_rope of attention_flax.py:2653-2677."""
+  jax, jnp = _require_jax()
+  b, s, n3 = qkv.shape
+  n = n3 // 3
+  d = n // heads
+  rope, has_bias = cos is not None, bias is not None
+  dummy = jnp.zeros((8,), jnp.float32)
+  out = jax.ShapeDtypeStruct((b, s, heads, d), jnp.bfloat16)
+  v_out = out if has_bias else jax.ShapeDtypeStruct((8,), jnp.bfloat16)
+  call = jax.ffi.ffi_call("mdattn_norm_rope_qkv", (out, out, v_out), vmap_method="sequential")
+  q_out, k_out, v_res = call(qkv, bias if has_bias else wq, wq, wk, cos if rope else dummy, sin if rope else dummy,
+                             eps=_f32(eps), q_mul=_f32(q_mul), heads=_i64(heads), rope=_i64(rope), has_bias=_i64(has_bias),
+                             has_v=_i64(has_bias))
+  return q_out, k_out, (v_res if has_bias else qkv[:, :, 2 * n:].reshape(b, s, heads, d))
 
 
 def hip_norm_rope_perhead(q, k, wq, wk, cos, sin, eps: float = 1e-6, wq_txt=None, wk_txt=None, n_txt: int = 0, q_mul: float = 1.0):

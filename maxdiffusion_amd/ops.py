@@ -16,7 +16,7 @@ from . import _lib
 from ._lib import Strides
 
 __all__ = [
-    "norm_rope_fullrow", "norm_rope_perhead", "norm_rope_rows", "flash_attention", "flash_attention_backward", "flash_attention_backward_static", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
+    "norm_rope_fullrow", "norm_rope_qkv", "norm_rope_perhead", "norm_rope_rows", "flash_attention", "flash_attention_backward", "flash_attention_backward_static", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
     "merge_partial", "flash_attention_merge", "finalize", "new_merge_state", "LSE_INIT", "FOLDED_SCALE", "folded_q_mul", "set_fwd_schedule", "FWD_SCHEDULES", "FP8_SOFTMAX_MODES",
 ]
 
@@ -104,6 +104,38 @@ def norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6, out
       b, s, heads, d, eps, q_mul, q.stride(0), q.stride(1), ctypes.byref(st))
   _lib.check(rc, "mdattn_norm_rope_fullrow")
   return q_out, k_out
+
+
+def norm_rope_qkv(qkv, wq, wk, cos, sin, heads: int, bias=None, eps: float = 1e-6, out_layout: str = "bshd", q_mul: float = 1.0,
+                  inplace: bool = False):
+  """The prologue over the output of one fused q|k|v projection: qkv bf16 [B, S, 3*H*D] (column blocks q | k | v).
+
+  bias bf16 [3*H*D] or None: the projections' biases, added in f32 before the statistics.  Returns (q, k, v) logical
+  [B,S,H,D] views.  Without bias v is a view of the fused buffer itself (never copied).  inplace=True writes q, k
+  (and the biased v) back into the fused buffer, which then holds the three attention operands."""
+  _check_dev(qkv, wq, wk, cos, sin, bias)
+  if qkv.dim() != 3 or qkv.dtype != torch.bfloat16 or qkv.stride(2) != 1 or qkv.shape[2] % (3 * heads):
+    raise ValueError("qkv must be bf16 [B, S, 3*H*D] with a contiguous last axis")
+  b, s, n3 = qkv.shape
+  n = n3 // 3
+  d = n // heads
+  cos, sin = _table(cos, s, d, "cos"), _table(sin, s, d, "sin")
+  if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != n3 or not bias.is_contiguous()):
+    raise ValueError("bias must be a contiguous bf16 [3*H*D] tensor")
+  blocks = [qkv[:, :, i * n:(i + 1) * n].unflatten(2, (heads, d)) for i in range(3)]  # views of the fused buffer
+  if inplace:
+    q_out, k_out = blocks[0], blocks[1]
+    v_out = blocks[2] if bias is not None else None
+  else:
+    q_out = _alloc_like_layout(b, s, heads, d, out_layout, torch.bfloat16, qkv.device)
+    k_out = _alloc_like_layout(b, s, heads, d, out_layout, torch.bfloat16, qkv.device)
+    v_out = _alloc_like_layout(b, s, heads, d, out_layout, torch.bfloat16, qkv.device) if bias is not None else None
+  st = _strides(q_out)
+  rc = _lib.load().mdattn_norm_rope_qkv(
+      _stream(), _ptr(qkv), _ptr(bias), _ptr(q_out), _ptr(k_out), _ptr(v_out), _ptr(wq), _ptr(wk), _ptr(cos), _ptr(sin),
+      b, s, heads, d, eps, q_mul, qkv.stride(0), qkv.stride(1), ctypes.byref(st))
+  _lib.check(rc, "mdattn_norm_rope_qkv")
+  return q_out, k_out, (v_out if v_out is not None else blocks[2])
 
 
 def norm_rope_rows(x, w, cos=None, sin=None, heads: int = 1, mode: str = "none", eps: float = 1e-6, out_layout: str = "bshd"):

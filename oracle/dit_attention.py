@@ -21,6 +21,8 @@ Pinning status of each function (what fixes it besides its own formula):
   ltx2_apply_rotary_emb          equals apply_rope_interleaved on repeat-interleaved tables
   ltx2_apply_split_rotary_emb    brute-force loop, norm preservation, and: split rotation of x equals
                                  the interleaved rotation of x with each head's halves interleaved
+  norm_rope_fullrow / _perhead   compositions of rmsnorm and apply_rope_interleaved (both pinned above)
+  / _qkv                         plus, for _qkv, the bias add and the column split of the fused projection
   attention / attention_rows     scipy logsumexp, torch SDPA (fp32, CPU),
                                  invariants (K=0 -> mean(V), lse=ln Skv; ...),
                                  hand fixtures of tests/ltx2/test_attention_ltx2.py:38-116
@@ -51,7 +53,7 @@ __all__ = [
     "bf16_round", "to_bf16_bits", "from_bf16_bits", "e4m3_round", "E4M3_MAX",
     "rmsnorm", "wan_rope_angles", "wan_rope_table", "wan_rope_table_complex",
     "flux_ids", "flux_rope_angles", "flux_rope_table", "flux_rope_table_matrix",
-    "apply_rope_interleaved", "apply_rope_matrix_form", "norm_rope_fullrow", "norm_rope_perhead",
+    "apply_rope_interleaved", "apply_rope_matrix_form", "norm_rope_fullrow", "norm_rope_qkv", "norm_rope_perhead",
     "norm_rope_wan_reference_flow", "attention", "attention_rows", "attention_dot_product_bf16",
     "ltx2_apply_rotary_emb", "ltx2_apply_split_rotary_emb", "norm_rope_ltx2", "attention_bwd", "merge_lse", "merge_mlo", "merge_scan_ring", "ring_replay", "quant_e4m3", "attention_fp8_emulated",
     "LSE_INIT",
@@ -234,6 +236,20 @@ def norm_rope_fullrow(x, w, cos, sin, heads: int, eps: float = 1e-6, dtype=np.fl
   if cos is None:
     return y
   return apply_rope_interleaved(y, cos, sin, seq_axis=-3)
+
+
+def norm_rope_qkv(qkv, wq, wk, cos, sin, heads: int, bias=None, eps: float = 1e-6, dtype=np.float64):
+  """The Wan prologue over a fused projection output qkv [B,S,3*H*D] (column blocks q | k | v) whose Linear biases
+  (attention_flax.py:2471-2510) may still have to be added: q = rope(norm(x_q + b_q)), k likewise, v = x_v + b_v.
+  Returns (q, k, v) as [B,S,H,D].  A composition of `norm_rope_fullrow` (pinned) with the bias add and the split."""
+  qkv = np.asarray(qkv, dtype)
+  b, s, n3 = qkv.shape
+  n = n3 // 3
+  if bias is not None:
+    qkv = qkv + np.asarray(bias, dtype)[None, None, :]
+  q = norm_rope_fullrow(qkv[..., :n], wq, cos, sin, heads, eps, dtype)
+  k = norm_rope_fullrow(qkv[..., n:2 * n], wk, cos, sin, heads, eps, dtype)
+  return q, k, qkv[..., 2 * n:].reshape(b, s, heads, n // heads)
 
 
 def norm_rope_perhead(x, w, cos, sin, eps: float = 1e-6, dtype=np.float64, w_txt=None, n_txt: int = 0):

@@ -96,6 +96,10 @@ class _FakeArray:
   def __mul__(self, other):
     return _FakeArray(self.shape, self.dtype)
 
+  def __getitem__(self, idx):  # slicing of the last axis only: x[:, :, a:]
+    a = idx[-1].start or 0
+    return _FakeArray(self.shape[:-1] + (self.shape[-1] - a,), self.dtype)
+
 
 @pytest.fixture
 def fake_jax(monkeypatch):
@@ -159,6 +163,9 @@ def test_python_wrappers_follow_the_bind_lines(fake_jax):
   P.hip_norm_rope_fullrow(q3, q3, w, w, tab, tab, H)
   P.hip_norm_rope_fullrow(q3, None, w, None, None, None, H)                    # norm only, cached K/V
   P.hip_norm_rope_perhead(q, q, wd, wd, tab, tab, wq_txt=wd, wk_txt=wd, n_txt=7)
+  qkv, b3 = _FakeArray((B, S, 3 * H * D), bf), _FakeArray((3 * H * D,), bf)
+  assert [t.shape for t in P.hip_norm_rope_qkv(qkv, w, w, tab, tab, H, bias=b3)] == [(B, S, H, D)] * 3
+  assert [t.shape for t in P.hip_norm_rope_qkv(qkv, w, w, None, None, H)] == [(B, S, H, D)] * 3   # v sliced from the fused buffer
   P.hip_norm_rope_ltx2(q3, q3, _FakeArray((H * D,), f32), _FakeArray((H * D,), f32), H,
                        rotary_emb=(_FakeArray((B, S, H * D), f32), _FakeArray((B, S, H * D), f32)))
   binds = _bind_lines()
@@ -274,6 +281,12 @@ def test_marshalling_rejects_bad_buffers_by_name(lib):
         buf((S, D // 2), F32), buf((S, D // 2), F32), out, out, f(1e-6), f(1.0), i(H), i(1), i(1)), "wq must hold 384"),
       (("norm_rope_perhead", q, q, buf((D,), BF16), buf((D,), BF16), buf((D,), BF16), buf((D,), BF16), buf((S, D // 2), F32),
         buf((S, D // 2), F32), out, out, f(1e-6), f(1.0), i(S + 1), i(1), i(1)), "n_txt"),
+      (("norm_rope_qkv", buf((B, S, 3 * H * D), BF16), buf((3 * H * D,), BF16), buf((H * D,), BF16), buf((H * D,), BF16),
+        buf((S, D // 2), F32), buf((S, D // 2), F32), out, out, out, f(1e-6), f(1.0), i(H), i(1), i(1), i(0)), "has_v must be set"),
+      (("norm_rope_qkv", buf((B, S, 3 * H * D), BF16), buf((H * D,), BF16), buf((H * D,), BF16), buf((H * D,), BF16),
+        buf((S, D // 2), F32), buf((S, D // 2), F32), out, out, out, f(1e-6), f(1.0), i(H), i(1), i(1), i(1)), "bias must hold 1152"),
+      (("norm_rope_qkv", buf((B, S, 2 * H * D), BF16), buf((3 * H * D,), BF16), buf((H * D,), BF16), buf((H * D,), BF16),
+        buf((S, D // 2), F32), buf((S, D // 2), F32), out, out, out, f(1e-6), f(1.0), i(H), i(1), i(0), i(0)), "qkv must be [B,S,3*H*D]"),
       (("norm_rope_perhead", q, q, buf((D,), BF16), buf((D,), BF16), buf((2 * D,), BF16), buf((D,), BF16), buf((S, D // 2), F32),
         buf((S, D // 2), F32), out, out, f(1e-6), f(1.0), i(5), i(1), i(1)), "wq_txt must hold 128"),
       (("norm_rope_rows", buf((B, S, H * D), BF16), buf((H * D,), F32), buf((B, S, H * D), F32), buf((B, S, H * D), F32), out,

@@ -100,6 +100,15 @@ def test_prologue_handlers(dev, lib):
   dummy, dummy_out = torch.zeros(8, device=dev), torch.zeros(8, dtype=torch.bfloat16, device=dev)
   xla(lib, "norm_rope_fullrow", q, q, wq, wq, dummy, dummy, qo, dummy_out, f(1e-6), f(1.0), i(H), i(0), i(0))
   assert torch.equal(qo, ops.norm_rope_fullrow(q, None, wq, None, None, None, H)[0])
+  # the fused q|k|v projection form, with and without the projection biases
+  qkv, b3 = rn(B, S, 3 * H * D).to(torch.bfloat16), (0.5 * rn(3 * H * D)).to(torch.bfloat16)
+  vo = torch.empty((B, S, H, D), dtype=torch.bfloat16, device=dev)
+  xla(lib, "norm_rope_qkv", qkv, b3, wq, wk, cos, sin, qo, ko, vo, f(1e-6), f(1.25), i(H), i(1), i(1), i(1))
+  want = ops.norm_rope_qkv(qkv, wq, wk, cos, sin, H, bias=b3, q_mul=1.25)
+  assert all(torch.equal(a_, b_) for a_, b_ in zip((qo, ko, vo), want))
+  xla(lib, "norm_rope_qkv", qkv, wq, wq, wk, cos, sin, qo, ko, dummy_out, f(1e-6), f(1.0), i(H), i(1), i(0), i(0))
+  want = ops.norm_rope_qkv(qkv, wq, wk, cos, sin, H)
+  assert torch.equal(qo, want[0]) and torch.equal(ko, want[1])
   # per head, with the text-token weights of Flux's double blocks
   q4, k4 = q.view(B, S, H, D), k.view(B, S, H, D)
   w = [(1 + 0.1 * rn(D)).to(torch.bfloat16) for _ in range(4)]

@@ -172,3 +172,57 @@ def test_q_mul_scales_the_query_only(dev):
   qo, ko = ops.norm_rope_perhead(q, k, w[0], w[1], _t(f["cos"], dev), _t(f["sin"], dev), wq_txt=w[2], wk_txt=w[3], n_txt=int(f["n_txt"]), q_mul=m)
   _assert_close(to_np(qo) / m, f["q_out"], "flux golden q with q_mul")
   _assert_close(to_np(ko), f["k_out"], "flux golden k with q_mul")
+
+
+@pytest.mark.parametrize("heads,hidden", [(4, 512), (12, 1536), (40, 5120)])
+def test_fused_qkv_projection_prologue(dev, heads, hidden):
+  """mdattn_norm_rope_qkv: one launch over the output of a fused q|k|v projection [B,S,3*H*D] -- bias adds of the three
+  Linear layers (attention_flax.py:2471-2510), norm_q / norm_k, the head split and the rotation -- against the oracle;
+  without a bias it equals the two-tensor entry point bit for bit and leaves v in the fused buffer; in place, the
+  fused buffer itself becomes the attention operands and attention on those strided views equals attention on dense
+  copies bit for bit."""
+  B, grid, D = 2, (3, 6, 7), 128
+  S, N = grid[0] * grid[1] * grid[2], heads * 128
+  assert N == hidden
+  qkv = O.normal_bf16((B, S, 3 * N), 0)
+  bias = O.bf16_round(0.5 * O.normal_bf16((3 * N,), 5))
+  wq, wk = O.norm_weight(N, 3), O.norm_weight(N, 4)
+  cos, sin = O.wan_rope_table(grid, D)
+  dq, db, dwq, dwk = (to_dev_bf16(x, dev) for x in (qkv, bias, wq, wk))
+  dcos, dsin = _t(cos, dev), _t(sin, dev)
+  # (a) no bias: the same arithmetic as the two-tensor entry point on the q and k column blocks; v is the buffer's own block
+  q0, k0, v0 = ops.norm_rope_qkv(dq, dwq, dwk, dcos, dsin, heads)
+  wq_, wk_ = ops.norm_rope_fullrow(dq[:, :, :N], dq[:, :, N:2 * N], dwq, dwk, dcos, dsin, heads)
+  assert torch.equal(q0, wq_) and torch.equal(k0, wk_)
+  assert v0.data_ptr() == dq.data_ptr() + 2 * N * 2 and torch.equal(v0.reshape(B, S, N), dq[:, :, 2 * N:])
+  # (b) with the projection biases, against the oracle
+  for layout in ("bshd", "bhsd"):
+    q1, k1, v1 = ops.norm_rope_qkv(dq, dwq, dwk, dcos, dsin, heads, bias=db, out_layout=layout, q_mul=1.0)
+    rq, rk, rv = O.norm_rope_qkv(qkv, wq, wk, cos, sin, heads, bias=bias)
+    _assert_close(to_np(q1), rq, f"fused qkv q {layout} H={heads}")
+    _assert_close(to_np(k1), rk, f"fused qkv k {layout} H={heads}")
+    _assert_close(to_np(v1), rv, f"fused qkv v {layout} H={heads}")
+    assert not torch.equal(q1, q0.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3) if layout == "bhsd" else q0)  # the bias matters
+  # (c) in place: the fused buffer becomes q | k | v, element for element what (b) returned in [B,S,H,D]
+  q1, k1, v1 = ops.norm_rope_qkv(dq, dwq, dwk, dcos, dsin, heads, bias=db)
+  buf = dq.clone()
+  q2, k2, v2 = ops.norm_rope_qkv(buf, dwq, dwk, dcos, dsin, heads, bias=db, inplace=True)
+  assert q2.data_ptr() == buf.data_ptr() and v2.data_ptr() == buf.data_ptr() + 2 * N * 2
+  assert torch.equal(q2, q1) and torch.equal(k2, k1) and torch.equal(v2, v1)
+  # (d) attention straight on the strided views of the fused buffer (row stride 3*H*D) == attention on dense copies
+  out_f, lse_f = ops.flash_attention(q2, k2, v2, return_lse=True)
+  out_d, lse_d = ops.flash_attention(q1, k1, v1, return_lse=True)
+  assert torch.equal(out_f, out_d) and torch.equal(lse_f, lse_d)
+  assert out_f.is_contiguous() and out_f.reshape(B, S, N).shape == (B, S, N)  # the [B,S,H*D] rows proj_attn consumes
+
+
+def test_fused_qkv_rejects_a_bias_without_a_value_output(dev, lib):
+  import ctypes
+  from maxdiffusion_amd import _lib
+
+  P, fake = ctypes.c_void_p, ctypes.c_void_p(0x1000)
+  st = ctypes.byref(_lib.Strides(8 * 1536, 1536, 128))
+  args = lambda bias, v_out, stride: (None, fake, bias, fake, fake, v_out, fake, fake, None, None, 1, 8, 4, 128, 1e-6, 1.0, 0, stride, st)
+  assert lib.mdattn_norm_rope_qkv(*args(fake, None, 1536)) == _lib.E_BADARG      # bias but nowhere to put v + bias
+  assert lib.mdattn_norm_rope_qkv(*args(None, None, 1024)) == _lib.E_BADARG      # row stride below 3*H*D
+  assert lib.mdattn_norm_rope_qkv(*args(P(0x1004), fake, 1536)) == _lib.E_ALIGN
