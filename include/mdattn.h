@@ -241,7 +241,7 @@ int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, const void* v8,
  *   dout, out    bf16 [B,Sq,H,D] by o_strides;  dq by q_strides;  dk by k_strides;  dv by v_strides
  *   lse          f32 [B,H,Sq] as written by the forward
  *   workspace    f32 device buffer of at least mdattn_bwd_workspace_floats(B,H,Sq) elements, 16-byte aligned
- * Requires D == 128.
+ * Requires D == 128 or D == 64 (LTX-2's audio stream).
  */
 int64_t mdattn_bwd_workspace_floats(int B, int H, int Sq);
 int mdattn_bwd_bf16(void* stream, const void* q, const void* k, const void* v, const void* out, const void* dout,
@@ -249,6 +249,19 @@ int mdattn_bwd_bf16(void* stream, const void* q, const void* k, const void* v, c
                     int B, int H, int Sq, int Skv, int D,
                     const mdattn_strides* q_strides, const mdattn_strides* k_strides,
                     const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale);
+
+/*
+ * Backward of mdattn_fwd_bf16_bias: the same gradients with the additive per-key bias of the forward (a key padding
+ * mask, models/attention_flax.py:1926-1939) inside the recomputed probabilities.  Masked keys (-inf) get dk = dv = 0;
+ * query rows without any kept key (forward: out = 0, lse = -inf) get dq = 0 and contribute nothing.
+ *   key_bias     f32 [B, bias_stride] as for mdattn_fwd_bf16_bias (entries past Skv are ignored)
+ */
+int mdattn_bwd_bf16_bias(void* stream, const void* q, const void* k, const void* v, const void* out, const void* dout,
+                         const float* lse, void* dq, void* dk, void* dv, float* workspace, int64_t workspace_floats,
+                         int B, int H, int Sq, int Skv, int D,
+                         const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                         const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
+                         const float* key_bias, int64_t bias_stride);
 
 /*
  * mdattn_bwd_bf16 for callers that cannot allocate device memory and have no workspace to hand over: code under HIP

@@ -123,6 +123,12 @@ int mdattn_xla_bwd_bf16(void* stream, const mdattn_buffer* q, const mdattn_buffe
                         const mdattn_buffer* dq, const mdattn_buffer* dk, const mdattn_buffer* dv,
                         const mdattn_buffer* workspace, float scale, char* err, int err_len);
 
+/* "mdattn_bwd_bf16_bias": (q, k, v, out, dout, lse, key_bias f32 [B, Skv rounded up to 32]) -> (dq, dk, dv, workspace) */
+int mdattn_xla_bwd_bf16_bias(void* stream, const mdattn_buffer* q, const mdattn_buffer* k, const mdattn_buffer* v,
+                             const mdattn_buffer* out, const mdattn_buffer* dout, const mdattn_buffer* lse,
+                             const mdattn_buffer* key_bias, const mdattn_buffer* dq, const mdattn_buffer* dk,
+                             const mdattn_buffer* dv, const mdattn_buffer* workspace, float scale, char* err, int err_len);
+
 /* "mdattn_bwd_bf16_static": the same without the workspace result (mdattn_bwd_bf16_static's static scratch) */
 int mdattn_xla_bwd_bf16_static(void* stream, const mdattn_buffer* q, const mdattn_buffer* k, const mdattn_buffer* v,
                                const mdattn_buffer* out, const mdattn_buffer* dout, const mdattn_buffer* lse,

@@ -44,6 +44,7 @@ SIGNATURES = {
     "mdattn_key_mask_bias": ([_P, _P, _P, _I, _I, _L, _F], _I),
     "mdattn_bwd_workspace_floats": ([_I, _I, _I], _L),
     "mdattn_bwd_bf16": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),
+    "mdattn_bwd_bf16_bias": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F, _P, _L], _I),
     "mdattn_bwd_static_max_floats": ([], _L),
     "mdattn_bwd_bf16_static": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),
     "mdattn_quant_e4m3": ([_P, _P, _P, _P, _L, _F, _I], _I),

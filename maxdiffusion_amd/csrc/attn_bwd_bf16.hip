@@ -24,13 +24,22 @@
 namespace mdattn {
 namespace {
 
-constexpr int kBD = 128;                 // head dim
 constexpr int kBT = 32;                  // stream rows per tile
-constexpr int kBGK = 4 * kBD + 32;       // group stride of the row-read layout (see attn_fwd_bf16.hip)
-constexpr int kBGV = 4 * kBD;            // group stride of the transposed-read layout
-constexpr int kBTileA = (kBT / 4) * kBGK;
-constexpr int kBTileB = (kBT / 4) * kBGV;
-constexpr int kBStage = 2 * kBTileA + kBTileB;  // elements per ring slot
+// Tile layouts of the forward's flat schedule (see attn_fwd_bf16.hip).  Head dim 128: groups of 4 rows, row-read
+// layout padded by 64 B per group (chunk c of row r at c ^ (r & 3)), transposed-read layout with 64-byte segments at
+// s ^ (r & 3).  Head dim 64 (LTX-2's audio stream): 128-byte rows, groups of 8 rows, chunk c at c ^ ((r >> 1) & 7) for
+// the row reads and at c ^ 4*((r >> 1) & 1) for the transposing reads, both unpadded.
+template <int HD>
+struct BwdLayout {
+  static constexpr int RPI = HD == 128 ? 4 : 8;                          // rows one load instruction fills
+  static constexpr int GA = HD == 128 ? 4 * 128 + 32 : 8 * 64;           // group stride, row-read layout (elements)
+  static constexpr int GB = HD == 128 ? 4 * 128 : 8 * 64;                // group stride, transposed-read layout
+  static constexpr int TileA = (kBT / RPI) * GA;
+  static constexpr int TileB = (kBT / RPI) * GB;
+  static constexpr int Stage = 2 * TileA + TileB;                        // elements per ring slot
+  static constexpr int V8 = HD == 128 ? 2 * GB : 8 * 64;                 // second transposing read: rows + 8
+  static constexpr int VH = HD == 128 ? 4 * GB : 16 * 64;                // second 16-row half of the tile
+};
 
 typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr_b;
 typedef __attribute__((ext_vector_type(8))) short s16x8_b;
@@ -57,15 +66,21 @@ struct BwdArgs {
   int64_t s1_sb, s1_ss, s1_sh, s2_sb, s2_ss, s2_sh, s3_sb, s3_ss, s3_sh;
   int64_t o_sb, o_ss, o_sh;
   float c, scale;
+  const float* bias;   // BIAS: additive per-key bias [B, bias_sb] in natural-log units (mdattn_fwd_bf16_bias)
+  int64_t bias_sb;
 };
 
 // MODE 0: dq (entity = q rows, stream = keys), 1: dk, 2: dv (entity = key rows, stream = q rows)
-template <int MODE>
+template <int MODE, int HD, bool BIAS>
 __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw_b[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw_b);
   constexpr int NW = 4;
   constexpr bool HAS2 = MODE != 2;
+  using L = BwdLayout<HD>;
+  constexpr int NJ = HD / 16;   // MFMAs per 32 x 32 block of a contraction over the head dim
+  constexpr int ND = HD / 32;   // 32-wide slabs of d = accumulators
+  constexpr int kBD = HD, kBGK = L::GA, kBGV = L::GB, kBTileA = L::TileA, kBTileB = L::TileB, kBStage = L::Stage;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -83,15 +98,15 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
   // ---- entity fragments
   int erow = r0 + l32;
   erow = erow < a.Se ? erow : a.Se - 1;
-  bf16x8 ef1[8], ef2[8];
+  bf16x8 ef1[NJ], ef2[NJ];
   {
     const __bf16* p = a.e1 + b * a.e1_sb + h * a.e1_sh + (int64_t)erow * a.e1_ss + hh * 8;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) ef1[s] = *reinterpret_cast<const bf16x8*>(p + s * 16);
+    for (int s = 0; s < NJ; ++s) ef1[s] = *reinterpret_cast<const bf16x8*>(p + s * 16);
     if constexpr (HAS2) {
       const __bf16* p2 = a.e2 + b * a.e2_sb + h * a.e2_sh + (int64_t)erow * a.e2_ss + hh * 8;
 #pragma unroll
-      for (int s = 0; s < 8; ++s) ef2[s] = *reinterpret_cast<const bf16x8*>(p2 + s * 16);
+      for (int s = 0; s < NJ; ++s) ef2[s] = *reinterpret_cast<const bf16x8*>(p2 + s * 16);
     }
   }
   const float* lrow = a.lse2 + ((int64_t)b * a.H + h) * a.Sp;
@@ -101,23 +116,29 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
     lse_e = lrow[erow];
     delta_e = drow[erow];
   }
+  // key bias in log2 units: a per-lane scalar when the keys are the entity rows, sixteen values per tile otherwise
+  [[maybe_unused]] const float* bias_row = BIAS ? a.bias + b * a.bias_sb : nullptr;
+  [[maybe_unused]] float bias_e = 0.f;
+  if constexpr (BIAS && MODE != 0) bias_e = bias_row[erow] * kLog2e;
 
   // ---- direct global -> LDS loads of one stream tile (layouts and lane maps of the forward kernel)
   const __bf16* s1p = a.s1 + b * a.s1_sb + h * a.s1_sh;
   const __bf16* s2p = HAS2 ? a.s2 + b * a.s2_sb + h * a.s2_sh : nullptr;
   const __bf16* s3p = a.s3 + b * a.s3_sb + h * a.s3_sh;
-  const int grow = lane >> 4;
-  const int acol = ((lane & 15) ^ grow) * 8;         // row-read layout: chunk c of row r at position c ^ (r & 3)
-  const int bcol = ((lane & 15) ^ (grow << 2)) * 8;  // transposed-read layout: 64-byte segment s at s ^ (r & 3)
+  constexpr int RPI = L::RPI;
+  const int grow = HD == 128 ? lane >> 4 : lane >> 3;
+  // lane -> logical 16-byte chunk stored at this lane's position (a wave fills the row groups wave, wave + NW, ...)
+  const int acol = HD == 128 ? ((lane & 15) ^ grow) * 8 : ((lane & 7) ^ ((4 * (wave & 1) + (grow >> 1)) & 7)) * 8;
+  const int bcol = HD == 128 ? ((lane & 15) ^ (grow << 2)) * 8 : ((lane & 7) ^ (((grow >> 1) & 1) << 2)) * 8;
   const unsigned smem_addr = lds_addr_of(smem);
   auto dma = [&](int slot, int t) __attribute__((always_inline)) {
     const unsigned A1 = smem_addr + (unsigned)(slot * kBStage) * 2u;
     const unsigned A2 = A1 + kBTileA * 2u;
     const unsigned Bt = A2 + kBTileA * 2u;
 #pragma unroll
-    for (int i = 0; i < (kBT / 4) / NW; ++i) {
+    for (int i = 0; i < (kBT / RPI) / NW; ++i) {
       const int g = wave + NW * i;
-      int rr = t * kBT + 4 * g + grow;
+      int rr = t * kBT + RPI * g + grow;
       rr = rr < a.Ss ? rr : a.Ss - 1;
       lds_dma16(s1p + (int64_t)rr * a.s1_ss + acol, A1 + (unsigned)(g * kBGK) * 2u);
       if constexpr (HAS2) lds_dma16(s2p + (int64_t)rr * a.s2_ss + acol, A2 + (unsigned)(g * kBGK) * 2u);
@@ -125,22 +146,31 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
     }
   };
 
-  f32x16 acc[4];
+  f32x16 acc[ND];
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < ND; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
 
   // per-lane fragment offsets (elements)
-  const int kx0 = l32 & 1, kx1 = (l32 >> 1) & 1;
-  const int k_base = (l32 >> 2) * kBGK + (l32 & 3) * kBD + (hh ^ kx0) * 8;
-  int k_off[8], v_off[4];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) k_off[j] = k_base + ((j & 1) ? -16 : 16) * kx1 + j * 16;
+  int k_off[NJ], v_off[ND];
   const int vxr = (lane & 15) >> 2;
+  if constexpr (HD == 128) {
+    const int kx0 = l32 & 1, kx1 = (l32 >> 1) & 1;
+    const int k_base = (l32 >> 2) * kBGK + (l32 & 3) * kBD + (hh ^ kx0) * 8;
 #pragma unroll
-  for (int sg = 0; sg < 4; ++sg)
-    v_off[sg] = 2 * kBTileA + hh * kBGV + vxr * kBD + (sg ^ vxr) * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+    for (int j = 0; j < NJ; ++j) k_off[j] = k_base + ((j & 1) ? -16 : 16) * kx1 + j * 16;
+#pragma unroll
+    for (int sg = 0; sg < ND; ++sg)
+      v_off[sg] = 2 * kBTileA + hh * kBGV + vxr * kBD + (sg ^ vxr) * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+  } else {
+    const int kx = (l32 >> 1) & 7, vx = (vxr >> 1) & 1;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) k_off[j] = l32 * 64 + (((2 * j + hh) ^ kx) * 8);
+#pragma unroll
+    for (int sg = 0; sg < ND; ++sg)
+      v_off[sg] = 2 * kBTileA + (4 * hh + vxr) * 64 + (sg ^ vx) * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+  }
 
   dma(0, 0);
   for (int t = 0; t < nt; ++t) {
@@ -153,13 +183,13 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) { S[i] = 0.f; dP[i] = 0.f; }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       const bf16x8 f = *reinterpret_cast<const bf16x8*>(base + k_off[j]);
       S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, ef1[j], S, 0, 0, 0);
     }
     if constexpr (HAS2) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         const bf16x8 f = *reinterpret_cast<const bf16x8*>(base + kBTileA + k_off[j]);
         dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, ef2[j], dP, 0, 0, 0);
       }
@@ -169,11 +199,22 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
     if constexpr (MODE == 0) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) { ls[i] = lse_e; dl[i] = delta_e; }
+      if constexpr (BIAS) {  // the tile's keys: subtracting the bias from lse adds it to the logit
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_row + t * kBT + 8 * g + 4 * hh);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) ls[4 * g + e] -= bv[e] * kLog2e;
+        }
+      }
       if (t == nt - 1) {  // keys past the end of a ragged last tile take no part
         const int sbase = t * kBT + 4 * hh;
 #pragma unroll
         for (int i = 0; i < 16; ++i)
-          if (sbase + 8 * (i >> 2) + (i & 3) >= a.Ss) S[i] = -INFINITY;
+          if (sbase + 8 * (i >> 2) + (i & 3) >= a.Ss) {
+            S[i] = -INFINITY;
+            if constexpr (BIAS) ls[i] = INFINITY;  // whatever the bias padding holds
+          }
       }
     } else {
 #pragma unroll
@@ -181,7 +222,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
         const f32x4 lv = *reinterpret_cast<const f32x4*>(lrow + t * kBT + 8 * g + 4 * hh);
         const f32x4 dv = *reinterpret_cast<const f32x4*>(drow + t * kBT + 8 * g + 4 * hh);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { ls[4 * g + e] = lv[e]; dl[4 * g + e] = dv[e]; }
+        for (int e = 0; e < 4; ++e) { ls[4 * g + e] = lv[e] - (BIAS ? bias_e : 0.f); dl[4 * g + e] = dv[e]; }
       }
     }
     bf16x8 W[2];
@@ -197,10 +238,10 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
       W[hb] = __builtin_bit_cast(bf16x8, pack8(wv));
     }
 #pragma unroll
-    for (int jv = 0; jv < 8; ++jv) {
-      const __bf16* src = base + v_off[jv & 3] + (jv >> 2) * 4 * kBGV;
-      const bf16x8 f = read_vt_b(src, src + 2 * kBGV);
-      acc[jv & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, W[jv >> 2], acc[jv & 3], 0, 0, 0);
+    for (int jv = 0; jv < 2 * ND; ++jv) {
+      const __bf16* src = base + v_off[jv % ND] + (jv / ND) * L::VH;
+      const bf16x8 f = read_vt_b(src, src + L::V8);
+      acc[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, W[jv / ND], acc[jv % ND], 0, 0, 0);
     }
   }
 
@@ -209,7 +250,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
   if (row < a.Se) {
     __bf16* orow = a.out + b * a.o_sb + h * a.o_sh + (int64_t)row * a.o_ss + 4 * hh;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < ND; ++db)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         uint2 u;
@@ -220,10 +261,11 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
   }
 }
 
-// delta[b,h,q] = sum_d dout*out, lse2 = lse*log2(e); rows q in [Sq, Sp) get delta 0, lse2 +inf.  16 lanes per row.
+// delta[b,h,q] = sum_d dout*out, lse2 = lse*log2(e); rows q in [Sq, Sp) get delta 0, lse2 +inf.  16 lanes per row
+// (head dim 64: the upper 8 stay idle).
 __global__ __launch_bounds__(256) void bwd_prep_kernel(const __bf16* out, const __bf16* dout, const float* lse,
-                                                       float* lse2, float* delta, int H, int Sq, int Sp, int64_t rows,
-                                                       int64_t o_sb, int64_t o_ss, int64_t o_sh) {
+                                                       float* lse2, float* delta, int H, int Sq, int Sp, int D,
+                                                       int64_t rows, int64_t o_sb, int64_t o_ss, int64_t o_sh) {
   const int64_t r = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   if (r >= rows) return;
   const int lane = threadIdx.x & 15;
@@ -232,7 +274,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const __bf16* out, const 
   const int h = (int)(bh % H);
   const int64_t b = bh / H;
   float acc = 0.f;
-  if (q < Sq) {
+  if (q < Sq && lane * 8 < D) {
     const int64_t off = b * o_sb + (int64_t)q * o_ss + h * o_sh + lane * 8;
     float x[8], y[8];
     unpack8(*reinterpret_cast<const uint4*>(out + off), x);
@@ -243,23 +285,31 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const __bf16* out, const 
   acc = row16_sum(acc);
   if (lane == 0) {
     delta[r] = q < Sq ? acc : 0.f;
-    lse2[r] = q < Sq ? lse[bh * Sq + q] * kLog2e : INFINITY;
+    // padded rows, and rows whose keys were all masked (the forward wrote lse = -inf, out = 0), take no part: p = 0
+    const float lv = q < Sq ? lse[bh * Sq + q] : -INFINITY;
+    lse2[r] = lv > -INFINITY ? lv * kLog2e : INFINITY;
   }
 }
 
-template <int MODE>
+template <int MODE, int HD, bool BIAS>
 int launch_bwd(hipStream_t st, BwdArgs a, int B) {
-  constexpr int lds_bytes = 2 * kBStage * 2;
+  constexpr int lds_bytes = 2 * BwdLayout<HD>::Stage * 2;
   a.net = (a.Se + 127) / 128;
   const int64_t total = (int64_t)B * a.H * a.net;
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
-  auto kern = attn_bwd_kernel<MODE>;
+  auto kern = attn_bwd_kernel<MODE, HD, BIAS>;
   static LdsOptIn opted;
   if (lds_opt_in(opted, reinterpret_cast<const void*>(kern), lds_bytes) != MDATTN_OK) return MDATTN_E_LAUNCH;
   hipLaunchKernelGGL(kern, dim3(a.chunk * 8), dim3(256), lds_bytes, st, a);
   return launch_status();
+}
+
+template <int MODE>
+int launch_bwd_any(hipStream_t st, const BwdArgs& a, int B, int D) {
+  if (D == 128) return a.bias ? launch_bwd<MODE, 128, true>(st, a, B) : launch_bwd<MODE, 128, false>(st, a, B);
+  return a.bias ? launch_bwd<MODE, 64, true>(st, a, B) : launch_bwd<MODE, 64, false>(st, a, B);
 }
 
 }  // namespace
@@ -277,12 +327,17 @@ static int bwd_run(hipStream_t st, const void* q, const void* k, const void* v, 
                    const float* lse, void* dq, void* dk, void* dv, float* workspace, int64_t workspace_floats,
                    int B, int H, int Sq, int Skv, int D,
                    const mdattn_strides* q_strides, const mdattn_strides* k_strides,
-                   const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
+                   const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
+                   const float* key_bias, int64_t bias_stride) {
   if (!q || !k || !v || !out || !dout || !lse || !dq || !dk || !dv || !workspace) return MDATTN_E_BADARG;
+  if (key_bias) {
+    if (bias_stride < ((int64_t)Skv + 31) / 32 * 32 || bias_stride % 32 != 0) return MDATTN_E_BADARG;
+    if (!aligned16(key_bias)) return MDATTN_E_ALIGN;
+  }
   if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return MDATTN_E_BADARG;
   if (!q_strides || !k_strides || !v_strides || !o_strides) return MDATTN_E_BADARG;
   if (!(scale > 0.f) || !(scale < 1e30f)) return MDATTN_E_BADARG;
-  if (D != kBD) return MDATTN_E_UNSUPPORTED;
+  if (D != 128 && D != 64) return MDATTN_E_UNSUPPORTED;
   if (workspace_floats < mdattn_bwd_workspace_floats(B, H, Sq)) return MDATTN_E_BADARG;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || !aligned16(dout) || !aligned16(dq) ||
       !aligned16(dk) || !aligned16(dv) || !aligned16(workspace) || (reinterpret_cast<uintptr_t>(lse) & 3u))
@@ -297,11 +352,12 @@ static int bwd_run(hipStream_t st, const void* q, const void* k, const void* v, 
   const int64_t rows = (int64_t)B * H * Sp;
   if ((rows + 15) / 16 > 0x7FFFFFFF) return MDATTN_E_UNSUPPORTED;
   hipLaunchKernelGGL(bwd_prep_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const __bf16*)out,
-                     (const __bf16*)dout, lse, lse2, delta, H, Sq, Sp, rows, o_strides->batch, o_strides->seq, o_strides->head);
+                     (const __bf16*)dout, lse, lse2, delta, H, Sq, Sp, D, rows, o_strides->batch, o_strides->seq, o_strides->head);
   if (launch_status() != MDATTN_OK) return MDATTN_E_LAUNCH;
 
   BwdArgs a;
   a.lse2 = lse2; a.delta = delta; a.H = H; a.Sp = Sp; a.c = scale * kLog2e; a.scale = scale;
+  a.bias = key_bias; a.bias_sb = bias_stride;
   auto set = [](int64_t& sb, int64_t& ss, int64_t& sh, const mdattn_strides* s) { sb = s->batch; ss = s->seq; sh = s->head; };
   // dq: entity q / dout, stream k (scores), v (dP), k (accumulate)
   a.e1 = (const __bf16*)q; a.e2 = (const __bf16*)dout; a.s1 = (const __bf16*)k; a.s2 = (const __bf16*)v; a.s3 = (const __bf16*)k;
@@ -309,7 +365,7 @@ static int bwd_run(hipStream_t st, const void* q, const void* k, const void* v, 
   set(a.e1_sb, a.e1_ss, a.e1_sh, q_strides); set(a.e2_sb, a.e2_ss, a.e2_sh, o_strides);
   set(a.s1_sb, a.s1_ss, a.s1_sh, k_strides); set(a.s2_sb, a.s2_ss, a.s2_sh, v_strides); set(a.s3_sb, a.s3_ss, a.s3_sh, k_strides);
   set(a.o_sb, a.o_ss, a.o_sh, q_strides);
-  int rc = launch_bwd<0>(st, a, B);
+  int rc = launch_bwd_any<0>(st, a, B, D);
   if (rc != MDATTN_OK) return rc;
   // dk: entity k / v, stream q (scores), dout (dP), q (accumulate)
   a.e1 = (const __bf16*)k; a.e2 = (const __bf16*)v; a.s1 = (const __bf16*)q; a.s2 = (const __bf16*)dout; a.s3 = (const __bf16*)q;
@@ -317,14 +373,14 @@ static int bwd_run(hipStream_t st, const void* q, const void* k, const void* v, 
   set(a.e1_sb, a.e1_ss, a.e1_sh, k_strides); set(a.e2_sb, a.e2_ss, a.e2_sh, v_strides);
   set(a.s1_sb, a.s1_ss, a.s1_sh, q_strides); set(a.s2_sb, a.s2_ss, a.s2_sh, o_strides); set(a.s3_sb, a.s3_ss, a.s3_sh, q_strides);
   set(a.o_sb, a.o_ss, a.o_sh, k_strides);
-  rc = launch_bwd<1>(st, a, B);
+  rc = launch_bwd_any<1>(st, a, B, D);
   if (rc != MDATTN_OK) return rc;
   // dv: entity k, stream q (scores), dout (accumulate)
   a.e2 = nullptr; a.s2 = nullptr; a.s3 = (const __bf16*)dout;
   a.out = (__bf16*)dv;
   set(a.s3_sb, a.s3_ss, a.s3_sh, o_strides);
   set(a.o_sb, a.o_ss, a.o_sh, v_strides);
-  return launch_bwd<2>(st, a, B);
+  return launch_bwd_any<2>(st, a, B, D);
 }
 
 
@@ -334,7 +390,18 @@ extern "C" int mdattn_bwd_bf16(void* stream, const void* q, const void* k, const
                                const mdattn_strides* q_strides, const mdattn_strides* k_strides,
                                const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale) {
   return bwd_run((hipStream_t)stream, q, k, v, out, dout, lse, dq, dk, dv, workspace, workspace_floats, B, H, Sq, Skv, D,
-                 q_strides, k_strides, v_strides, o_strides, scale);
+                 q_strides, k_strides, v_strides, o_strides, scale, nullptr, 0);
+}
+
+extern "C" int mdattn_bwd_bf16_bias(void* stream, const void* q, const void* k, const void* v, const void* out, const void* dout,
+                                    const float* lse, void* dq, void* dk, void* dv, float* workspace, int64_t workspace_floats,
+                                    int B, int H, int Sq, int Skv, int D,
+                                    const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                                    const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
+                                    const float* key_bias, int64_t bias_stride) {
+  if (!key_bias) return MDATTN_E_BADARG;
+  return bwd_run((hipStream_t)stream, q, k, v, out, dout, lse, dq, dk, dv, workspace, workspace_floats, B, H, Sq, Skv, D,
+                 q_strides, k_strides, v_strides, o_strides, scale, key_bias, bias_stride);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -384,5 +451,5 @@ extern "C" int mdattn_bwd_bf16_static(void* stream, const void* q, const void* k
   float* ws = scratch_on_current_device();
   if (!ws) return MDATTN_E_LAUNCH;
   return bwd_run((hipStream_t)stream, q, k, v, out, dout, lse, dq, dk, dv, ws, need, B, H, Sq, Skv, D,
-                 q_strides, k_strides, v_strides, o_strides, scale);
+                 q_strides, k_strides, v_strides, o_strides, scale, nullptr, 0);
 }

@@ -120,6 +120,13 @@ ffi::Error BwdBf16(hipStream_t s, Buf q, Buf k, Buf v, Buf out, Buf dout, Buf ls
                       ws = Out(workspace);
   return m.done(mdattn_xla_bwd_bf16(s, &a, &b, &c, &o, &d, &l, &gq, &gk, &gv, &ws, scale, m.text, sizeof m.text));
 }
+ffi::Error BwdBf16Bias(hipStream_t s, Buf q, Buf k, Buf v, Buf out, Buf dout, Buf lse, Buf key_bias, Res dq, Res dk, Res dv, Res workspace,
+                       float scale) {
+  Msg m;
+  const mdattn_buffer a = In(q), b = In(k), c = In(v), o = In(out), d = In(dout), l = In(lse), kb = In(key_bias), gq = Out(dq),
+                      gk = Out(dk), gv = Out(dv), ws = Out(workspace);
+  return m.done(mdattn_xla_bwd_bf16_bias(s, &a, &b, &c, &o, &d, &l, &kb, &gq, &gk, &gv, &ws, scale, m.text, sizeof m.text));
+}
 ffi::Error BwdBf16Static(hipStream_t s, Buf q, Buf k, Buf v, Buf out, Buf dout, Buf lse, Res dq, Res dk, Res dv, float scale) {
   Msg m;
   const mdattn_buffer a = In(q), b = In(k), c = In(v), o = In(out), d = In(dout), l = In(lse), gq = Out(dq), gk = Out(dk), gv = Out(dv);
@@ -168,6 +175,9 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnFwdFp8, FwdFp8,
                                   .Attr<float>("scale").Attr<int64_t>("layout").Attr<int64_t>("softmax_mode"));
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnBwdBf16, BwdBf16,
                               MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>()
+                                  .Ret<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>().Attr<float>("scale"));
+XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnBwdBf16Bias, BwdBf16Bias,
+                              MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>()
                                   .Ret<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>().Attr<float>("scale"));
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnBwdBf16Static, BwdBf16Static,
                               MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>()

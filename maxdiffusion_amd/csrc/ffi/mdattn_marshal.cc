@@ -437,6 +437,29 @@ extern "C" int mdattn_xla_bwd_bf16(void* stream, const mdattn_buffer* q, const m
                                 (int)vq.S, (int)vk.S, (int)vq.D, &vq.st, &vk.st, &vk.st, &vq.st, scale));
 }
 
+extern "C" int mdattn_xla_bwd_bf16_bias(void* stream, const mdattn_buffer* q, const mdattn_buffer* k, const mdattn_buffer* v,
+                                        const mdattn_buffer* out, const mdattn_buffer* dout, const mdattn_buffer* lse,
+                                        const mdattn_buffer* key_bias, const mdattn_buffer* dq, const mdattn_buffer* dk,
+                                        const mdattn_buffer* dv, const mdattn_buffer* workspace, float scale, char* err,
+                                        int err_len) {
+  const Err e{err, err_len, "mdattn_bwd_bf16_bias"};
+  View4 vq, vk;
+  TRY(check_bwd(e, q, k, v, out, dout, lse, dq, dk, dv, &vq, &vk));
+  CHECK_BUF(e, workspace, "workspace");
+  CHECK_DT(e, workspace, "workspace", MDATTN_DT_F32);
+  const int64_t need = mdattn_bwd_workspace_floats((int)vq.B, (int)vq.H, (int)vq.S);
+  if (count(workspace) < need) return e.fail(MDATTN_E_BADARG, "workspace must hold at least %lld floats, got %lld", (long long)need, (long long)count(workspace));
+  CHECK_BUF(e, key_bias, "key_bias");
+  CHECK_DT(e, key_bias, "key_bias", MDATTN_DT_F32);
+  const int64_t padded = (vk.S + 31) / 32 * 32;
+  if (key_bias->rank != 2 || key_bias->dims[0] != vq.B || key_bias->dims[1] != padded)
+    return e.fail(MDATTN_E_BADARG, "key_bias must be [B, Skv rounded up to 32] = [%lld,%lld]", (long long)vq.B, (long long)padded);
+  return e.from(mdattn_bwd_bf16_bias(stream, q->data, k->data, v->data, out->data, dout->data, static_cast<const float*>(lse->data),
+                                     dq->data, dk->data, dv->data, static_cast<float*>(workspace->data), count(workspace), (int)vq.B,
+                                     (int)vq.H, (int)vq.S, (int)vk.S, (int)vq.D, &vq.st, &vk.st, &vk.st, &vq.st, scale,
+                                     static_cast<const float*>(key_bias->data), padded));
+}
+
 extern "C" int mdattn_xla_bwd_bf16_static(void* stream, const mdattn_buffer* q, const mdattn_buffer* k, const mdattn_buffer* v,
                                           const mdattn_buffer* out, const mdattn_buffer* dout, const mdattn_buffer* lse,
                                           const mdattn_buffer* dq, const mdattn_buffer* dk, const mdattn_buffer* dv, float scale,

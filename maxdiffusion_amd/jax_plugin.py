@@ -35,6 +35,7 @@ FFI_TARGETS = {
     "mdattn_quant_e4m3": "MdattnQuantE4m3",
     "mdattn_fwd_fp8": "MdattnFwdFp8",
     "mdattn_bwd_bf16": "MdattnBwdBf16",
+    "mdattn_bwd_bf16_bias": "MdattnBwdBf16Bias",
     "mdattn_bwd_bf16_static": "MdattnBwdBf16Static",
 }
 # entry points of mdattn.h that are host-side helpers, not kernels: no custom call
@@ -173,30 +174,45 @@ def hip_finalize(o_run):
   return call(o_run)
 
 
-def hip_flash_attention_vjp(q, k, v, scale: float, static_scratch: bool = False):
+def hip_flash_attention_vjp(q, k, v, scale: float, static_scratch: bool = False, keep_mask=None):
   """Differentiable attention on [B,S,H,D] bf16 arrays: jax.custom_vjp around the forward and backward custom calls
   (what kernels/splash_attention/splash_attention_kernel.py:1277-1600 does for the Pallas kernel).  static_scratch:
-  the backward that needs no workspace result (its scratch is a static device array of the library)."""
+  the backward that needs no workspace result (its scratch is a static device array of the library); keep_mask: a
+  [B,Skv] key padding mask, honoured by the forward and the backward alike."""
   jax, jnp = _require_jax()
+  bias = hip_key_mask_bias(keep_mask) if keep_mask is not None else None
+
+  def forward(q, k, v):
+    if bias is None:
+      return hip_flash_attention(q, k, v, scale, 0)
+    b, sq, h, d = q.shape
+    call = jax.ffi.ffi_call("mdattn_fwd_bf16_bias", (jax.ShapeDtypeStruct((b, sq, h, d), jnp.bfloat16), jax.ShapeDtypeStruct((b, h, sq), jnp.float32)),
+                            vmap_method="sequential")
+    return call(q, k, v, bias, scale=_f32(scale), layout=_i64(0))
 
   @jax.custom_vjp
   def attn(q, k, v):
-    return hip_flash_attention(q, k, v, scale, 0)[0]
+    return forward(q, k, v)[0]
 
   def fwd(q, k, v):
-    out, lse = hip_flash_attention(q, k, v, scale, 0)
+    out, lse = forward(q, k, v)
     return out, (q, k, v, out, lse)
 
   def bwd(res, dout):
     q, k, v, out, lse = res
     b, sq, h, d = q.shape
     grads = (jax.ShapeDtypeStruct(q.shape, jnp.bfloat16), jax.ShapeDtypeStruct(k.shape, jnp.bfloat16), jax.ShapeDtypeStruct(v.shape, jnp.bfloat16))
-    if static_scratch:
+    if static_scratch and bias is None:
       call = jax.ffi.ffi_call("mdattn_bwd_bf16_static", grads, vmap_method="sequential")
       return tuple(call(q, k, v, out, dout.astype(jnp.bfloat16), lse, scale=_f32(scale)))
     nws = 2 * b * h * ((sq + 31) // 32 * 32)  # mdattn_bwd_workspace_floats
-    call = jax.ffi.ffi_call("mdattn_bwd_bf16", grads + (jax.ShapeDtypeStruct((nws,), jnp.float32),), vmap_method="sequential")
-    dq, dk, dv, _ = call(q, k, v, out, dout.astype(jnp.bfloat16), lse, scale=_f32(scale))
+    results = grads + (jax.ShapeDtypeStruct((nws,), jnp.float32),)
+    if bias is not None:
+      call = jax.ffi.ffi_call("mdattn_bwd_bf16_bias", results, vmap_method="sequential")
+      dq, dk, dv, _ = call(q, k, v, out, dout.astype(jnp.bfloat16), lse, bias, scale=_f32(scale))
+    else:
+      call = jax.ffi.ffi_call("mdattn_bwd_bf16", results, vmap_method="sequential")
+      dq, dk, dv, _ = call(q, k, v, out, dout.astype(jnp.bfloat16), lse, scale=_f32(scale))
     return dq, dk, dv
 
   attn.defvjp(fwd, bwd)

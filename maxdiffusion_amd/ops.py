@@ -243,9 +243,10 @@ def flash_attention(q, k, v, scale: float | None = None, return_lse: bool = Fals
   return (out, lse) if return_lse else out
 
 
-def flash_attention_backward(q, k, v, out, dout, lse, scale: float | None = None):
+def flash_attention_backward(q, k, v, out, dout, lse, scale: float | None = None, key_bias: torch.Tensor | None = None):
   """Gradients of `flash_attention`: q, out, dout [B,Sq,H,D]; k, v [B,Skv,H,D] logical views, bf16; lse f32 [B,H,Sq] as
-  returned by the forward.  out and dout must share strides.  Returns (dq, dk, dv) shaped and laid out like q, k, v."""
+  returned by the forward; `key_bias` the additive key bias the forward was given, if any.  Returns (dq, dk, dv) shaped
+  and laid out like q, k, v."""
   _check_dev(q, k, v, out, dout, lse)
   if not all(t.dtype == torch.bfloat16 for t in (q, k, v, out, dout)):
     raise ValueError("flash_attention_backward needs bf16 q, k, v, out, dout")
@@ -265,10 +266,15 @@ def flash_attention_backward(q, k, v, out, dout, lse, scale: float | None = None
   nws = lib.mdattn_bwd_workspace_floats(b, h, sq)
   ws = torch.empty(nws, dtype=torch.float32, device=q.device)
   sq_, sk_, sv_, so_ = _strides(q), _strides(k), _strides(v), _strides(out)
-  rc = lib.mdattn_bwd_bf16(
-      _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), nws,
-      b, h, sq, skv, d, ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale))
-  _lib.check(rc, "mdattn_bwd_bf16")
+  args = (_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), nws,
+          b, h, sq, skv, d, ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale))
+  if key_bias is None:
+    _lib.check(lib.mdattn_bwd_bf16(*args), "mdattn_bwd_bf16")
+  else:
+    _check_dev(key_bias)
+    if key_bias.dtype != torch.float32 or tuple(key_bias.shape) != (b, (skv + 31) // 32 * 32) or key_bias.stride(1) != 1:
+      raise ValueError("key_bias must be the f32 [batch, kv_length rounded up to 32] tensor the forward was given")
+    _lib.check(lib.mdattn_bwd_bf16_bias(*args, _ptr(key_bias), key_bias.stride(0)), "mdattn_bwd_bf16_bias")
   return dq, dk, dv
 
 

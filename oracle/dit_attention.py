@@ -371,15 +371,21 @@ def norm_rope_ltx2(x, w, cos, sin, mode: str, eps: float = 1e-6, dtype=np.float6
 
 
 # --------------------------------------------------------------------------- backward
-def attention_bwd(q, k, v, do, scale: float, dtype=np.float64):
+def attention_bwd(q, k, v, do, scale: float, dtype=np.float64, kv_mask=None):
   """Gradients of `attention` w.r.t. q, k, v for an upstream gradient `do` of the output.
 
   kernels/splash_attention/base.py:108-160 (`_attention_reference_custom_bwd`, "flash" form
   di = rowsum(o * do)) with the dispatcher's `scale` applied inside: logits = scale * q k^T.
-  q, do [H,Sq,D]; k, v [H,Skv,D] -> (dq, dk, dv).
+  q, do [H,Sq,D]; k, v [H,Skv,D] -> (dq, dk, dv).  kv_mask [Skv] bool keeps keys (as in `attention`): masked keys
+  get no probability, hence dk = dv = 0 for them; with no kept key at all every gradient is 0.
   """
   q, k, v, do = (np.asarray(x, dtype) for x in (q, k, v, do))
   s = np.matmul(q, np.swapaxes(k, -1, -2)) * dtype(scale)
+  if kv_mask is not None:
+    keep = np.asarray(kv_mask, bool)
+    if not keep.any():
+      return np.zeros_like(q), np.zeros_like(k), np.zeros_like(v)
+    s = np.where(keep[None, None, :], s, -np.inf)
   m = s.max(axis=-1, keepdims=True)
   e = np.exp(s - m)
   lse = m + np.log(e.sum(axis=-1, keepdims=True))

@@ -160,6 +160,7 @@ def test_python_wrappers_follow_the_bind_lines(fake_jax):
   P.hip_finalize(o_run)
   P.hip_flash_attention_vjp(q, k, v, 0.1)                                      # fwd_bf16 + bwd_bf16
   P.hip_flash_attention_vjp(q, k, v, 0.1, static_scratch=True)                 # fwd_bf16 + bwd_bf16_static
+  P.hip_flash_attention_vjp(q, k, v, 0.1, keep_mask=mask)                      # key_mask_bias + fwd_bf16_bias + bwd_bf16_bias
   P.hip_norm_rope_fullrow(q3, q3, w, w, tab, tab, H)
   P.hip_norm_rope_fullrow(q3, None, w, None, None, None, H)                    # norm only, cached K/V
   P.hip_norm_rope_perhead(q, q, wd, wd, tab, tab, wq_txt=wd, wk_txt=wd, n_txt=7)

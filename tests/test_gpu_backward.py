@@ -117,3 +117,59 @@ def test_backward_golden(dev):
   _check(to_np(dq), g["dq"], "golden dq")
   _check(to_np(dk), g["dk"], "golden dk")
   _check(to_np(dv), g["dv"], "golden dv")
+
+
+@pytest.mark.parametrize("sq,skv", [(1, 1), (31, 65), (257, 63), (300, 333), (513, 512)])
+def test_backward_head_dim_64(dev, sq, skv):
+  # LTX-2's audio stream: heads of 64 (models/ltx2/transformer_ltx2.py:788-789)
+  B, H, D = 2, 3, 64
+  q, do = O.normal_bf16((B, sq, H, D), 0), O.normal_bf16((B, sq, H, D), 3)
+  k, v = O.normal_bf16((B, skv, H, D), 1), O.normal_bf16((B, skv, H, D), 2)
+  for layout in ("bshd", "bhsd"):
+    dq, dk, dv = _run(q, k, v, do, dev, layout=layout)
+    for b in range(B):
+      rq, rk, rv = O.attention_bwd(hsd(q[b:b + 1]), hsd(k[b:b + 1]), hsd(v[b:b + 1]), hsd(do[b:b + 1]), D**-0.5)
+      _check(hsd(dq[b:b + 1]), rq, f"D=64 dq Sq={sq} Skv={skv} b{b} {layout}")
+      _check(hsd(dk[b:b + 1]), rk, f"D=64 dk Sq={sq} Skv={skv} b{b} {layout}")
+      _check(hsd(dv[b:b + 1]), rv, f"D=64 dv Sq={sq} Skv={skv} b{b} {layout}")
+
+
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("sq,skv,kind", [(70, 333, "random"), (257, 512, "prefix"), (64, 97, "holes"), (33, 64, "one"), (40, 50, "none")])
+def test_backward_with_key_mask(dev, D, sq, skv, kind):
+  """Gradients through mdattn_fwd_bf16_bias: masked keys get exactly zero dk and dv; a batch element without any kept
+  key (forward: out = 0, lse = -inf) gets zero gradients everywhere."""
+  B, H = 2, 3
+  q, do = O.normal_bf16((B, sq, H, D), 0), O.normal_bf16((B, sq, H, D), 3)
+  k, v = O.normal_bf16((B, skv, H, D), 1), O.normal_bf16((B, skv, H, D), 2)
+  rng = np.random.default_rng(5)
+  keep = np.ones((B, skv), bool)
+  if kind == "random":
+    keep = rng.random((B, skv)) < 0.6
+  elif kind == "prefix":
+    keep[0, 300:] = False
+    keep[1, 77:] = False
+  elif kind == "holes":
+    keep[0, :32] = False
+    keep[1, 32:64] = False
+    keep[1, 90:] = False
+  elif kind == "one":
+    keep[:] = False
+    keep[0, 40] = True
+    keep[1, 63] = True
+  else:  # batch 1 keeps nothing
+    keep[1] = False
+  qd, kd, vd, dod = (to_dev_bf16(x, dev) for x in (q, k, v, do))
+  bias = ops.key_mask_bias(torch.from_numpy(keep).to(dev))
+  out, lse = ops.flash_attention(qd, kd, vd, return_lse=True, key_bias=bias)
+  dq, dk, dv = (to_np(t) for t in ops.flash_attention_backward(qd, kd, vd, out, dod, lse, key_bias=bias))
+  assert np.isfinite(dq).all() and np.isfinite(dk).all() and np.isfinite(dv).all()
+  for b in range(B):
+    rq, rk, rv = O.attention_bwd(hsd(q[b:b + 1]), hsd(k[b:b + 1]), hsd(v[b:b + 1]), hsd(do[b:b + 1]), D**-0.5, kv_mask=keep[b])
+    assert not dk[b][~keep[b]].any() and not dv[b][~keep[b]].any()
+    if not keep[b].any():
+      assert not dq[b].any()
+      continue
+    _check(hsd(dq[b:b + 1]), rq, f"masked {kind} D={D} dq b{b}")
+    _check(hsd(dk[b:b + 1]), rk, f"masked {kind} D={D} dk b{b}")
+    _check(hsd(dv[b:b + 1]), rv, f"masked {kind} D={D} dv b{b}")

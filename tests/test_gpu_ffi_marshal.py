@@ -161,3 +161,8 @@ def test_backward_handlers(dev, lib):
   dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
   xla(lib, "bwd_bf16_static", q, k, v, out, dout, lse, dq, dk, dv, f(0.08))
   assert all(torch.equal(a, b) for a, b in zip((dq, dk, dv), want))
+  bias = ops.key_mask_bias(torch.rand((B, Skv), device=dev) < 0.6)
+  out, lse = ops.flash_attention(q, k, v, scale=0.08, return_lse=True, key_bias=bias)
+  want = ops.flash_attention_backward(q, k, v, out, dout, lse, scale=0.08, key_bias=bias)
+  xla(lib, "bwd_bf16_bias", q, k, v, out, dout, lse, bias, dq, dk, dv, ws, f(0.08))
+  assert all(torch.equal(a, b) for a, b in zip((dq, dk, dv), want))

@@ -447,6 +447,16 @@ def test_attention_bwd_matches_torch_autograd_and_finite_differences():
     args_p[idx], args_m[idx] = x + eps * d, x - eps * d
     fd = (f(*args_p) - f(*args_m)) / (2 * eps)
     assert abs(fd - float((g * d).sum())) <= 1e-6 * max(1.0, abs(fd))
+  # with a key mask: torch autograd through SDPA with a boolean keep-mask; masked keys get exactly zero gradients
+  keep = np.array([1, 0, 1, 1, 0, 0, 1, 1, 1, 0, 1], bool)
+  dq, dk, dv = O.attention_bwd(q, k, v, do, scale, kv_mask=keep)
+  tq, tk, tv = (torch.tensor(x, dtype=torch.float64, requires_grad=True) for x in (q, k, v))
+  out = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, attn_mask=torch.tensor(keep)[None, None, :], scale=scale)
+  out.backward(torch.tensor(do))
+  for got, t in ((dq, tq), (dk, tk), (dv, tv)):
+    np.testing.assert_allclose(got, t.grad.numpy(), rtol=1e-9, atol=1e-12)
+  assert not dk[:, ~keep].any() and not dv[:, ~keep].any() and dk[:, keep].any()
+  assert all(not g.any() for g in O.attention_bwd(q, k, v, do, scale, kv_mask=np.zeros(Skv, bool)))
 
 
 # ----------------------------------------------------------------------------- fp8 emulation
