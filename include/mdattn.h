@@ -234,6 +234,20 @@ int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, const void* v8,
                    const float* q_scale, const float* k_scale, const float* v_scale, int softmax_mode);
 
 /*
+ * mdattn_fwd_fp8 with the additive per-key bias of mdattn_fwd_bf16_bias (a key padding mask,
+ * models/attention_flax.py:1926-1939): logits = scale * q.k (de-quantised) + key_bias[b, key]; rows without any kept
+ * key give out = 0 and lse = -inf.  The bias joins the products before the multiply per logit, so this entry point
+ * always runs the exact-exponential softmax with that multiply, whatever the scales (MDATTN_FP8_SOFTMAX_EXP2
+ * semantics).  key_bias as for mdattn_fwd_bf16_bias.
+ */
+int mdattn_fwd_fp8_bias(void* stream, const void* q8, const void* k8, const void* v8, void* out, float* lse,
+                        int B, int H, int Sq, int Skv, int D,
+                        const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                        const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
+                        const float* q_scale, const float* k_scale, const float* v_scale,
+                        const float* key_bias, int64_t bias_stride);
+
+/*
  * Backward of mdattn_fwd_bf16: dq, dk, dv from (q, k, v, out, dout, lse), non-causal, no mask.  Replaces: the
  * backward of the reference's attention kernels, contract in kernels/splash_attention/base.py:108-160
  * (`_attention_reference_custom_bwd`, "flash" form of di = rowsum(o * do)) and

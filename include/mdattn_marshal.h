@@ -116,6 +116,12 @@ int mdattn_xla_fwd_fp8(void* stream, const mdattn_buffer* q8, const mdattn_buffe
                        const mdattn_buffer* out, const mdattn_buffer* lse, float scale, int64_t layout,
                        int64_t softmax_mode, char* err, int err_len);
 
+/* "mdattn_fwd_fp8_bias": (q8, k8, v8, q_scale, k_scale, v_scale, key_bias f32 [B, Skv rounded up to 32]) -> (out, lse) */
+int mdattn_xla_fwd_fp8_bias(void* stream, const mdattn_buffer* q8, const mdattn_buffer* k8, const mdattn_buffer* v8,
+                            const mdattn_buffer* q_scale, const mdattn_buffer* k_scale, const mdattn_buffer* v_scale,
+                            const mdattn_buffer* key_bias, const mdattn_buffer* out, const mdattn_buffer* lse, float scale,
+                            int64_t layout, char* err, int err_len);
+
 /* "mdattn_bwd_bf16": (q, k, v, out, dout bf16 [B,S,H,D], lse f32 [B,H,Sq]) -> (dq, dk, dv bf16, workspace f32
  * [mdattn_bwd_workspace_floats(B,H,Sq)]): XLA allocates the workspace as a fourth result */
 int mdattn_xla_bwd_bf16(void* stream, const mdattn_buffer* q, const mdattn_buffer* k, const mdattn_buffer* v,

@@ -49,6 +49,7 @@ SIGNATURES = {
     "mdattn_bwd_bf16_static": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),
     "mdattn_quant_e4m3": ([_P, _P, _P, _P, _L, _F, _I], _I),
     "mdattn_fwd_fp8": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F, _P, _P, _P, _I], _I),
+    "mdattn_fwd_fp8_bias": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F, _P, _P, _P, _P, _L], _I),
     "mdattn_merge": ([_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S], _I),
     "mdattn_fwd_bf16_merge": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),
     "mdattn_finalize": ([_P, _P, _P, _L], _I),

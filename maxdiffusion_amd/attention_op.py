@@ -70,13 +70,22 @@ def _as_bshd(x: torch.Tensor, heads: int) -> torch.Tensor:
   raise ValueError(f"attention inputs must have rank 3 or 4, got {x.dim()}")
 
 
-def _reject_unsupported(context, masks_ok: bool) -> None:
-  # The custom kernels of the reference raise NotImplementedError for masks they cannot honour
+def _reject_unsupported(context) -> None:
+  # The custom kernels of the reference raise NotImplementedError for what they cannot honour
   # (attention_flax.py:850-854, :1300-1304); these kernels are non-causal.
-  if context.get("attention_mask") is not None and not masks_ok:
-    raise NotImplementedError("hip_flash_fp8 does not take an attention_mask")
   if context.get("is_causal"):
     raise NotImplementedError("hip_flash is non-causal")
+
+
+def _mask_bias(context, qv, kv):
+  """context["attention_mask"] ([B,Skv] keep-mask or None) -> additive key bias for the kernels, or None."""
+  mask = context.get("attention_mask")
+  if mask is None:
+    return None
+  if tuple(mask.shape) != (qv.shape[0], kv.shape[1]):
+    # the reference's additive bias would fail to broadcast against the [B,H,Sq,Skv] scores (:1550)
+    raise ValueError(f"attention_mask must have shape [batch, kv_length] = {(qv.shape[0], kv.shape[1])}, got {tuple(mask.shape)}.")
+  return ops.key_mask_bias(mask)
 
 
 @register_kernel("hip_flash")
@@ -87,7 +96,7 @@ def hip_flash_kernel(q, k, v, context):
   to the kernel and is folded into the exp2 argument; `flash_block_sizes`, `mesh` and the axis names
   are accepted and ignored (one GPU, tiles fixed by the kernel).
   """
-  _reject_unsupported(context, masks_ok=True)
+  _reject_unsupported(context)
   heads = context["heads"]
   qv, kv, vv = _as_bshd(q, heads), _as_bshd(k, heads), _as_bshd(v, heads)
   cast = q.dtype != torch.bfloat16
@@ -95,11 +104,7 @@ def hip_flash_kernel(q, k, v, context):
     qv, kv, vv = qv.to(torch.bfloat16), kv.to(torch.bfloat16), vv.to(torch.bfloat16)
   # [B,Skv] keep-mask (attention_flax.py:1926-1939): masked keys are excluded, as the flash wrappers do with
   # segment ids (:390-438); rows without a kept key return 0 (:1552-1554)
-  mask = context.get("attention_mask")
-  if mask is not None and tuple(mask.shape) != (qv.shape[0], kv.shape[1]):
-    # the reference's additive bias would fail to broadcast against the [B,H,Sq,Skv] scores (:1550)
-    raise ValueError(f"attention_mask must have shape [batch, kv_length] = {(qv.shape[0], kv.shape[1])}, got {tuple(mask.shape)}.")
-  bias = ops.key_mask_bias(mask) if mask is not None else None
+  bias = _mask_bias(context, qv, kv)
   out = ops.flash_attention(qv, kv, vv, scale=context["scale"], key_bias=bias)
   b, s, h, d = out.shape
   out = out.reshape(b, s, h * d)
@@ -109,7 +114,7 @@ def hip_flash_kernel(q, k, v, context):
 @register_kernel("hip_flash_fp8")
 def hip_flash_fp8_kernel(q, k, v, context):
   """fp8-e4m3 variant: per-tensor absmax quantisation of q, k, v on the device, then the fp8 kernel."""
-  _reject_unsupported(context, masks_ok=False)
+  _reject_unsupported(context)
   heads = context["heads"]
   qv, kv, vv = (_as_bshd(t, heads).to(torch.bfloat16).contiguous() for t in (q, k, v))
   # the softmax scale rides on q's quantisation (one rounding either way) and the q and k scales are powers of two:
@@ -119,7 +124,8 @@ def hip_flash_fp8_kernel(q, k, v, context):
   q8, sq = ops.quant_e4m3(qv, premul=context["scale"] * math.log2(math.e), pow2_scale=True)
   k8, sk = ops.quant_e4m3(kv, pow2_scale=True)
   v8, sv = ops.quant_e4m3(vv)
-  out = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=ops.FOLDED_SCALE, softmax="byte_grid")
+  # a [B,Skv] keep-mask goes in as an additive key bias (exact-exponential softmax), as for hip_flash
+  out = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=ops.FOLDED_SCALE, softmax="byte_grid", key_bias=_mask_bias(context, qv, kv))
   b, s, h, d = out.shape
   return out.reshape(b, s, h * d).to(q.dtype)
 

@@ -66,12 +66,17 @@ struct Fp8Args {
   int64_t v_sb, v_ss, v_sh;
   int64_t o_sb, o_ss, o_sh;
   float c;  // scale * log2(e)
+  const float* bias;   // BIAS: additive per-key bias [B, bias_sb], natural-log units (-inf excludes a key)
+  int64_t bias_sb;
 };
 
 // Register budget: three waves per SIMD (<= 168 VGPRs).  The kernel is bound by the vector ALU (softmax)
 // and by latencies a single wave cannot hide, so the third wave per SIMD is worth more than registers.
-template <int NW, int MODE>
+// BIAS (MODE 0 only): an additive per-key bias (a key padding mask) joins the raw products right after the MFMAs,
+// divided by the logit scale so that the multiply per logit carries it; this instance serves every kind of scale.
+template <int NW, int MODE, bool BIAS = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_fwd_fp8_kernel(Fp8Args a) {
+  static_assert(!BIAS || MODE == 0, "the key bias lives in the path with a multiply per logit");
   constexpr bool PRE = MODE != 0;    // the logit scale is a power of two and rides in the MFMAs' block scale
   constexpr bool CODE = MODE == 2;   // ... and P is formed without exp2: see kCodeOne
   extern __shared__ __attribute__((aligned(16))) char smem8[];
@@ -96,11 +101,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   const float c = a.c * a.q_scale[0] * a.k_scale[0];
   // The scales live in device memory, so the host cannot know which of the two instances of this kernel applies:
   // it launches both, and the one whose case this is not ends here.
-  {
+  if constexpr (!BIAS) {
     const unsigned cbits = __float_as_uint(c);
     const bool c_pow2 = (cbits & 0x007FFFFFu) == 0u && cbits > 0x00800000u && cbits < 0x7F000000u;
     if (c_pow2 != PRE) return;
   }
+  [[maybe_unused]] const float* bias_row = BIAS ? a.bias + b * a.bias_sb + 4 * hh : nullptr;
+  [[maybe_unused]] const float bias_mul = kLog2e / c;            // natural-log bias -> units of the raw products
+  [[maybe_unused]] const int bias_cols = (a.Skv + 31) / 32 * 32;  // entries the caller's bias rows are sure to hold
 
   // ---- Q fragments: lane (row l32, half hh) holds bytes 64*j + 32*hh .. +31 of its row
   i32x8 qf[2];
@@ -204,6 +212,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
         for (int i = 0; i < 16; ++i) z[i] = 0.f;
         z = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[0], qf[0], z, 0, 0, 0, 0, 0, 0);
         S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], z, 0, 0, 0, 0, 0, 0);
+      }
+      if constexpr (BIAS) {
+        if (t * kBN8 + 32 * blk < bias_cols) {  // a block wholly past the keys (last tile) is masked below anyway
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_row + t * kBN8 + 32 * blk + 8 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) S[4 * g + e] = __builtin_fmaf(bv[e], bias_mul, S[4 * g + e]);
+          }
+        }
       }
       if constexpr (decltype(masked)::value) {
         const int kbase = t * kBN8 + 4 * hh + 32 * blk;
@@ -334,7 +352,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   // ---- epilogue
   __bf16* op = a.out + b * a.o_sb + h * a.o_sh;
   const float lt = xhalf_sum(l);
-  const float inv = a.v_scale[0] / lt;
+  const float inv = lt > 0.f ? a.v_scale[0] / lt : 0.f;  // rows whose keys are all excluded return 0 (and lse = -inf)
   const int row = q0 + l32;
   if (row < a.Sq) {
     __bf16* orow = op + (int64_t)row * a.o_ss + 4 * hh;
@@ -360,6 +378,10 @@ int launch_fwd8(hipStream_t st, Fp8Args a, int B, int softmax_mode) {
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
+  if (a.bias) {  // one instance for every kind of scale
+    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 0, true>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+    return launch_status();
+  }
   hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 0>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   // Power-of-two logit scale (the instance above then returns at once, this one otherwise): exp2, or the
   // exponential-free softmax when the caller asked for it.
@@ -375,11 +397,12 @@ int launch_fwd8(hipStream_t st, Fp8Args a, int B, int softmax_mode) {
 
 using namespace mdattn;
 
-extern "C" int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, const void* v8, void* out, float* lse,
-                              int B, int H, int Sq, int Skv, int D,
-                              const mdattn_strides* q_strides, const mdattn_strides* k_strides,
-                              const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
-                              const float* q_scale, const float* k_scale, const float* v_scale, int softmax_mode) {
+static int fp8_run(void* stream, const void* q8, const void* k8, const void* v8, void* out, float* lse,
+                   int B, int H, int Sq, int Skv, int D,
+                   const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                   const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
+                   const float* q_scale, const float* k_scale, const float* v_scale, int softmax_mode,
+                   const float* key_bias, int64_t bias_stride) {
   if (softmax_mode != MDATTN_FP8_SOFTMAX_EXP2 && softmax_mode != MDATTN_FP8_SOFTMAX_BYTE_GRID) return MDATTN_E_BADARG;
   if (!q8 || !k8 || !v8 || !out || !q_scale || !k_scale || !v_scale) return MDATTN_E_BADARG;
   if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return MDATTN_E_BADARG;
@@ -407,7 +430,34 @@ extern "C" int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, cons
   a.o_sb = o_strides->batch; a.o_ss = o_strides->seq; a.o_sh = o_strides->head;
   a.c = scale * kLog2e;
   if (a.c > 1.0f - 1e-6f && a.c < 1.0f + 1e-6f) a.c = 1.0f;  // scale = ln 2: the caller's q carries the softmax scale
+  a.bias = key_bias;
+  a.bias_sb = bias_stride;
+  if (key_bias) {
+    if (bias_stride < ((int64_t)Skv + 31) / 32 * 32 || bias_stride % 32 != 0) return MDATTN_E_BADARG;
+    if (!aligned16(key_bias)) return MDATTN_E_ALIGN;
+  }
   hipStream_t st = (hipStream_t)stream;
   // Four waves per workgroup (three workgroups per CU) measured faster than eight at every shape tried.
   return launch_fwd8<4>(st, a, B, softmax_mode);
+}
+
+
+extern "C" int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, const void* v8, void* out, float* lse,
+                              int B, int H, int Sq, int Skv, int D,
+                              const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                              const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
+                              const float* q_scale, const float* k_scale, const float* v_scale, int softmax_mode) {
+  return fp8_run(stream, q8, k8, v8, out, lse, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides, scale, q_scale,
+                 k_scale, v_scale, softmax_mode, nullptr, 0);
+}
+
+extern "C" int mdattn_fwd_fp8_bias(void* stream, const void* q8, const void* k8, const void* v8, void* out, float* lse,
+                                   int B, int H, int Sq, int Skv, int D,
+                                   const mdattn_strides* q_strides, const mdattn_strides* k_strides,
+                                   const mdattn_strides* v_strides, const mdattn_strides* o_strides, float scale,
+                                   const float* q_scale, const float* k_scale, const float* v_scale,
+                                   const float* key_bias, int64_t bias_stride) {
+  if (!key_bias) return MDATTN_E_BADARG;
+  return fp8_run(stream, q8, k8, v8, out, lse, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides, scale, q_scale,
+                 k_scale, v_scale, MDATTN_FP8_SOFTMAX_EXP2, key_bias, bias_stride);
 }

@@ -114,6 +114,13 @@ ffi::Error FwdFp8(hipStream_t s, Buf q8, Buf k8, Buf v8, Buf q_scale, Buf k_scal
   const mdattn_buffer a = In(q8), b = In(k8), c = In(v8), qs = In(q_scale), ks = In(k_scale), vs = In(v_scale), o = Out(out), l = Out(lse);
   return m.done(mdattn_xla_fwd_fp8(s, &a, &b, &c, &qs, &ks, &vs, &o, &l, scale, layout, softmax_mode, m.text, sizeof m.text));
 }
+ffi::Error FwdFp8Bias(hipStream_t s, Buf q8, Buf k8, Buf v8, Buf q_scale, Buf k_scale, Buf v_scale, Buf key_bias, Res out, Res lse,
+                      float scale, int64_t layout) {
+  Msg m;
+  const mdattn_buffer a = In(q8), b = In(k8), c = In(v8), qs = In(q_scale), ks = In(k_scale), vs = In(v_scale), kb = In(key_bias),
+                      o = Out(out), l = Out(lse);
+  return m.done(mdattn_xla_fwd_fp8_bias(s, &a, &b, &c, &qs, &ks, &vs, &kb, &o, &l, scale, layout, m.text, sizeof m.text));
+}
 ffi::Error BwdBf16(hipStream_t s, Buf q, Buf k, Buf v, Buf out, Buf dout, Buf lse, Res dq, Res dk, Res dv, Res workspace, float scale) {
   Msg m;
   const mdattn_buffer a = In(q), b = In(k), c = In(v), o = In(out), d = In(dout), l = In(lse), gq = Out(dq), gk = Out(dk), gv = Out(dv),
@@ -173,6 +180,9 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnQuantE4m3, QuantE4m3,
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnFwdFp8, FwdFp8,
                               MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Ret<Buf>().Ret<Buf>()
                                   .Attr<float>("scale").Attr<int64_t>("layout").Attr<int64_t>("softmax_mode"));
+XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnFwdFp8Bias, FwdFp8Bias,
+                              MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>()
+                                  .Ret<Buf>().Ret<Buf>().Attr<float>("scale").Attr<int64_t>("layout"));
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnBwdBf16, BwdBf16,
                               MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>()
                                   .Ret<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>().Attr<float>("scale"));

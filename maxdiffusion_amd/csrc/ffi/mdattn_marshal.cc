@@ -405,8 +405,34 @@ extern "C" int mdattn_xla_fwd_fp8(void* stream, const mdattn_buffer* q8, const m
                                static_cast<const float*>(v_scale->data), (int)softmax_mode));
 }
 
+extern "C" int mdattn_xla_fwd_fp8_bias(void* stream, const mdattn_buffer* q8, const mdattn_buffer* k8, const mdattn_buffer* v8,
+                                       const mdattn_buffer* q_scale, const mdattn_buffer* k_scale, const mdattn_buffer* v_scale,
+                                       const mdattn_buffer* key_bias, const mdattn_buffer* out, const mdattn_buffer* lse, float scale,
+                                       int64_t layout, char* err, int err_len) {
+  const Err e{err, err_len, "mdattn_fwd_fp8_bias"};
+  View4 vq, vk, vv, vo;
+  TRY(check_qkv(e, q8, k8, v8, layout, true, &vq, &vk, &vv));
+  TRY(check_out_bshd(e, out, "out", MDATTN_DT_BF16, vq, &vo));
+  TRY(check_lse(e, lse, "lse", vq));
+  const mdattn_buffer* sc[3] = {q_scale, k_scale, v_scale};
+  const char* names[3] = {"q_scale", "k_scale", "v_scale"};
+  for (int i = 0; i < 3; ++i) {
+    CHECK_BUF(e, sc[i], names[i]);
+    CHECK_DT(e, sc[i], names[i], MDATTN_DT_F32);
+  }
+  CHECK_BUF(e, key_bias, "key_bias");
+  CHECK_DT(e, key_bias, "key_bias", MDATTN_DT_F32);
+  const int64_t padded = (vk.S + 31) / 32 * 32;
+  if (key_bias->rank != 2 || key_bias->dims[0] != vq.B || key_bias->dims[1] != padded)
+    return e.fail(MDATTN_E_BADARG, "key_bias must be [B, Skv rounded up to 32] = [%lld,%lld]", (long long)vq.B, (long long)padded);
+  return e.from(mdattn_fwd_fp8_bias(stream, q8->data, k8->data, v8->data, out->data, static_cast<float*>(lse->data), (int)vq.B,
+                                    (int)vq.H, (int)vq.S, (int)vk.S, (int)vq.D, &vq.st, &vk.st, &vv.st, &vo.st, scale,
+                                    static_cast<const float*>(q_scale->data), static_cast<const float*>(k_scale->data),
+                                    static_cast<const float*>(v_scale->data), static_cast<const float*>(key_bias->data), padded));
+}
+
 namespace {
-// the checks the two backward handlers share; q, out, dout, dq are [B,Sq,H,D], k, v, dk, dv [B,Skv,H,D]
+// the checks the backward handlers share; q, out, dout, dq are [B,Sq,H,D], k, v, dk, dv [B,Skv,H,D]
 int check_bwd(const Err& e, const mdattn_buffer* q, const mdattn_buffer* k, const mdattn_buffer* v, const mdattn_buffer* out,
               const mdattn_buffer* dout, const mdattn_buffer* lse, const mdattn_buffer* dq, const mdattn_buffer* dk,
               const mdattn_buffer* dv, View4* vq, View4* vk) {

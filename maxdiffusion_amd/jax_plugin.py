@@ -34,6 +34,7 @@ FFI_TARGETS = {
     "mdattn_norm_rope_rows": "MdattnNormRopeRows",
     "mdattn_quant_e4m3": "MdattnQuantE4m3",
     "mdattn_fwd_fp8": "MdattnFwdFp8",
+    "mdattn_fwd_fp8_bias": "MdattnFwdFp8Bias",
     "mdattn_bwd_bf16": "MdattnBwdBf16",
     "mdattn_bwd_bf16_bias": "MdattnBwdBf16Bias",
     "mdattn_bwd_bf16_static": "MdattnBwdBf16Static",
@@ -123,9 +124,10 @@ def hip_quant_e4m3(x, premul: float = 1.0, pow2_scale: bool = False):
   return call(x.astype(jnp.bfloat16), premul=_f32(premul), pow2_scale=_i64(bool(pow2_scale)))
 
 
-def hip_flash_attention_fp8(q, k, v, scale: float, layout: int, softmax: str = "byte_grid"):
+def hip_flash_attention_fp8(q, k, v, scale: float, layout: int, softmax: str = "byte_grid", keep_mask=None):
   """BASELINE configs[4]: quantises bf16 q, k, v per tensor (q carries scale * log2(e), q and k scales are powers of
-  two) and runs the fp8-e4m3 kernel.  softmax "byte_grid" (fastest; use `out`) or "exp2" (exact lse, mergeable).
+  two) and runs the fp8-e4m3 kernel.  softmax "byte_grid" (fastest; use `out`) or "exp2" (exact lse, mergeable);
+  keep_mask [B,Skv] bool: masked keys are excluded (exact exponentials).
   Returns (out [B,Sq,H,D] bf16, lse [B,H,Sq] f32)."""
   jax, jnp = _require_jax()
   modes = {"exp2": 0, "byte_grid": 1}
@@ -135,8 +137,14 @@ def hip_flash_attention_fp8(q, k, v, scale: float, layout: int, softmax: str = "
   q8, qs = hip_quant_e4m3(q, premul=scale * math.log2(math.e), pow2_scale=True)
   k8, ks = hip_quant_e4m3(k, pow2_scale=True)
   v8, vs = hip_quant_e4m3(v)
-  call = jax.ffi.ffi_call("mdattn_fwd_fp8", (jax.ShapeDtypeStruct((b, sq, h, d), jnp.bfloat16), jax.ShapeDtypeStruct((b, h, sq), jnp.float32)),
-                          vmap_method="sequential")
+  results = (jax.ShapeDtypeStruct((b, sq, h, d), jnp.bfloat16), jax.ShapeDtypeStruct((b, h, sq), jnp.float32))
+  if keep_mask is not None:
+    skv = _bshd_dims(k, layout)[1]
+    if tuple(keep_mask.shape) != (b, skv):
+      raise ValueError(f"attention_mask must have shape [batch, kv_length] = {(b, skv)}, got {tuple(keep_mask.shape)}.")
+    call = jax.ffi.ffi_call("mdattn_fwd_fp8_bias", results, vmap_method="sequential")
+    return call(q8, k8, v8, qs, ks, vs, hip_key_mask_bias(keep_mask), scale=_f32(FOLDED_SCALE), layout=_i64(layout))
+  call = jax.ffi.ffi_call("mdattn_fwd_fp8", results, vmap_method="sequential")
   return call(q8, k8, v8, qs, ks, vs, scale=_f32(FOLDED_SCALE), layout=_i64(layout), softmax_mode=_i64(modes[softmax]))
 
 
@@ -324,15 +332,14 @@ def hip_flash_kernel(q, k, v, context):
 
 def hip_flash_fp8_kernel(q, k, v, context):
   """The KERNEL_REGISTRY entry `hip_flash_fp8` (BASELINE configs[4]): per-tensor e4m3 q, k, v on the device, then the
-  fp8 kernel.  Masks are not supported (the custom kernels of the reference raise the same way, attention_flax.py:850-854)."""
+  fp8 kernel; a [B,Skv] attention_mask is honoured like hip_flash honours it."""
   _, jnp = _require_jax()
-  if context.get("attention_mask") is not None:
-    raise NotImplementedError("hip_flash_fp8 does not take an attention_mask")
   if context.get("is_causal"):
     raise NotImplementedError("hip_flash is non-causal")
   q4, k4, v4, layout = _as_rank4(q, k, v, context["heads"])
   dt = q.dtype
-  out, _ = hip_flash_attention_fp8(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"], layout)
+  out, _ = hip_flash_attention_fp8(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"], layout,
+                                   keep_mask=context.get("attention_mask"))
   b, sq, h, d = out.shape
   return out.reshape(b, sq, h * d).astype(dt)
 

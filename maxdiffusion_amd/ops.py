@@ -323,13 +323,14 @@ FP8_SOFTMAX_MODES = {"exp2": 0, "byte_grid": 1}
 
 
 def flash_attention_fp8(q8, k8, v8, q_scale, k_scale, v_scale, scale: float | None = None, return_lse: bool = False,
-                        out_layout: str = "bshd", softmax: str = "exp2"):
+                        out_layout: str = "bshd", softmax: str = "exp2", key_bias: torch.Tensor | None = None):
   """fp8-e4m3 variant: q8/k8/v8 uint8 logical [B,S,H,D] views, *_scale device f32 tensors (element 0 is used).
 
   softmax="exp2": exact exponentials; the lse is the logsumexp of the quantised logits and the pair (out, lse) can be
   merged like a bf16 partial.  softmax="byte_grid": with power-of-two q and k scales and the softmax scale carried by
   q (see `quant_e4m3`) P is a piecewise-linear exponential read off the e4m3 byte grid (12 % faster; out keeps its
-  accuracy, the lse is only good to about 0.08); with any other scales it is the same as "exp2"."""
+  accuracy, the lse is only good to about 0.08); with any other scales it is the same as "exp2".
+  `key_bias` (see `key_mask_bias`): additive per-key bias, -inf excludes a key; always the exact-exponential softmax."""
   if softmax not in FP8_SOFTMAX_MODES:
     raise ValueError(f"softmax={softmax!r} not supported. Choose between 'exp2' and 'byte_grid'.")
   _check_dev(q8, k8, v8, q_scale, k_scale, v_scale)
@@ -340,11 +341,16 @@ def flash_attention_fp8(q8, k8, v8, q_scale, k_scale, v_scale, scale: float | No
   out = _alloc_like_layout(b, sq, h, d, out_layout, torch.bfloat16, q8.device)
   lse = torch.empty((b, h, sq), dtype=torch.float32, device=q8.device) if return_lse else None
   sq_, sk_, sv_, so_ = _strides(q8), _strides(k8), _strides(v8), _strides(out)
-  rc = _lib.load().mdattn_fwd_fp8(
-      _stream(), _ptr(q8), _ptr(k8), _ptr(v8), _ptr(out), _ptr(lse), b, h, sq, skv, d,
-      ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale),
-      _ptr(q_scale), _ptr(k_scale), _ptr(v_scale), FP8_SOFTMAX_MODES[softmax])
-  _lib.check(rc, "mdattn_fwd_fp8")
+  args = (_stream(), _ptr(q8), _ptr(k8), _ptr(v8), _ptr(out), _ptr(lse), b, h, sq, skv, d,
+          ctypes.byref(sq_), ctypes.byref(sk_), ctypes.byref(sv_), ctypes.byref(so_), float(scale),
+          _ptr(q_scale), _ptr(k_scale), _ptr(v_scale))
+  if key_bias is None:
+    _lib.check(_lib.load().mdattn_fwd_fp8(*args, FP8_SOFTMAX_MODES[softmax]), "mdattn_fwd_fp8")
+  else:
+    _check_dev(key_bias)
+    if key_bias.dtype != torch.float32 or tuple(key_bias.shape) != (b, (skv + 31) // 32 * 32) or key_bias.stride(1) != 1:
+      raise ValueError(f"key_bias must be an f32 [batch, kv_length rounded up to 32] = [{b}, {(skv + 31) // 32 * 32}] tensor")
+    _lib.check(_lib.load().mdattn_fwd_fp8_bias(*args, _ptr(key_bias), key_bias.stride(0)), "mdattn_fwd_fp8_bias")
   return (out, lse) if return_lse else out
 
 

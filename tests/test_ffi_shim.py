@@ -155,6 +155,7 @@ def test_python_wrappers_follow_the_bind_lines(fake_jax):
   P.hip_flash_attention(q, k, v, 0.1, 0)
   P.hip_flash_attention(q, k, v, 0.1, 0, keep_mask=mask)                       # key_mask_bias + fwd_bf16_bias
   P.hip_flash_attention_fp8(q, k, v, 0.1, 0, softmax="exp2")                   # 3 x quant_e4m3 + fwd_fp8
+  P.hip_flash_attention_fp8(q, k, v, 0.1, 0, keep_mask=mask)                   # ... + key_mask_bias + fwd_fp8_bias
   P.hip_ring_step(q, k, v, o_run, l_run, 0.1)
   P.hip_merge(o_run, l_run, q, l_run)
   P.hip_finalize(o_run)
@@ -193,8 +194,7 @@ def test_python_wrappers_follow_the_bind_lines(fake_jax):
   for fn in (P.hip_flash_kernel, P.hip_flash_fp8_kernel):
     out = fn(q3, k3, k3, ctx)
     assert out.shape == (B, S, H * D)
-  with pytest.raises(NotImplementedError):
-    P.hip_flash_fp8_kernel(q3, k3, k3, dict(ctx, attention_mask=mask))
+  assert P.hip_flash_fp8_kernel(q3, k3, k3, dict(ctx, attention_mask=mask)).shape == (B, S, H * D)
   with pytest.raises(NotImplementedError):
     P.hip_flash_kernel(q3, k3, k3, dict(ctx, is_causal=True))
   with pytest.raises(ValueError, match=r"\[batch, kv_length\]"):

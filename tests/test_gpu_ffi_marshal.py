@@ -146,6 +146,11 @@ def test_fp8_handlers(dev, lib, softmax):
   w_out, w_lse = ops.flash_attention_fp8(want[0][0], want[1][0], want[2][0], want[0][1], want[1][1], want[2][1],
                                          scale=ops.FOLDED_SCALE, return_lse=True, softmax=softmax)
   assert torch.equal(out, w_out) and torch.equal(lse, w_lse)
+  bias = ops.key_mask_bias(torch.rand((B, Skv), device=dev) < 0.6)
+  xla(lib, "fwd_fp8_bias", xs[0][0], xs[1][0], xs[2][0], xs[0][1], xs[1][1], xs[2][1], bias, out, lse, f(ops.FOLDED_SCALE), i(0))
+  w_out, w_lse = ops.flash_attention_fp8(want[0][0], want[1][0], want[2][0], want[0][1], want[1][1], want[2][1],
+                                         scale=ops.FOLDED_SCALE, return_lse=True, key_bias=bias)
+  assert torch.equal(out, w_out) and torch.equal(lse, w_lse)
 
 
 def test_backward_handlers(dev, lib):

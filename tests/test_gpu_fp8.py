@@ -250,3 +250,63 @@ def test_fp8_seeded_sweep_of_shapes_layouts_and_scale_kinds(dev):
     assert bool(torch.isfinite(o).all()) and bool(torch.isfinite(lse).all()), what
     assert float((o * ref).sum() / (o.norm() * ref.norm())) >= (COS_BAR if mult == 1.0 else 0.985), what
     assert float((lse - rl).abs().max()) <= (0.3 if mult == 1.0 else 2.0), what
+
+
+@pytest.mark.parametrize("sq,skv,kind", [(70, 333, "random"), (257, 512, "prefix"), (64, 97, "holes"), (33, 64, "one"), (40, 50, "none")])
+@pytest.mark.parametrize("pow2", [False, True])
+def test_fp8_with_key_mask(dev, sq, skv, kind, pow2):
+  """mdattn_fwd_fp8_bias: a [B,Skv] keep-mask as an additive key bias.  The masked result must be the attention over
+  the kept keys only: against the f32 oracle with the mask (cosine bar), and against the fp8 kernel itself run,
+  without a mask, on the kept keys of the same quantised operands (only the tiling of the keys differs, so only the
+  e4m3 rounding grid of P moves).  Batch elements without a kept key return out = 0, lse = -inf."""
+  B, H = 2, 2
+  q, k, v = O.normal_bf16((B, sq, H, 128), 0), O.normal_bf16((B, skv, H, 128), 1), O.normal_bf16((B, skv, H, 128), 2)
+  rng = np.random.default_rng(5)
+  keep = np.ones((B, skv), bool)
+  if kind == "random":
+    keep = rng.random((B, skv)) < 0.6
+  elif kind == "prefix":
+    keep[0, 300:] = False
+    keep[1, 77:] = False
+  elif kind == "holes":  # whole 64-key tiles and 32-key blocks masked out, the first tile included
+    keep[0, :64] = False
+    keep[1, 32:64] = False
+    keep[1, 90:] = False
+  elif kind == "one":
+    keep[:] = False
+    keep[0, 40] = True
+    keep[1, 63] = True
+  else:
+    keep[1] = False
+  qd, kd, vd = (to_dev_bf16(x, dev) for x in (q, k, v))
+  if pow2:
+    q8, sq_ = ops.quant_e4m3(qd, premul=ops.folded_q_mul(128), pow2_scale=True)
+    k8, sk_ = ops.quant_e4m3(kd, pow2_scale=True)
+    sc = ops.FOLDED_SCALE
+  else:
+    (q8, sq_), (k8, sk_), sc = ops.quant_e4m3(qd), ops.quant_e4m3(kd), 128**-0.5
+  v8, sv_ = ops.quant_e4m3(vd)
+  keep_d = torch.from_numpy(keep).to(dev)
+  out, lse = ops.flash_attention_fp8(q8, k8, v8, sq_, sk_, sv_, scale=sc, return_lse=True, key_bias=ops.key_mask_bias(keep_d))
+  for b in range(B):
+    if not keep[b].any():
+      assert torch.count_nonzero(out[b]) == 0 and bool(torch.isneginf(lse[b]).all())
+      continue
+    exact, lse_exact = O.attention(hsd(q[b:b + 1]), hsd(k[b:b + 1]), hsd(v[b:b + 1]), 128**-0.5, kv_mask=keep[b])
+    assert cosine(hsd(to_np(out[b:b + 1])), exact) >= COS_BAR, (kind, b)
+    assert np.abs(to_np(lse[b]) - lse_exact).max() <= 0.25
+    sub, sub_l = ops.flash_attention_fp8(q8[b:b + 1], k8[b:b + 1, keep_d[b]], v8[b:b + 1, keep_d[b]], sq_, sk_, sv_, scale=sc, return_lse=True)
+    # two runs whose reference points differ round P on two different e4m3 grids: 2.6 % rms each, independent; the
+    # row sums use the unrounded P, so the lse agrees to f32 summation order
+    assert rel_l2(to_np(out[b:b + 1]), to_np(sub)) <= 4.5e-2 and float((lse[b] - sub_l[0]).abs().max()) <= 2e-3, (kind, b)
+
+
+def test_fp8_registry_entry_honours_the_mask(dev):
+  B, S, Skv, H = 2, 90, 150, 2
+  q, k, v = (to_dev_bf16(O.normal_bf16((B, s_, H * 128), i), dev) for i, s_ in enumerate((S, Skv, Skv)))
+  keep = torch.rand((B, Skv), device=dev) < 0.5
+  op8 = attention_op.AttentionOp(attention_kernel="hip_flash_fp8", heads=H, dim_head=128, scale=128**-0.5)
+  op16 = attention_op.AttentionOp(attention_kernel="hip_flash", heads=H, dim_head=128, scale=128**-0.5)
+  got, want = op8.apply_attention(q, k, v, attention_mask=keep), op16.apply_attention(q, k, v, attention_mask=keep)
+  assert got.shape == want.shape == (B, S, H * 128)
+  assert cosine(to_np(got), to_np(want)) >= COS_BAR
