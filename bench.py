@@ -266,10 +266,10 @@ def main():
     e1.record()
     torch.cuda.synchronize()
     bms = e0.elapsed_time(e1) / 5
-    # the five matrix products of the backward pass: S, dP, dV, dK, dQ (the three passes execute eight)
+    # the five matrix products of the backward pass: S, dP, dV, dK, dQ (the two passes execute seven: S and dP are formed in both)
     bfl = 2.5 * O.attention_flops(1, H, S, Skv, D)
     backward = {"Sq": S, "Skv": Skv, "ms": bms, "TFLOP/s": bfl / (bms * 1e-3) / 1e12,
-                "flop_counted": bfl, "note": "5 matrix products counted, 8 executed (three atomic-free passes)"}
+                "flop_counted": bfl, "note": "5 matrix products counted, 7 executed (two atomic-free passes: dq; dk and dv)"}
 
   flops = O.attention_flops(1, H, S, Skv * ring, D)
   att_ms = sum(t_att) / len(t_att)

@@ -2,20 +2,24 @@
 // (q, k, v, out, dout, lse).  With logits s = scale*q.k, p = exp(s - lse), dp = dout.v^T, delta = rowsum(dout*out):
 //   dv = p^T dout,   ds = p * (dp - delta),   dq = scale * ds k,   dk = scale * ds^T q.
 //
-// One kernel, three instantiations, no atomics: every gradient is accumulated by the waves that own its rows.
-//   "entity" rows: 32 per wave, their operands live in registers for the whole kernel (q and dout for dq; k and v
-//                  for dk; k for dv); the gradient rows are theirs.
-//   "stream" rows: walked in tiles of 32 through a 2-slot LDS ring filled by direct global->LDS loads (k and v for
-//                  dq; q and dout for dk and dv).
+// One kernel body, two passes, no atomics: every gradient is accumulated by the waves that own its rows.
+//   dq pass:      "entity" rows = 32 q rows per wave (q and dout fragments in registers), "stream" rows = keys
+//                 (k for the scores and for the accumulation, v for dP).
+//   dk / dv pass: entity rows = 32 key rows per wave (k and v fragments in registers), stream rows = q rows (q for
+//                 the scores and the dk accumulation, dout for dP and the dv accumulation).  S^T and dP^T are formed
+//                 once per tile; P feeds the dv accumulators and dS the dk ones: seven matrix products per call
+//                 where five are necessary (S and dP are formed in both passes).
+// Stream rows are walked in tiles of 32 through a 2-slot LDS ring filled by direct global->LDS loads.
 // Per tile, with the forward kernel's layouts and fragment reads:
 //   S^T  = stream1 . entity1^T      (A = tile rows by ds_read_b128, B = entity fragments)   lane = entity row
-//   dP^T = stream2 . entity2^T      (not for dv)
+//   dP^T = stream2 . entity2^T
 //   W    = exp2(c*S - lse*log2e) [* (dP - delta)]     f32, packed to bf16 in B-operand order (the factor `scale` of
 //                                                      dS is applied once, to the finished accumulators)
 //   acc^T += stream3^T . W          (A = the tile through the transposing LDS read)
-// lse and delta belong to the q rows: per-lane scalars for dq, sixteen values per lane and tile for dk / dv, read
-// from a workspace that a small kernel fills first (delta, lse in log2 units, both padded to a multiple of 32 rows
-// with lse = +inf so that padded q rows get p = 0).
+// lse and delta belong to the q rows: per-lane scalars for dq; for dk / dv sixteen values per lane and tile, which
+// ride through the ring next to the tile (a register load inside the loop would be waited for in issue order, i.e.
+// behind the next tile's loads).  They come from a workspace that a small kernel fills first (delta, lse in log2
+// units, both padded to a multiple of 32 rows with lse = +inf so that padded q rows get p = 0).
 #include <atomic>
 #include <mutex>
 
@@ -41,6 +45,14 @@ struct BwdLayout {
   static constexpr int VH = HD == 128 ? 4 * GB : 16 * 64;                // second 16-row half of the tile
 };
 
+// Per-row f32 values of a stream tile (lse and delta of its q rows, or the bias of its keys) travel through the ring as
+// well: 64 floats behind the tiles of a slot.
+constexpr int kAuxFloats = 64;
+template <int MODE, int HD, bool BIAS>
+constexpr int bwd_slot_elems() {  // bf16 elements per ring slot
+  return BwdLayout<HD>::Stage + (MODE == 3 ? BwdLayout<HD>::TileB : 0) + ((MODE != 0 || BIAS) ? 2 * kAuxFloats : 0);
+}
+
 typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr_b;
 typedef __attribute__((ext_vector_type(8))) short s16x8_b;
 
@@ -58,6 +70,9 @@ struct BwdArgs {
   const __bf16* s2;  // stream tensor of the dP contraction (unused for dv)
   const __bf16* s3;  // stream tensor the gradient accumulates with
   __bf16* out;       // gradient of the entity rows
+  const __bf16* s4;  // MODE 3: second stream tensor to accumulate with (dout, for dv); s3 is q (for dk)
+  __bf16* out2;      // MODE 3: dv
+  int64_t s4_sb, s4_ss, s4_sh, o2_sb, o2_ss, o2_sh;
   const float* lse2;   // [B,H,Sp] lse * log2(e), +inf on padded rows
   const float* delta;  // [B,H,Sp]
   int H, Se, Ss, Sp;
@@ -70,17 +85,22 @@ struct BwdArgs {
   int64_t bias_sb;
 };
 
-// MODE 0: dq (entity = q rows, stream = keys), 1: dk, 2: dv (entity = key rows, stream = q rows)
+// MODE 0: dq (entity = q rows, stream = keys); 3: dk and dv in one pass (entity = key rows, stream = q rows).
+// MODE 1 (dk alone) and 2 (dv alone) are the same body with one accumulator set; the library launches 0 and 3.
 template <int MODE, int HD, bool BIAS>
-__global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
+__device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw_b[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw_b);
   constexpr int NW = 4;
   constexpr bool HAS2 = MODE != 2;
+  constexpr bool BOTH = MODE == 3;
   using L = BwdLayout<HD>;
   constexpr int NJ = HD / 16;   // MFMAs per 32 x 32 block of a contraction over the head dim
   constexpr int ND = HD / 32;   // 32-wide slabs of d = accumulators
-  constexpr int kBD = HD, kBGK = L::GA, kBGV = L::GB, kBTileA = L::TileA, kBTileB = L::TileB, kBStage = L::Stage;
+  constexpr int kBD = HD, kBGK = L::GA, kBGV = L::GB, kBTileA = L::TileA, kBTileB = L::TileB;
+  constexpr int kBStage = bwd_slot_elems<MODE, HD, BIAS>();  // MODE 3: a second transposed-read tile (dout)
+  constexpr bool AUX = MODE != 0 || BIAS;
+  constexpr int kBAux = L::Stage + (BOTH ? L::TileB : 0);    // where a slot's f32 values start (elements)
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -125,32 +145,89 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
   const __bf16* s1p = a.s1 + b * a.s1_sb + h * a.s1_sh;
   const __bf16* s2p = HAS2 ? a.s2 + b * a.s2_sb + h * a.s2_sh : nullptr;
   const __bf16* s3p = a.s3 + b * a.s3_sb + h * a.s3_sh;
+  [[maybe_unused]] const __bf16* s4p = BOTH ? a.s4 + b * a.s4_sb + h * a.s4_sh : nullptr;
   constexpr int RPI = L::RPI;
   const int grow = HD == 128 ? lane >> 4 : lane >> 3;
   // lane -> logical 16-byte chunk stored at this lane's position (a wave fills the row groups wave, wave + NW, ...)
   const int acol = HD == 128 ? ((lane & 15) ^ grow) * 8 : ((lane & 7) ^ ((4 * (wave & 1) + (grow >> 1)) & 7)) * 8;
   const int bcol = HD == 128 ? ((lane & 15) ^ (grow << 2)) * 8 : ((lane & 7) ^ (((grow >> 1) & 1) << 2)) * 8;
   const unsigned smem_addr = lds_addr_of(smem);
+  // byte offsets of this lane's chunk from the first row of its row group: the same for every full tile.  The merged
+  // pass at head dim 128 has no registers to keep them in (spilled, every reload would wait for the load issued
+  // before it): it forms them again per tile from the lane number, a dozen full-rate instructions.
+  constexpr bool REFORM = BOTH && HD == 128;
+  auto chunk_ofs = [&](int ln, int64_t ss, bool transposed) __attribute__((always_inline)) {
+    const int gr = HD == 128 ? ln >> 4 : ln >> 3;
+    const int col = transposed ? (HD == 128 ? ((ln & 15) ^ (gr << 2)) * 8 : ((ln & 7) ^ (((gr >> 1) & 1) << 2)) * 8)
+                               : (HD == 128 ? ((ln & 15) ^ gr) * 8 : ((ln & 7) ^ ((4 * (wave & 1) + (gr >> 1)) & 7)) * 8);
+    return (__umul24((unsigned)gr, (unsigned)ss) + (unsigned)col) * 2u;  // strides are below 2^23
+  };
+  [[maybe_unused]] const unsigned ofs1 = REFORM ? 0u : chunk_ofs(lane, a.s1_ss, false);
+  [[maybe_unused]] const unsigned ofs2 = HAS2 && !REFORM ? chunk_ofs(lane, a.s2_ss, false) : 0u;
+  [[maybe_unused]] const unsigned ofs3 = REFORM ? 0u : chunk_ofs(lane, a.s3_ss, true);
+  [[maybe_unused]] const unsigned ofs4 = BOTH && !REFORM ? chunk_ofs(lane, a.s4_ss, true) : 0u;
+  // wave 0 brings a tile's f32 values: lanes 0-31 the lse of its 32 q rows and lanes 32-63 their delta, or (dq pass)
+  // every lane the bias of key lane % 32.  Through LDS because a register load here would be waited for in order
+  // behind the next tile's loads.
+  [[maybe_unused]] const unsigned ofs_aux =
+      MODE != 0 ? (lane < 32 ? 0u : (unsigned)((a.delta - a.lse2) * 4)) + (unsigned)l32 * 4u : (unsigned)l32 * 4u;
   auto dma = [&](int slot, int t) __attribute__((always_inline)) {
     const unsigned A1 = smem_addr + (unsigned)(slot * kBStage) * 2u;
     const unsigned A2 = A1 + kBTileA * 2u;
     const unsigned Bt = A2 + kBTileA * 2u;
+    if constexpr (AUX) {
+      if (wave == 0) {
+        unsigned oa = ofs_aux;
+        if constexpr (REFORM) {
+          int ln = lane;
+          asm volatile("" : "+v"(ln));
+          oa = (ln < 32 ? 0u : (unsigned)((a.delta - a.lse2) * 4)) + (unsigned)(ln & 31) * 4u;
+        }
+        lds_dma4((MODE != 0 ? lrow : bias_row) + t * kBT, oa, A1 + kBAux * 2u);
+      }
+    }
+    if (t * kBT + kBT <= a.Ss) {  // a full tile: uniform row-group bases, one per-lane offset per stream
+      unsigned o1 = ofs1, o2 = ofs2, o3 = ofs3, o4 = ofs4;
+      if constexpr (REFORM) {
+        int ln = lane;
+        asm volatile("" : "+v"(ln));  // opaque: keeps the four offsets from being hoisted out of the loop
+        o1 = chunk_ofs(ln, a.s1_ss, false);
+        o2 = chunk_ofs(ln, a.s2_ss, false);
+        o3 = chunk_ofs(ln, a.s3_ss, true);
+        o4 = chunk_ofs(ln, a.s4_ss, true);
+      }
 #pragma unroll
-    for (int i = 0; i < (kBT / RPI) / NW; ++i) {
-      const int g = wave + NW * i;
-      int rr = t * kBT + RPI * g + grow;
-      rr = rr < a.Ss ? rr : a.Ss - 1;
-      lds_dma16(s1p + (int64_t)rr * a.s1_ss + acol, A1 + (unsigned)(g * kBGK) * 2u);
-      if constexpr (HAS2) lds_dma16(s2p + (int64_t)rr * a.s2_ss + acol, A2 + (unsigned)(g * kBGK) * 2u);
-      lds_dma16(s3p + (int64_t)rr * a.s3_ss + bcol, Bt + (unsigned)(g * kBGV) * 2u);
+      for (int i = 0; i < (kBT / RPI) / NW; ++i) {
+        const int g = wave + NW * i;
+        const int64_t r = t * kBT + RPI * g;
+        lds_dma16(s1p + r * a.s1_ss, o1, A1 + (unsigned)(g * kBGK) * 2u);
+        if constexpr (HAS2) lds_dma16(s2p + r * a.s2_ss, o2, A2 + (unsigned)(g * kBGK) * 2u);
+        lds_dma16(s3p + r * a.s3_ss, o3, Bt + (unsigned)(g * kBGV) * 2u);
+        if constexpr (BOTH) lds_dma16(s4p + r * a.s4_ss, o4, Bt + (unsigned)(kBTileB + g * kBGV) * 2u);
+      }
+    } else {  // the ragged last tile: rows past the end repeat the last row
+#pragma unroll
+      for (int i = 0; i < (kBT / RPI) / NW; ++i) {
+        const int g = wave + NW * i;
+        int rr = t * kBT + RPI * g + grow;
+        rr = rr < a.Ss ? rr : a.Ss - 1;
+        lds_dma16(s1p + (int64_t)rr * a.s1_ss + acol, A1 + (unsigned)(g * kBGK) * 2u);
+        if constexpr (HAS2) lds_dma16(s2p + (int64_t)rr * a.s2_ss + acol, A2 + (unsigned)(g * kBGK) * 2u);
+        lds_dma16(s3p + (int64_t)rr * a.s3_ss + bcol, Bt + (unsigned)(g * kBGV) * 2u);
+        if constexpr (BOTH) lds_dma16(s4p + (int64_t)rr * a.s4_ss + bcol, Bt + (unsigned)(kBTileB + g * kBGV) * 2u);
+      }
     }
   };
 
   f32x16 acc[ND];
+  [[maybe_unused]] f32x16 acc2[BOTH ? ND : 1];  // MODE 3: dv next to dk
 #pragma unroll
   for (int db = 0; db < ND; ++db)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+    for (int i = 0; i < 16; ++i) {
+      acc[db][i] = 0.f;
+      if constexpr (BOTH) acc2[db][i] = 0.f;
+    }
 
   // per-lane fragment offsets (elements)
   int k_off[NJ], v_off[ND];
@@ -194,54 +271,65 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
         dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, ef2[j], dP, 0, 0, 0);
       }
     }
-    // lse (log2 units) and delta of the q row each logit belongs to
-    float ls[16], dl[16];
+    // W = P or dS, eight logits (one B operand) at a time; lse (log2 units) and delta belong to the q row of each logit:
+    // per-lane scalars when the q rows are the entity rows, loaded per half tile otherwise
     if constexpr (MODE == 0) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) { ls[i] = lse_e; dl[i] = delta_e; }
-      if constexpr (BIAS) {  // the tile's keys: subtracting the bias from lse adds it to the logit
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_row + t * kBT + 8 * g + 4 * hh);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) ls[4 * g + e] -= bv[e] * kLog2e;
-        }
-      }
       if (t == nt - 1) {  // keys past the end of a ragged last tile take no part
         const int sbase = t * kBT + 4 * hh;
 #pragma unroll
         for (int i = 0; i < 16; ++i)
-          if (sbase + 8 * (i >> 2) + (i & 3) >= a.Ss) {
-            S[i] = -INFINITY;
-            if constexpr (BIAS) ls[i] = INFINITY;  // whatever the bias padding holds
-          }
-      }
-    } else {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x4 lv = *reinterpret_cast<const f32x4*>(lrow + t * kBT + 8 * g + 4 * hh);
-        const f32x4 dv = *reinterpret_cast<const f32x4*>(drow + t * kBT + 8 * g + 4 * hh);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) { ls[4 * g + e] = lv[e] - (BIAS ? bias_e : 0.f); dl[4 * g + e] = dv[e]; }
+          if (sbase + 8 * (i >> 2) + (i & 3) >= a.Ss) S[i] = -INFINITY;
       }
     }
+    [[maybe_unused]] const float* aux = reinterpret_cast<const float*>(base + kBAux);
     bf16x8 W[2];
+    [[maybe_unused]] bf16x8 Wp[2];  // MODE 3: the probabilities themselves, for dv
 #pragma unroll
     for (int hb = 0; hb < 2; ++hb) {
-      float wv[8];
+      float ls[8], dl[8];
+      if constexpr (MODE == 0) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int i = 8 * hb + e;
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(S[i], c, -ls[i]));
-        wv[e] = HAS2 ? p * (dP[i] - dl[i]) : p;  // dS without its factor `scale`: applied once, to the accumulators
+        for (int e = 0; e < 8; ++e) { ls[e] = lse_e; dl[e] = delta_e; }
+        if constexpr (BIAS) {  // the tile's keys: subtracting the bias from lse adds it to the logit
+#pragma unroll
+          for (int g = 0; g < 2; ++g) {
+            const int col = t * kBT + 8 * (2 * hb + g) + 4 * hh;
+            const f32x4 bv = *reinterpret_cast<const f32x4*>(aux + 8 * (2 * hb + g) + 4 * hh);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ls[4 * g + e] = col + e < a.Ss ? lse_e - bv[e] * kLog2e : INFINITY;  // whatever the padding holds
+          }
+        }
+      } else {
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          const f32x4 lv = *reinterpret_cast<const f32x4*>(aux + 8 * (2 * hb + g) + 4 * hh);
+          const f32x4 dv = *reinterpret_cast<const f32x4*>(aux + 32 + 8 * (2 * hb + g) + 4 * hh);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { ls[4 * g + e] = lv[e] - (BIAS ? bias_e : 0.f); dl[4 * g + e] = dv[e]; }
+        }
       }
-      W[hb] = __builtin_bit_cast(bf16x8, pack8(wv));
+      unsigned wpk[4];
+      [[maybe_unused]] unsigned ppk[4];
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[8 * hb + e], c, -ls[e]));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[8 * hb + e + 1], c, -ls[e + 1]));
+        // dS without its factor `scale`: applied once, to the accumulators
+        wpk[e >> 1] = HAS2 ? pack2(p0 * (dP[8 * hb + e] - dl[e]), p1 * (dP[8 * hb + e + 1] - dl[e + 1])) : pack2(p0, p1);
+        if constexpr (BOTH) ppk[e >> 1] = pack2(p0, p1);
+      }
+      W[hb] = __builtin_bit_cast(bf16x8, u32x4{wpk[0], wpk[1], wpk[2], wpk[3]});
+      if constexpr (BOTH) Wp[hb] = __builtin_bit_cast(bf16x8, u32x4{ppk[0], ppk[1], ppk[2], ppk[3]});
     }
 #pragma unroll
     for (int jv = 0; jv < 2 * ND; ++jv) {
       const __bf16* src = base + v_off[jv % ND] + (jv / ND) * L::VH;
       const bf16x8 f = read_vt_b(src, src + L::V8);
       acc[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, W[jv / ND], acc[jv % ND], 0, 0, 0);
+      if constexpr (BOTH) {
+        const bf16x8 f2 = read_vt_b(src + kBTileB, src + kBTileB + L::V8);
+        acc2[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f2, Wp[jv / ND], acc2[jv % ND], 0, 0, 0);
+      }
     }
   }
 
@@ -258,7 +346,31 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
         u.y = pack2(acc[db][4 * g + 2] * osc, acc[db][4 * g + 3] * osc);
         *reinterpret_cast<uint2*>(orow + db * 32 + 8 * g) = u;
       }
+    if constexpr (BOTH) {
+      __bf16* orow2 = a.out2 + b * a.o2_sb + h * a.o2_sh + (int64_t)row * a.o2_ss + 4 * hh;
+#pragma unroll
+      for (int db = 0; db < ND; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          uint2 u;
+          u.x = pack2(acc2[db][4 * g], acc2[db][4 * g + 1]);
+          u.y = pack2(acc2[db][4 * g + 2], acc2[db][4 * g + 3]);
+          *reinterpret_cast<uint2*>(orow2 + db * 32 + 8 * g) = u;
+        }
+    }
   }
+}
+
+template <int MODE, int HD, bool BIAS>
+__global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
+  attn_bwd_body<MODE, HD, BIAS>(a);
+}
+// The dk / dv pass at head dim 128 wants a few registers more than half the register file (128 accumulators, 64 of
+// entity fragments, 32 of S and dP): held to two waves per SIMD, which the schedule needs to overlap one wave's
+// exponentials with the other's MFMAs; at one wave per SIMD it measured 28 % slower.
+template <int HD, bool BIAS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_bwd_both_kernel(BwdArgs a) {
+  attn_bwd_body<3, HD, BIAS>(a);
 }
 
 // delta[b,h,q] = sum_d dout*out, lse2 = lse*log2(e); rows q in [Sq, Sp) get delta 0, lse2 +inf.  16 lanes per row
@@ -293,13 +405,15 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const __bf16* out, const 
 
 template <int MODE, int HD, bool BIAS>
 int launch_bwd(hipStream_t st, BwdArgs a, int B) {
-  constexpr int lds_bytes = 2 * BwdLayout<HD>::Stage * 2;
+  constexpr int lds_bytes = 2 * bwd_slot_elems<MODE, HD, BIAS>() * 2;
   a.net = (a.Se + 127) / 128;
   const int64_t total = (int64_t)B * a.H * a.net;
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
-  auto kern = attn_bwd_kernel<MODE, HD, BIAS>;
+  void (*kern)(BwdArgs);
+  if constexpr (MODE == 3) kern = attn_bwd_both_kernel<HD, BIAS>;
+  else kern = attn_bwd_kernel<MODE, HD, BIAS>;
   static LdsOptIn opted;
   if (lds_opt_in(opted, reinterpret_cast<const void*>(kern), lds_bytes) != MDATTN_OK) return MDATTN_E_LAUNCH;
   hipLaunchKernelGGL(kern, dim3(a.chunk * 8), dim3(256), lds_bytes, st, a);
@@ -322,7 +436,7 @@ extern "C" int64_t mdattn_bwd_workspace_floats(int B, int H, int Sq) {
   return 2 * (int64_t)B * H * (((int64_t)Sq + 31) / 32 * 32);
 }
 
-// Shared body of mdattn_bwd_bf16 and mdattn_bwd_bf16_static: validation, the preparation kernel and the three passes.
+// Shared body of mdattn_bwd_bf16 and mdattn_bwd_bf16_static: validation, the preparation kernel and the two passes.
 static int bwd_run(hipStream_t st, const void* q, const void* k, const void* v, const void* out, const void* dout,
                    const float* lse, void* dq, void* dk, void* dv, float* workspace, int64_t workspace_floats,
                    int B, int H, int Sq, int Skv, int D,
@@ -345,12 +459,15 @@ static int bwd_run(hipStream_t st, const void* q, const void* k, const void* v, 
   if (!strides_ok(q_strides, 8) || !strides_ok(k_strides, 8) || !strides_ok(v_strides, 8) || !strides_ok(o_strides, 8))
     return MDATTN_E_ALIGN;
   if (q_strides->seq < D || k_strides->seq < D || v_strides->seq < D || o_strides->seq < D) return MDATTN_E_BADARG;
+  // every tensor is streamed by one of the passes with 32-bit byte offsets inside a row group
+  if (q_strides->seq >= (1 << 23) || k_strides->seq >= (1 << 23) || v_strides->seq >= (1 << 23) || o_strides->seq >= (1 << 23))
+    return MDATTN_E_UNSUPPORTED;
 
   const int Sp = (Sq + 31) / 32 * 32;
   float* lse2 = workspace;
   float* delta = workspace + (int64_t)B * H * Sp;
   const int64_t rows = (int64_t)B * H * Sp;
-  if ((rows + 15) / 16 > 0x7FFFFFFF) return MDATTN_E_UNSUPPORTED;
+  if ((rows + 15) / 16 > 0x7FFFFFFF || rows >= (1 << 29)) return MDATTN_E_UNSUPPORTED;  // delta - lse2 as a 32-bit byte offset
   hipLaunchKernelGGL(bwd_prep_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const __bf16*)out,
                      (const __bf16*)dout, lse, lse2, delta, H, Sq, Sp, D, rows, o_strides->batch, o_strides->seq, o_strides->head);
   if (launch_status() != MDATTN_OK) return MDATTN_E_LAUNCH;
@@ -367,20 +484,15 @@ static int bwd_run(hipStream_t st, const void* q, const void* k, const void* v, 
   set(a.o_sb, a.o_ss, a.o_sh, q_strides);
   int rc = launch_bwd_any<0>(st, a, B, D);
   if (rc != MDATTN_OK) return rc;
-  // dk: entity k / v, stream q (scores), dout (dP), q (accumulate)
+  // dk and dv in one pass: entity k / v, stream q (scores, and accumulate for dk), dout (dP, and accumulate for dv)
   a.e1 = (const __bf16*)k; a.e2 = (const __bf16*)v; a.s1 = (const __bf16*)q; a.s2 = (const __bf16*)dout; a.s3 = (const __bf16*)q;
-  a.out = (__bf16*)dk; a.Se = Skv; a.Ss = Sq;
+  a.s4 = (const __bf16*)dout;
+  a.out = (__bf16*)dk; a.out2 = (__bf16*)dv; a.Se = Skv; a.Ss = Sq;
   set(a.e1_sb, a.e1_ss, a.e1_sh, k_strides); set(a.e2_sb, a.e2_ss, a.e2_sh, v_strides);
   set(a.s1_sb, a.s1_ss, a.s1_sh, q_strides); set(a.s2_sb, a.s2_ss, a.s2_sh, o_strides); set(a.s3_sb, a.s3_ss, a.s3_sh, q_strides);
-  set(a.o_sb, a.o_ss, a.o_sh, k_strides);
-  rc = launch_bwd_any<1>(st, a, B, D);
-  if (rc != MDATTN_OK) return rc;
-  // dv: entity k, stream q (scores), dout (accumulate)
-  a.e2 = nullptr; a.s2 = nullptr; a.s3 = (const __bf16*)dout;
-  a.out = (__bf16*)dv;
-  set(a.s3_sb, a.s3_ss, a.s3_sh, o_strides);
-  set(a.o_sb, a.o_ss, a.o_sh, v_strides);
-  return launch_bwd_any<2>(st, a, B, D);
+  set(a.s4_sb, a.s4_ss, a.s4_sh, o_strides);
+  set(a.o_sb, a.o_ss, a.o_sh, k_strides); set(a.o2_sb, a.o2_ss, a.o2_sh, v_strides);
+  return launch_bwd_any<3>(st, a, B, D);
 }
 
 

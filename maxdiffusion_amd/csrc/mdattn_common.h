@@ -90,6 +90,10 @@ __device__ __forceinline__ void lds_dma16(const void* base, unsigned byte_off, u
 __device__ __forceinline__ void lds_dma16(const void* addr, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(addr) : "memory", "m0");
 }
+// The 4-byte form: lane i's dword lands at lds_addr + 4*i.
+__device__ __forceinline__ void lds_dma4(const void* base, unsigned byte_off, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds_addr), "v"(byte_off), "s"(base) : "memory", "m0");
+}
 __device__ __forceinline__ unsigned lds_addr_of(const void* p) {
   return (unsigned)(uintptr_t)(const void __attribute__((address_space(3)))*)p;
 }
