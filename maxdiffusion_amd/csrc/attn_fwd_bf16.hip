@@ -442,7 +442,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   constexpr int NJ = HD / 16;                                    // QK MFMAs per 32-key tile
   constexpr int ND = HD / 32;                                    // 32-wide slabs of d = O accumulators
   constexpr int KTILE = HD == 128 ? kKTileS : kTS * 64;          // elements
-  constexpr int STAGE = HD == 128 ? kStageS : 2 * kTS * 64;
+  constexpr int TILES = HD == 128 ? kStageS : 2 * kTS * 64;      // the K and the V tile of a slot
+  // with a bias, a slot also carries the tile's 32 bias values (f32) behind its tiles: a register load inside the
+  // loop would be waited for in issue order, i.e. behind the loads of the tile after next
+  constexpr int STAGE = TILES + (BIAS ? 4 * kTS : 0);  // 64 floats: one per lane of the load that brings them
   constexpr int RPI = HD == 128 ? 4 : 8;                          // rows one load instruction fills
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
@@ -467,7 +470,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   const float c = a.c;
   // with a bias the logits are brought to log2 units (scale folded, bias added) right after the MFMAs
   const float cs = BIAS ? 1.0f : c;
-  const float* bias_row = BIAS ? a.bias + b * a.bias_sb + 4 * hh : nullptr;
+  const float* bias_row = BIAS ? a.bias + b * a.bias_sb : nullptr;
 
   bf16x8 qf[NJ];  // filled from LDS below: the wave's 32 Q rows arrive like a K tile, by whole-row loads
 
@@ -483,6 +486,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   auto dma = [&](int slot, int kt) __attribute__((always_inline)) {
     const unsigned Ks = smem_addr + (unsigned)(slot * STAGE) * 2u;
     const unsigned Vs = Ks + KTILE * 2u;
+    // every wave fetches the same values to the same place (a load more per wave and tile, counted in the loop's
+    // s_waitcnt): lane l and lane l + 32 the bias of key l of the tile; the ring runs up to two tiles past the end
+    if constexpr (BIAS) lds_dma4(bias_row + (kt < nt ? kt : nt - 1) * kTS, (unsigned)l32 * 4u, Ks + TILES * 2u);
     if (kt * kTS + kTS <= a.Skv) {
       const __bf16* kt0 = kp + (int64_t)(kt * kTS + RPI * wave) * a.k_ss;
       const __bf16* vt0 = vp + (int64_t)(kt * kTS + RPI * wave) * a.v_ss;
@@ -550,7 +556,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
     if constexpr (BIAS) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_row + t * kTS + 8 * g);
+        const f32x4 bv = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(base + TILES) + 8 * g + 4 * hh);
 #pragma unroll
         for (int e = 0; e < 4; ++e) S[4 * g + e] = __builtin_fmaf(S[4 * g + e], c, bv[e] * kLog2e);
       }
@@ -641,7 +647,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   dma(1, 1);
   int slot = 0, fill = 2;
   for (int t = 0; t < nt - 1; ++t) {
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * GPW));  // vmcnt: this wave's share of tile t has landed
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * GPW + (BIAS ? 1 : 0)));  // vmcnt: this wave's share of tile t has landed
     __syncthreads();                                  // ... and everyone's; slot `fill` (tile t-1) is free
     dma(fill, t + 2);
     tile(t, slot, std::false_type{});
@@ -665,7 +671,7 @@ template <int NW, bool BIAS, int HD = 128>
 static int launch_flat(hipStream_t st, AttnArgs a, int B) {
   constexpr int BM = NW * 32;
   // the ring, or ring slot 0 plus one K-shaped Q staging tile per wave, whichever is larger
-  constexpr int stage_el = HD == 128 ? kStageS : 2 * kTS * 64, ktile_el = HD == 128 ? kKTileS : kTS * 64;
+  constexpr int stage_el = (HD == 128 ? kStageS : 2 * kTS * 64) + (BIAS ? 4 * kTS : 0), ktile_el = HD == 128 ? kKTileS : kTS * 64;
   constexpr int lds_bytes = (kSlotsS * stage_el > stage_el + NW * ktile_el ? kSlotsS * stage_el : stage_el + NW * ktile_el) * 2;
   a.nqt = (a.Sq + BM - 1) / BM;
   const int64_t total = (int64_t)B * a.H * a.nqt;
