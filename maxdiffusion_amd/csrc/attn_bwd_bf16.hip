@@ -18,8 +18,10 @@
 //   acc^T += stream3^T . W          (A = the tile through the transposing LDS read)
 // lse and delta belong to the q rows: per-lane scalars for dq; for dk / dv sixteen values per lane and tile, which
 // ride through the ring next to the tile (a register load inside the loop would be waited for in issue order, i.e.
-// behind the next tile's loads).  They come from a workspace that a small kernel fills first (delta, lse in log2
-// units, both padded to a multiple of 32 rows with lse = +inf so that padded q rows get p = 0).
+// behind the next tile's loads).  They come from a workspace that a small kernel fills first (-delta and -lse in log2
+// units, padded to a multiple of 32 rows with -lse = -inf so that padded q rows get p = 0).  Both are stored negated
+// because they start the MFMA chains they are subtracted from: dP^T - delta comes out of the chain, and so does
+// S^T - lse when the caller's q already carries scale * log2(e) (the factor c is then 1).
 #include <atomic>
 #include <mutex>
 
@@ -73,8 +75,8 @@ struct BwdArgs {
   const __bf16* s4;  // MODE 3: second stream tensor to accumulate with (dout, for dv); s3 is q (for dk)
   __bf16* out2;      // MODE 3: dv
   int64_t s4_sb, s4_ss, s4_sh, o2_sb, o2_ss, o2_sh;
-  const float* lse2;   // [B,H,Sp] lse * log2(e), +inf on padded rows
-  const float* delta;  // [B,H,Sp]
+  const float* lse2;   // [B,H,Sp] -lse * log2(e), -inf on padded rows
+  const float* delta;  // [B,H,Sp] -rowsum(dout * out)
   int H, Se, Ss, Sp;
   int net, total, chunk;
   int64_t e1_sb, e1_ss, e1_sh, e2_sb, e2_ss, e2_sh;
@@ -87,8 +89,9 @@ struct BwdArgs {
 
 // MODE 0: dq (entity = q rows, stream = keys); 3: dk and dv in one pass (entity = key rows, stream = q rows).
 // MODE 1 (dk alone) and 2 (dv alone) are the same body with one accumulator set; the library launches 0 and 3.
-template <int MODE, int HD, bool BIAS>
+template <int MODE, int HD, bool BIAS, bool PRE>
 __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
+  static_assert(!(PRE && BIAS), "a biased logit is touched after the MFMAs anyway");
   extern __shared__ __attribute__((aligned(16))) char smem_raw_b[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw_b);
   constexpr int NW = 4;
@@ -131,10 +134,10 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
   }
   const float* lrow = a.lse2 + ((int64_t)b * a.H + h) * a.Sp;
   const float* drow = a.delta + ((int64_t)b * a.H + h) * a.Sp;
-  float lse_e = 0.f, delta_e = 0.f;
+  float nlse_e = 0.f, ndelta_e = 0.f;  // the workspace holds both negated
   if constexpr (MODE == 0) {
-    lse_e = lrow[erow];
-    delta_e = drow[erow];
+    nlse_e = lrow[erow];
+    ndelta_e = drow[erow];
   }
   // key bias in log2 units: a per-lane scalar when the keys are the entity rows, sixteen values per tile otherwise
   [[maybe_unused]] const float* bias_row = BIAS ? a.bias + b * a.bias_sb : nullptr;
@@ -256,9 +259,30 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
     if (t + 1 < nt) dma((t + 1) & 1, t + 1);
     const __bf16* base = smem + (t & 1) * kBStage;
 
+    // Start values of the two MFMA chains: -delta for dP^T, so that the chain ends on dP - delta; and, when the
+    // logits come out of the MFMAs in log2 units (PRE), -lse for S^T, so that exp2 applies to the chain's result
+    // as it is.  Per-lane constants when the q rows are the entity rows, the tile's values from LDS otherwise.
+    [[maybe_unused]] const float* aux = reinterpret_cast<const float*>(base + kBAux);
     f32x16 S, dP;
+    if constexpr (MODE == 0) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { S[i] = 0.f; dP[i] = 0.f; }
+      for (int i = 0; i < 16; ++i) { S[i] = PRE ? nlse_e : 0.f; dP[i] = ndelta_e; }
+    } else {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 dv = *reinterpret_cast<const f32x4*>(aux + 32 + 8 * g + 4 * hh);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dP[4 * g + e] = dv[e];
+        if constexpr (PRE) {
+          const f32x4 lv = *reinterpret_cast<const f32x4*>(aux + 8 * g + 4 * hh);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) S[4 * g + e] = lv[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) S[4 * g + e] = 0.f;
+        }
+      }
+    }
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const bf16x8 f = *reinterpret_cast<const bf16x8*>(base + k_off[j]);
@@ -271,8 +295,7 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
         dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, ef2[j], dP, 0, 0, 0);
       }
     }
-    // W = P or dS, eight logits (one B operand) at a time; lse (log2 units) and delta belong to the q row of each logit:
-    // per-lane scalars when the q rows are the entity rows, loaded per half tile otherwise
+    // W = P or dS, eight logits (one B operand) at a time
     if constexpr (MODE == 0) {
       if (t == nt - 1) {  // keys past the end of a ragged last tile take no part
         const int sbase = t * kBT + 4 * hh;
@@ -281,41 +304,42 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
           if (sbase + 8 * (i >> 2) + (i & 3) >= a.Ss) S[i] = -INFINITY;
       }
     }
-    [[maybe_unused]] const float* aux = reinterpret_cast<const float*>(base + kBAux);
     bf16x8 W[2];
     [[maybe_unused]] bf16x8 Wp[2];  // MODE 3: the probabilities themselves, for dv
 #pragma unroll
     for (int hb = 0; hb < 2; ++hb) {
-      float ls[8], dl[8];
-      if constexpr (MODE == 0) {
+      [[maybe_unused]] float nl[8];  // -lse (log2 units) of each logit's q row, with the key's bias added
+      if constexpr (!PRE) {
+        if constexpr (MODE == 0) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { ls[e] = lse_e; dl[e] = delta_e; }
-        if constexpr (BIAS) {  // the tile's keys: subtracting the bias from lse adds it to the logit
+          for (int e = 0; e < 8; ++e) nl[e] = nlse_e;
+          if constexpr (BIAS) {
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+              const int col = t * kBT + 8 * (2 * hb + g) + 4 * hh;
+              const f32x4 bv = *reinterpret_cast<const f32x4*>(aux + 8 * (2 * hb + g) + 4 * hh);
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                nl[4 * g + e] = col + e < a.Ss ? __builtin_fmaf(bv[e], kLog2e, nlse_e) : -INFINITY;  // whatever the padding holds
+            }
+          }
+        } else {
 #pragma unroll
           for (int g = 0; g < 2; ++g) {
-            const int col = t * kBT + 8 * (2 * hb + g) + 4 * hh;
-            const f32x4 bv = *reinterpret_cast<const f32x4*>(aux + 8 * (2 * hb + g) + 4 * hh);
+            const f32x4 lv = *reinterpret_cast<const f32x4*>(aux + 8 * (2 * hb + g) + 4 * hh);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) ls[4 * g + e] = col + e < a.Ss ? lse_e - bv[e] * kLog2e : INFINITY;  // whatever the padding holds
+            for (int e = 0; e < 4; ++e) nl[4 * g + e] = lv[e] + (BIAS ? bias_e : 0.f);
           }
-        }
-      } else {
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
-          const f32x4 lv = *reinterpret_cast<const f32x4*>(aux + 8 * (2 * hb + g) + 4 * hh);
-          const f32x4 dv = *reinterpret_cast<const f32x4*>(aux + 32 + 8 * (2 * hb + g) + 4 * hh);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { ls[4 * g + e] = lv[e] - (BIAS ? bias_e : 0.f); dl[4 * g + e] = dv[e]; }
         }
       }
       unsigned wpk[4];
       [[maybe_unused]] unsigned ppk[4];
 #pragma unroll
       for (int e = 0; e < 8; e += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[8 * hb + e], c, -ls[e]));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[8 * hb + e + 1], c, -ls[e + 1]));
+        const float p0 = __builtin_amdgcn_exp2f(PRE ? S[8 * hb + e] : __builtin_fmaf(S[8 * hb + e], c, nl[e]));
+        const float p1 = __builtin_amdgcn_exp2f(PRE ? S[8 * hb + e + 1] : __builtin_fmaf(S[8 * hb + e + 1], c, nl[e + 1]));
         // dS without its factor `scale`: applied once, to the accumulators
-        wpk[e >> 1] = HAS2 ? pack2(p0 * (dP[8 * hb + e] - dl[e]), p1 * (dP[8 * hb + e + 1] - dl[e + 1])) : pack2(p0, p1);
+        wpk[e >> 1] = HAS2 ? pack2(p0 * dP[8 * hb + e], p1 * dP[8 * hb + e + 1]) : pack2(p0, p1);
         if constexpr (BOTH) ppk[e >> 1] = pack2(p0, p1);
       }
       W[hb] = __builtin_bit_cast(bf16x8, u32x4{wpk[0], wpk[1], wpk[2], wpk[3]});
@@ -361,19 +385,20 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
   }
 }
 
-template <int MODE, int HD, bool BIAS>
+template <int MODE, int HD, bool BIAS, bool PRE>
 __global__ __launch_bounds__(256) void attn_bwd_kernel(BwdArgs a) {
-  attn_bwd_body<MODE, HD, BIAS>(a);
+  attn_bwd_body<MODE, HD, BIAS, PRE>(a);
 }
 // The dk / dv pass at head dim 128 wants a few registers more than half the register file (128 accumulators, 64 of
 // entity fragments, 32 of S and dP): held to two waves per SIMD, which the schedule needs to overlap one wave's
 // exponentials with the other's MFMAs; at one wave per SIMD it measured 28 % slower.
-template <int HD, bool BIAS>
+template <int HD, bool BIAS, bool PRE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_bwd_both_kernel(BwdArgs a) {
-  attn_bwd_body<3, HD, BIAS>(a);
+  attn_bwd_body<3, HD, BIAS, PRE>(a);
 }
 
-// delta[b,h,q] = sum_d dout*out, lse2 = lse*log2(e); rows q in [Sq, Sp) get delta 0, lse2 +inf.  16 lanes per row
+// The workspace, both negated (they start the MFMA chains that they are subtracted from):
+// delta[b,h,q] = -sum_d dout*out, lse2 = -lse*log2(e); rows q in [Sq, Sp) get delta 0, lse2 -inf.  16 lanes per row
 // (head dim 64: the upper 8 stay idle).
 __global__ __launch_bounds__(256) void bwd_prep_kernel(const __bf16* out, const __bf16* dout, const float* lse,
                                                        float* lse2, float* delta, int H, int Sq, int Sp, int D,
@@ -396,15 +421,15 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const __bf16* out, const 
   }
   acc = row16_sum(acc);
   if (lane == 0) {
-    delta[r] = q < Sq ? acc : 0.f;
+    delta[r] = q < Sq ? -acc : 0.f;
     // padded rows, and rows whose keys were all masked (the forward wrote lse = -inf, out = 0), take no part: p = 0
     const float lv = q < Sq ? lse[bh * Sq + q] : -INFINITY;
-    lse2[r] = lv > -INFINITY ? lv * kLog2e : INFINITY;
+    lse2[r] = lv > -INFINITY ? -lv * kLog2e : -INFINITY;
   }
 }
 
-template <int MODE, int HD, bool BIAS>
-int launch_bwd(hipStream_t st, BwdArgs a, int B) {
+template <int MODE, int HD, bool BIAS, bool PRE>
+int launch_bwd_as(hipStream_t st, BwdArgs a, int B) {
   constexpr int lds_bytes = 2 * bwd_slot_elems<MODE, HD, BIAS>() * 2;
   a.net = (a.Se + 127) / 128;
   const int64_t total = (int64_t)B * a.H * a.net;
@@ -412,12 +437,22 @@ int launch_bwd(hipStream_t st, BwdArgs a, int B) {
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
   void (*kern)(BwdArgs);
-  if constexpr (MODE == 3) kern = attn_bwd_both_kernel<HD, BIAS>;
-  else kern = attn_bwd_kernel<MODE, HD, BIAS>;
+  if constexpr (MODE == 3) kern = attn_bwd_both_kernel<HD, BIAS, PRE>;
+  else kern = attn_bwd_kernel<MODE, HD, BIAS, PRE>;
   static LdsOptIn opted;
   if (lds_opt_in(opted, reinterpret_cast<const void*>(kern), lds_bytes) != MDATTN_OK) return MDATTN_E_LAUNCH;
   hipLaunchKernelGGL(kern, dim3(a.chunk * 8), dim3(256), lds_bytes, st, a);
   return launch_status();
+}
+
+// scale * log2(e) == 1 (to f32 round-off: the caller's q carries the factor, as for the forward): the logits leave the
+// MFMAs in log2 units and take -lse as the chain's start value instead of a multiply-add each.
+template <int MODE, int HD, bool BIAS>
+int launch_bwd(hipStream_t st, const BwdArgs& a, int B) {
+  if constexpr (!BIAS) {
+    if (a.c > 1.0f - 1e-6f && a.c < 1.0f + 1e-6f) return launch_bwd_as<MODE, HD, false, true>(st, a, B);
+  }
+  return launch_bwd_as<MODE, HD, BIAS, false>(st, a, B);
 }
 
 template <int MODE>
@@ -518,7 +553,7 @@ extern "C" int mdattn_bwd_bf16_bias(void* stream, const void* q, const void* k, 
 
 // ---------------------------------------------------------------------------------------------------
 // mdattn_bwd_bf16_static: the same backward for callers that cannot allocate (HIP graph capture, serving loops that
-// forbid hipMalloc).  The workspace (lse in log2 units and delta, one float each per padded query row) lives in a
+// forbid hipMalloc).  The workspace (-lse in log2 units and -delta, one float each per padded query row) lives in a
 // file-scope device array instead of a caller's buffer.  Every GPU holds its own copy of the array at its own
 // address: that address is looked up once per device with hipGetSymbolAddress and kept; host code never uses the
 // array's name as a pointer.  bwd_prep_kernel writes every element the passes read, so nothing has to be cleared

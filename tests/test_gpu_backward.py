@@ -65,6 +65,25 @@ def test_backward_layout_scale_and_sharp_logits(dev):
     _check(hsd(dv), rv, f"dv {layout} sharp")
 
 
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("sq,skv", [(1, 1), (257, 63), (300, 333), (513, 512)])
+def test_backward_scale_carried_by_q(dev, D, sq, skv):
+  """scale = ln 2 on a q that already carries D^-1/2 * log2(e) (what the prologue's q_mul produces for the forward):
+  scale * log2(e) is 1 and the library takes the kernels whose logits leave the MFMAs in log2 units.  dq is the
+  gradient with respect to the q that was passed."""
+  import math
+  B, H = 2, 3
+  q = O.bf16_round(O.normal_bf16((B, sq, H, D), 0) * np.float32(D**-0.5 * math.log2(math.e)))
+  do = O.normal_bf16((B, sq, H, D), 3)
+  k, v = O.normal_bf16((B, skv, H, D), 1), O.normal_bf16((B, skv, H, D), 2)
+  dq, dk, dv = _run(q, k, v, do, dev, scale=math.log(2.0))
+  for b in range(B):
+    rq, rk, rv = O.attention_bwd(hsd(q[b:b + 1]), hsd(k[b:b + 1]), hsd(v[b:b + 1]), hsd(do[b:b + 1]), math.log(2.0))
+    _check(hsd(dq[b:b + 1]), rq, f"folded D={D} dq Sq={sq} Skv={skv} b{b}")
+    _check(hsd(dk[b:b + 1]), rk, f"folded D={D} dk Sq={sq} Skv={skv} b{b}")
+    _check(hsd(dv[b:b + 1]), rv, f"folded D={D} dv Sq={sq} Skv={skv} b{b}")
+
+
 def test_backward_accepts_dout_in_another_layout_than_out(dev):
   """out stored [B,H,S,D], dout contiguous [B,S,H,D] (what autograd hands over): the wrapper has to re-lay dout like
   out, element by element."""
