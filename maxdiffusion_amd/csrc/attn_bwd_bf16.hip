@@ -103,6 +103,8 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
   constexpr int kBD = HD, kBGK = L::GA, kBGV = L::GB, kBTileA = L::TileA, kBTileB = L::TileB;
   constexpr int kBStage = bwd_slot_elems<MODE, HD, BIAS>();  // MODE 3: a second transposed-read tile (dout)
   constexpr bool AUX = MODE != 0 || BIAS;
+  constexpr int LA = MODE == 0 && HD == 128 ? 4 : 0;  // fragment look-ahead (the dk / dv pass has no registers for a window)
+  static_assert(LA == 0 || (HAS2 && !BOTH && LA <= 2 * ND), "the window covers the three-product passes");
   constexpr int kBAux = L::Stage + (BOTH ? L::TileB : 0);    // where a slot's f32 values start (elements)
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -283,16 +285,33 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
         }
       }
     }
+    // The tile's fragment reads as one stream: NJ row reads for S^T, NJ for dP^T, then the 2*ND transposing reads
+    // of the accumulation.  With LA > 0 a window of LA fragments runs ahead of the MFMAs (pinned by scheduling
+    // barriers: left to itself the compiler waits for every read right before its MFMA).
+    auto frag = [&](int n) __attribute__((always_inline)) {
+      if (n < NJ) return *reinterpret_cast<const bf16x8*>(base + k_off[n]);
+      if (n < 2 * NJ) return *reinterpret_cast<const bf16x8*>(base + kBTileA + k_off[n - NJ]);
+      const int jv = n - 2 * NJ;
+      const __bf16* src = base + v_off[jv % ND] + (jv / ND) * L::VH;
+      return read_vt_b(src, src + L::V8);
+    };
+    [[maybe_unused]] bf16x8 win[LA > 0 ? LA : 1];
+    if constexpr (LA > 0) {
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const bf16x8 f = *reinterpret_cast<const bf16x8*>(base + k_off[j]);
-      S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, ef1[j], S, 0, 0, 0);
-    }
-    if constexpr (HAS2) {
+      for (int n = 0; n < LA; ++n) win[n] = frag(n);
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        const bf16x8 f = *reinterpret_cast<const bf16x8*>(base + kBTileA + k_off[j]);
-        dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, ef2[j], dP, 0, 0, 0);
+      for (int n = 0; n < 2 * NJ; ++n) {
+        if (n < NJ) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(win[n % LA], ef1[n % NJ], S, 0, 0, 0);
+        else dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(win[n % LA], ef2[n % NJ], dP, 0, 0, 0);
+        win[n % LA] = frag(n + LA);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(j), ef1[j], S, 0, 0, 0);
+      if constexpr (HAS2) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(NJ + j), ef2[j], dP, 0, 0, 0);
       }
     }
     // W = P or dS, eight logits (one B operand) at a time
@@ -328,7 +347,7 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
           for (int g = 0; g < 2; ++g) {
             const f32x4 lv = *reinterpret_cast<const f32x4*>(aux + 8 * (2 * hb + g) + 4 * hh);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) nl[4 * g + e] = lv[e] + (BIAS ? bias_e : 0.f);
+            for (int e = 0; e < 4; ++e) nl[4 * g + e] = BIAS ? lv[e] + bias_e : lv[e];
           }
         }
       }
@@ -348,6 +367,12 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
 #pragma unroll
     for (int jv = 0; jv < 2 * ND; ++jv) {
       const __bf16* src = base + v_off[jv % ND] + (jv / ND) * L::VH;
+      if constexpr (LA > 0) {
+        acc[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(win[(2 * NJ + jv) % LA], W[jv / ND], acc[jv % ND], 0, 0, 0);
+        if (jv + LA < 2 * ND) win[(2 * NJ + jv) % LA] = frag(2 * NJ + jv + LA);
+        __builtin_amdgcn_sched_barrier(0);
+        continue;
+      }
       const bf16x8 f = read_vt_b(src, src + L::V8);
       acc[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, W[jv / ND], acc[jv % ND], 0, 0, 0);
       if constexpr (BOTH) {
