@@ -210,7 +210,7 @@ int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, float* scal
 /*
  * fp8-e4m3 attention forward: q8/k8/v8 are e4m3 bytes [B,S,H,D] by strides, *_scale device f32[1]
  * de-quantisation factors; P is re-quantised to e4m3 per tile before the PV MFMA; f32 accumulation;
- * bf16 out; lse as above.  Requires D == 128.
+ * bf16 out; lse as above.  Requires D == 128, or D == 64 (LTX-2's audio stream).
  * When scale * log2(e) * q_scale * k_scale is a power of two (see mdattn_quant_e4m3: premul, pow2_scale, and
  * scale = ln 2 here) the logit scale is applied inside the MFMAs and the softmax needs no multiply; the scales are
  * read on the device, so nothing has to be declared: two instances of the kernel are launched and the one whose

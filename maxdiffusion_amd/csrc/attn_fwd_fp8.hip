@@ -1,4 +1,5 @@
-// Non-causal flash-attention forward for gfx950 (MI355X) on fp8-e4m3 (OCP) operands, head_dim 128.
+// Non-causal flash-attention forward for gfx950 (MI355X) on fp8-e4m3 (OCP) operands, head_dim 128 (described below)
+// or 64 (template HD: one QK MFMA per 32-key block, two slabs of d, 64-byte rows; the differences are noted in place).
 //
 // Same decomposition as the bf16 kernel, on v_mfma_f32_32x32x64_f8f6f4 (K = 64 per instruction, twice
 // the bf16 rate):
@@ -30,11 +31,8 @@ namespace mdattn {
 namespace {
 
 constexpr int kBN8 = 64;                                  // keys per tile
-constexpr int kD8 = 128;                                  // head dim = bytes per row
-constexpr int kKS8 = kD8;                                 // K row stride in LDS, bytes (chunks permuted, not padded)
-constexpr int kVS8 = kD8;                                 // V row stride in LDS, bytes (chunks permuted, not padded)
-constexpr int kStage8 = kBN8 * kKS8 + kBN8 * kVS8;        // bytes per LDS stage
 constexpr int kSlots8 = 3;                                // LDS ring depth
+// K and V rows sit in LDS with a stride of head_dim bytes (chunks permuted, not padded): 2 * 64 * HD bytes per stage
 constexpr float kPOff = 3.0f;                             // P = exp2(logit - max + kPOff) at a fresh maximum
 // Softmax without exponentials (MODE 2).  An e4m3 byte read as an integer is a piecewise-linear log2 of its value:
 // code = 8 * (exponent + 7) + mantissa.  So the QK MFMAs are made to deliver x' = 8 * (logit - ref) + 56 (block scale
@@ -74,9 +72,14 @@ struct Fp8Args {
 // and by latencies a single wave cannot hide, so the third wave per SIMD is worth more than registers.
 // BIAS (MODE 0 only): an additive per-key bias (a key padding mask) joins the raw products right after the MFMAs,
 // divided by the logit scale so that the multiply per logit carries it; this instance serves every kind of scale.
-template <int NW, int MODE, bool BIAS = false>
+template <int NW, int MODE, bool BIAS = false, int HD = 128>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void attn_fwd_fp8_kernel(Fp8Args a) {
   static_assert(!BIAS || MODE == 0, "the key bias lives in the path with a multiply per logit");
+  static_assert(HD == 128 || HD == 64, "head dim");
+  constexpr int kKS8 = HD, kVS8 = HD;                 // row strides in LDS, bytes
+  constexpr int kStage8 = kBN8 * kKS8 + kBN8 * kVS8;  // bytes per LDS stage
+  constexpr int NJ = HD / 64;                         // QK MFMAs (K = 64) per 32-key block
+  constexpr int NSL = HD / 32;                        // 32-wide slabs of d = O accumulators
   constexpr bool PRE = MODE != 0;    // the logit scale is a power of two and rides in the MFMAs' block scale
   constexpr bool CODE = MODE == 2;   // ... and P is formed without exp2: see kCodeOne
   extern __shared__ __attribute__((aligned(16))) char smem8[];
@@ -111,13 +114,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   [[maybe_unused]] const int bias_cols = (a.Skv + 31) / 32 * 32;  // entries the caller's bias rows are sure to hold
 
   // ---- Q fragments: lane (row l32, half hh) holds bytes 64*j + 32*hh .. +31 of its row
-  i32x8 qf[2];
+  i32x8 qf[NJ];
   {
     int row = q0 + l32;
     row = row < a.Sq ? row : a.Sq - 1;
     const uint8_t* p = qp + (int64_t)row * a.q_ss + hh * 32;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       const u32x4 lo = *reinterpret_cast<const u32x4*>(p + j * 64);
       const u32x4 hi = *reinterpret_cast<const u32x4*>(p + j * 64 + 16);
       qf[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
@@ -130,39 +133,45 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   // c ^ 2*(((r >> 1) & 1) + 2*((r >> 3) & 1)).  Every 8 lanes fetch one whole 128-byte row.  Wave w fills
   // the row groups w, w+NW, ...  Rows past the end re-read the last valid row: they only ever meet
   // masked logits (P = 0), and every e4m3 code the quantiser emits is finite.
-  constexpr int GPW = 8 / NW;                                  // 8-row groups per wave, tile and tensor
-  const int grow = lane >> 3;                                  // row of the group this lane fills
-  const int kx_fill = (4 * (wave & 1) + (grow >> 1)) & 7;      // (row >> 1) & 7 of that row (groups w, w+NW: same parity)
-  const int vx_fill = 2 * (((grow >> 1) & 1) + 2 * (wave & 1));
-  const unsigned kofs = (unsigned)(grow * (int)a.k_ss + (((lane & 7) ^ kx_fill) * 16));
-  const unsigned vofs = (unsigned)(grow * (int)a.v_ss + (((lane & 7) ^ vx_fill) * 16));
+  // Head dim 64: one instruction writes 16 rows of 64 bytes, every 4 lanes one row; K chunk c of row r sits at
+  // c ^ ((r >> 2) & 3), V chunk c at c ^ 2*((r >> 3) & 1): conflict-free for the same two read patterns.
+  constexpr int RPI = 1024 / HD;                               // rows one load instruction fills
+  constexpr int CPR = HD / 16;                                 // 16-byte chunks per row
+  constexpr int GPW = (kBN8 / RPI) / NW;                       // row groups per wave, tile and tensor
+  static_assert(GPW >= 1, "a wave fills at least one row group per tile");
+  const int grow = lane / CPR;                                 // row of the group this lane fills
+  // the row's permutation key (groups w, w+NW of head dim 128 have the same parity; head dim 64 needs the row in its group only)
+  const int kx_fill = HD == 128 ? (4 * (wave & 1) + (grow >> 1)) & 7 : (grow >> 2) & 3;
+  const int vx_fill = HD == 128 ? 2 * (((grow >> 1) & 1) + 2 * (wave & 1)) : 2 * ((grow >> 3) & 1);
+  const unsigned kofs = (unsigned)(grow * (int)a.k_ss + (((lane & (CPR - 1)) ^ kx_fill) * 16));
+  const unsigned vofs = (unsigned)(grow * (int)a.v_ss + (((lane & (CPR - 1)) ^ vx_fill) * 16));
   const unsigned smem_addr = lds_addr_of(smem8);
   auto dma = [&](int slot, int kt) __attribute__((always_inline)) {
     const unsigned Ks = smem_addr + (unsigned)(slot * kStage8);
     const unsigned Vs = Ks + kBN8 * kKS8;
     if (kt * kBN8 + kBN8 <= a.Skv) {
-      const uint8_t* kt0 = kp + (int64_t)(kt * kBN8 + 8 * wave) * a.k_ss;
-      const uint8_t* vt0 = vp + (int64_t)(kt * kBN8 + 8 * wave) * a.v_ss;
+      const uint8_t* kt0 = kp + (int64_t)(kt * kBN8 + RPI * wave) * a.k_ss;
+      const uint8_t* vt0 = vp + (int64_t)(kt * kBN8 + RPI * wave) * a.v_ss;
 #pragma unroll
       for (int i = 0; i < GPW; ++i) {
-        lds_dma16(kt0 + (int64_t)(8 * NW * i) * a.k_ss, kofs, Ks + (unsigned)((wave + NW * i) * 8 * kKS8));
-        lds_dma16(vt0 + (int64_t)(8 * NW * i) * a.v_ss, vofs, Vs + (unsigned)((wave + NW * i) * 8 * kVS8));
+        lds_dma16(kt0 + (int64_t)(RPI * NW * i) * a.k_ss, kofs, Ks + (unsigned)((wave + NW * i) * RPI * kKS8));
+        lds_dma16(vt0 + (int64_t)(RPI * NW * i) * a.v_ss, vofs, Vs + (unsigned)((wave + NW * i) * RPI * kVS8));
       }
     } else {
 #pragma unroll
       for (int i = 0; i < GPW; ++i) {
         const int g = wave + NW * i;
-        int kk = kt * kBN8 + 8 * g + grow;
+        int kk = kt * kBN8 + RPI * g + grow;
         kk = kk < a.Skv ? kk : a.Skv - 1;
-        lds_dma16(kp + (int64_t)kk * a.k_ss + (((lane & 7) ^ kx_fill) * 16), Ks + (unsigned)(g * 8 * kKS8));
-        lds_dma16(vp + (int64_t)kk * a.v_ss + (((lane & 7) ^ vx_fill) * 16), Vs + (unsigned)(g * 8 * kVS8));
+        lds_dma16(kp + (int64_t)kk * a.k_ss + (((lane & (CPR - 1)) ^ kx_fill) * 16), Ks + (unsigned)(g * RPI * kKS8));
+        lds_dma16(vp + (int64_t)kk * a.v_ss + (((lane & (CPR - 1)) ^ vx_fill) * 16), Vs + (unsigned)(g * RPI * kVS8));
       }
     }
   };
 
-  f32x16 O[4];
+  f32x16 O[NSL];
 #pragma unroll
-  for (int sl = 0; sl < 4; ++sl)
+  for (int sl = 0; sl < NSL; ++sl)
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[sl][i] = 0.f;
   // When the whole logit scale c is a power of two (power-of-two q and k scales from the quantiser, the softmax
@@ -177,41 +186,43 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
 
   // lane-constant LDS offsets (bytes)
   // K fragment (d half j, 16-byte half i) of row l32 is logical chunk 4j + 2hh + i
-  int k_off[2][2];
+  int k_off[NJ][2];
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int j = 0; j < NJ; ++j)
 #pragma unroll
-    for (int i = 0; i < 2; ++i) k_off[j][i] = l32 * kKS8 + (((4 * j + 2 * hh + i) ^ ((l32 >> 1) & 7)) * 16);
-  int v_off[4];
+    for (int i = 0; i < 2; ++i)
+      k_off[j][i] = l32 * kKS8 + (((4 * j + 2 * hh + i) ^ (HD == 128 ? (l32 >> 1) & 7 : (l32 >> 2) & 3)) * 16);
+  int v_off[NSL];
   {
     const int e = (lane & 15) >> 1;
     const int rowl = 8 * (e >> 2) + 4 * hh + (e & 3);
-    const int fl = ((e >> 1) & 1) + 2 * ((e >> 2) & 1);
+    // the 32-byte slab's permutation key: row bits 1 and 3 (head dim 128), row bit 3 (head dim 64)
+    const int fl = HD == 128 ? ((e >> 1) & 1) + 2 * ((e >> 2) & 1) : (e >> 2) & 1;
     const int cl = 2 * ((lane >> 4) & 1) + (lane & 1);
 #pragma unroll
-    for (int sl = 0; sl < 4; ++sl) v_off[sl] = kBN8 * kKS8 + rowl * kVS8 + 32 * (sl ^ fl) + 8 * cl;
+    for (int sl = 0; sl < NSL; ++sl) v_off[sl] = kBN8 * kKS8 + rowl * kVS8 + 32 * (sl ^ fl) + 8 * cl;
   }
 
   auto tile = [&](int t, int slot, auto masked) __attribute__((always_inline)) {
     const char* Ks = smem8 + slot * kStage8;
     // ---- S^T = K.Q^T for one 32-key block
     auto qk = [&](f32x16& S, int blk, const char* Kb) __attribute__((always_inline)) {
-      i32x8 kf[2];
+      i32x8 kf[NJ];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         const u32x4 lo = *reinterpret_cast<const u32x4*>(Kb + k_off[j][0] + blk * 32 * kKS8);
         const u32x4 hi = *reinterpret_cast<const u32x4*>(Kb + k_off[j][1] + blk * 32 * kKS8);
         kf[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
       }
       if constexpr (PRE) {  // logits in log2 units minus the reference point, straight out of the MFMAs
-        const f32x16 z = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[0], qf[0], negref, 0, 0, 0, 127, 0, sexp);
-        S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], z, 0, 0, 0, 127, 0, sexp);
+        S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[0], qf[0], negref, 0, 0, 0, 127, 0, sexp);
+        if constexpr (NJ == 2) S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], S, 0, 0, 0, 127, 0, sexp);
       } else {
         f32x16 z;
 #pragma unroll
         for (int i = 0; i < 16; ++i) z[i] = 0.f;
-        z = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[0], qf[0], z, 0, 0, 0, 0, 0, 0);
-        S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], z, 0, 0, 0, 0, 0, 0);
+        S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[0], qf[0], z, 0, 0, 0, 0, 0, 0);
+        if constexpr (NJ == 2) S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], S, 0, 0, 0, 0, 0, 0);
       }
       if constexpr (BIAS) {
         if (t * kBN8 + 32 * blk < bias_cols) {  // a block wholly past the keys (last tile) is masked below anyway
@@ -304,7 +315,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       asm volatile("" : "+v"(alpha));  // keeps the rescale inside this rarely taken branch
       l *= alpha;
 #pragma unroll
-      for (int sl = 0; sl < 4; ++sl)
+      for (int sl = 0; sl < NSL; ++sl)
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[sl][i] *= alpha;
       // once more against the new reference points
@@ -321,7 +332,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
     l += ls;
     // ---- O^T += V^T.P^T
 #pragma unroll
-    for (int sl = 0; sl < 4; ++sl) {
+    for (int sl = 0; sl < NSL; ++sl) {
       const char* vsrc = Ks + v_off[sl];
       const i32x2 r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_ptr)(vsrc));
       const i32x2 r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_ptr)(vsrc + 16 * kVS8));
@@ -357,7 +368,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   if (row < a.Sq) {
     __bf16* orow = op + (int64_t)row * a.o_ss + 4 * hh;
 #pragma unroll
-    for (int sl = 0; sl < 4; ++sl)
+    for (int sl = 0; sl < NSL; ++sl)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         uint2 u;
@@ -369,26 +380,26 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
   }
 }
 
-template <int NW>
+template <int NW, int HD>
 int launch_fwd8(hipStream_t st, Fp8Args a, int B, int softmax_mode) {
   constexpr int BM = NW * 32;
-  constexpr int lds_bytes = kSlots8 * kStage8;
+  constexpr int lds_bytes = kSlots8 * 2 * kBN8 * HD;
   a.nqt = (a.Sq + BM - 1) / BM;
   const int64_t total = (int64_t)B * a.H * a.nqt;
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
   if (a.bias) {  // one instance for every kind of scale
-    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 0, true>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 0, true, HD>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
     return launch_status();
   }
-  hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 0>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 0, false, HD>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   // Power-of-two logit scale (the instance above then returns at once, this one otherwise): exp2, or the
   // exponential-free softmax when the caller asked for it.
   if (softmax_mode == MDATTN_FP8_SOFTMAX_BYTE_GRID)
-    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 2>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 2, false, HD>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   else
-    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 1>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 1, false, HD>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   return launch_status();
 }
 
@@ -408,7 +419,7 @@ static int fp8_run(void* stream, const void* q8, const void* k8, const void* v8,
   if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return MDATTN_E_BADARG;
   if (!q_strides || !k_strides || !v_strides || !o_strides) return MDATTN_E_BADARG;
   if (!(scale > 0.f) || !(scale < 1e30f)) return MDATTN_E_BADARG;
-  if (D != kD8) return MDATTN_E_UNSUPPORTED;
+  if (D != 128 && D != 64) return MDATTN_E_UNSUPPORTED;
   if (!aligned16(q8) || !aligned16(k8) || !aligned16(v8) || !aligned16(out) || (reinterpret_cast<uintptr_t>(lse) & 3u) ||
       (reinterpret_cast<uintptr_t>(q_scale) & 3u) || (reinterpret_cast<uintptr_t>(k_scale) & 3u) ||
       (reinterpret_cast<uintptr_t>(v_scale) & 3u))
@@ -438,7 +449,7 @@ static int fp8_run(void* stream, const void* q8, const void* k8, const void* v8,
   }
   hipStream_t st = (hipStream_t)stream;
   // Four waves per workgroup (three workgroups per CU) measured faster than eight at every shape tried.
-  return launch_fwd8<4>(st, a, B, softmax_mode);
+  return D == 128 ? launch_fwd8<4, 128>(st, a, B, softmax_mode) : launch_fwd8<4, 64>(st, a, B, softmax_mode);
 }
 
 

@@ -213,6 +213,42 @@ def test_fp8_softmax_mode_is_an_argument_of_the_abi(dev, lib):
   torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("sq,skv", [(1, 1), (31, 65), (257, 63), (300, 333), (64, 4097), (513, 512)])
+@pytest.mark.parametrize("scales,softmax", MODES)
+def test_fp8_head_dim_64(dev, sq, skv, scales, softmax):
+  """LTX-2's audio stream (heads of 64, models/ltx2/transformer_ltx2.py:788-789): one QK MFMA per key block, two
+  slabs of d, 64-byte rows in LDS.  Same bars as head dim 128."""
+  pow2, grid = scales == "pow2", softmax == "byte_grid"
+  B, H, D = 2, 3, 64
+  q, k, v = O.normal_bf16((B, sq, H, D), 0), O.normal_bf16((B, skv, H, D), 1), O.normal_bf16((B, skv, H, D), 2)
+  for layout in ("bshd", "bhsd"):
+    kw = {}
+    if layout == "bhsd":
+      kw["out_layout"] = "bhsd"
+    out, lse = _quant_run(q, k, v, dev, pow2=pow2, softmax=softmax, **kw)
+    for b in range(B):
+      qb, kb, vb = hsd(q[b:b + 1]), hsd(k[b:b + 1]), hsd(v[b:b + 1])
+      exact, lse_exact = O.attention(qb, kb, vb, D**-0.5)
+      got = hsd(out[b:b + 1])
+      assert cosine(got, exact) >= COS_BAR, (layout, b)
+      assert np.abs(lse[b] - lse_exact).max() <= 0.25
+
+
+def test_fp8_head_dim_64_against_emulation(dev):
+  """One batch element (the emulation takes per-tensor scales from the tensors it is given): the kernel's rounding
+  points at head dim 64 are the emulation's, so only f32 summation order differs."""
+  H, D, sq, skv = 3, 64, 300, 333
+  q, k, v = O.normal_bf16((1, sq, H, D), 0), O.normal_bf16((1, skv, H, D), 1), O.normal_bf16((1, skv, H, D), 2)
+  for scales, softmax in MODES:
+    pow2, grid = scales == "pow2", softmax == "byte_grid"
+    out, lse = _quant_run(q, k, v, dev, pow2=pow2, softmax=softmax)
+    emu, lse_emu = O.attention_fp8_emulated(hsd(q), hsd(k), hsd(v), D**-0.5, pow2_scales=pow2, code_softmax=grid)
+    dl = np.abs(lse[0] - lse_emu)
+    print(f"fp8 D=64 {scales} {softmax}: rel-l2 vs emulation {rel_l2(hsd(out), emu):.3e}, lse {dl.max():.2e}", flush=True)
+    assert cosine(hsd(out), emu) >= 0.99999 and rel_l2(hsd(out), emu) <= 5e-3
+    assert (np.mean(dl <= 1e-3) >= 0.98 and dl.max() <= 0.13) if grid else dl.max() <= 1e-3
+
+
 def test_fp8_cross_attention_shape(dev):
   # configs[2] cross-attention shape: 512 text keys
   H, Sq, Skv = 8, 2048, 512
@@ -254,13 +290,14 @@ def test_fp8_seeded_sweep_of_shapes_layouts_and_scale_kinds(dev):
 
 @pytest.mark.parametrize("sq,skv,kind", [(70, 333, "random"), (257, 512, "prefix"), (64, 97, "holes"), (33, 64, "one"), (40, 50, "none")])
 @pytest.mark.parametrize("pow2", [False, True])
-def test_fp8_with_key_mask(dev, sq, skv, kind, pow2):
+@pytest.mark.parametrize("D", [128, 64])
+def test_fp8_with_key_mask(dev, D, sq, skv, kind, pow2):
   """mdattn_fwd_fp8_bias: a [B,Skv] keep-mask as an additive key bias.  The masked result must be the attention over
   the kept keys only: against the f32 oracle with the mask (cosine bar), and against the fp8 kernel itself run,
   without a mask, on the kept keys of the same quantised operands (only the tiling of the keys differs, so only the
   e4m3 rounding grid of P moves).  Batch elements without a kept key return out = 0, lse = -inf."""
   B, H = 2, 2
-  q, k, v = O.normal_bf16((B, sq, H, 128), 0), O.normal_bf16((B, skv, H, 128), 1), O.normal_bf16((B, skv, H, 128), 2)
+  q, k, v = O.normal_bf16((B, sq, H, D), 0), O.normal_bf16((B, skv, H, D), 1), O.normal_bf16((B, skv, H, D), 2)
   rng = np.random.default_rng(5)
   keep = np.ones((B, skv), bool)
   if kind == "random":
@@ -280,11 +317,11 @@ def test_fp8_with_key_mask(dev, sq, skv, kind, pow2):
     keep[1] = False
   qd, kd, vd = (to_dev_bf16(x, dev) for x in (q, k, v))
   if pow2:
-    q8, sq_ = ops.quant_e4m3(qd, premul=ops.folded_q_mul(128), pow2_scale=True)
+    q8, sq_ = ops.quant_e4m3(qd, premul=ops.folded_q_mul(D), pow2_scale=True)
     k8, sk_ = ops.quant_e4m3(kd, pow2_scale=True)
     sc = ops.FOLDED_SCALE
   else:
-    (q8, sq_), (k8, sk_), sc = ops.quant_e4m3(qd), ops.quant_e4m3(kd), 128**-0.5
+    (q8, sq_), (k8, sk_), sc = ops.quant_e4m3(qd), ops.quant_e4m3(kd), D**-0.5
   v8, sv_ = ops.quant_e4m3(vd)
   keep_d = torch.from_numpy(keep).to(dev)
   out, lse = ops.flash_attention_fp8(q8, k8, v8, sq_, sk_, sv_, scale=sc, return_lse=True, key_bias=ops.key_mask_bias(keep_d))
@@ -292,7 +329,7 @@ def test_fp8_with_key_mask(dev, sq, skv, kind, pow2):
     if not keep[b].any():
       assert torch.count_nonzero(out[b]) == 0 and bool(torch.isneginf(lse[b]).all())
       continue
-    exact, lse_exact = O.attention(hsd(q[b:b + 1]), hsd(k[b:b + 1]), hsd(v[b:b + 1]), 128**-0.5, kv_mask=keep[b])
+    exact, lse_exact = O.attention(hsd(q[b:b + 1]), hsd(k[b:b + 1]), hsd(v[b:b + 1]), D**-0.5, kv_mask=keep[b])
     assert cosine(hsd(to_np(out[b:b + 1])), exact) >= COS_BAR, (kind, b)
     assert np.abs(to_np(lse[b]) - lse_exact).max() <= 0.25
     sub, sub_l = ops.flash_attention_fp8(q8[b:b + 1], k8[b:b + 1, keep_d[b]], v8[b:b + 1, keep_d[b]], sq_, sk_, sv_, scale=sc, return_lse=True)
