@@ -544,7 +544,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
 
   auto tile = [&](int t, int slot, auto masked) __attribute__((always_inline)) {
     const __bf16* base = smem + slot * STAGE;
-    // ---- S^T = K.Q^T: one chain of MFMAs; the other waves of the SIMD fill the gaps between them
+    // ---- S^T = K.Q^T: one chain of MFMAs; the other waves of the SIMD fill the gaps between them.  A wave in an
+    // MFMA phase issues ahead of the SIMD's waves in their softmax phase (1-2 % on short key sequences).
+    __builtin_amdgcn_s_setprio(1);
     f32x16 S;
 #pragma unroll
     for (int i = 0; i < 16; ++i) S[i] = 0.f;
@@ -571,6 +573,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
     // current reference point, and only a partial sum above kTrig (a logit far above the reference, or
     // many a little above) sends the wave through the branch that moves every row's reference to its true
     // maximum, rescales the accumulators and redoes the tile's P.
+    __builtin_amdgcn_s_setprio(0);
     bf16x8 P[2];
     auto soft = [&](float rf) __attribute__((always_inline)) {
       float lsum = 0.f;
@@ -614,6 +617,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(3, 3)))
       lsum = soft(mc);
     }
     l += lsum;
+    __builtin_amdgcn_s_setprio(1);
     // ---- O^T += V^T.P^T
 #pragma unroll
     for (int jv = 0; jv < 2 * ND; ++jv) {

@@ -114,6 +114,36 @@ def test_backward_wan13b_shape_against_torch_autograd_on_gpu(dev):
     _check(to_np(got), to_np(t.grad.permute(0, 2, 1, 3)), f"wan1.3b {name}")
 
 
+@pytest.mark.parametrize("folded", [False, True])
+def test_backward_wan14b_usp_shard_full_size(dev, folded):
+  """The shape `bench.py --workload wan14b-usp --with-backward` times (20 heads x 18,900 tokens), whole tensors,
+  head by head against torch's f32 autograd on the GPU (test harness only); `folded`: q carries the softmax scale and
+  scale = ln 2, which selects the kernels whose logits leave the MFMAs in log2 units."""
+  import math
+  H, S, D = 20, 18900, 128
+  gen = torch.Generator(device=dev).manual_seed(11)
+  q, k, v, do = (torch.randn((1, S, H, D), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(4))
+  scale = D**-0.5
+  if folded:
+    q = (q.float() * (scale * math.log2(math.e))).to(torch.bfloat16)
+    scale = math.log(2.0)
+  out, lse = ops.flash_attention(q, k, v, scale=scale, return_lse=True)
+  dq, dk, dv = ops.flash_attention_backward(q, k, v, out, do, lse, scale=scale)
+  worst = {}
+  for h in (range(H) if not folded else (0, 7, 13, 19)):
+    tq, tk, tv = (x[:, :, h].float().detach().requires_grad_(True) for x in (q, k, v))  # [1,S,D]
+    p = torch.softmax((tq @ tk.transpose(1, 2)) * scale, dim=-1)
+    (p @ tv).backward(do[:, :, h].float())
+    for name, got, t in (("dq", dq, tq), ("dk", dk, tk), ("dv", dv, tv)):
+      g, r = got[:, :, h].float(), t.grad
+      rel = float((g - r).norm() / r.norm())
+      mx = float((g - r).abs().max() / r.abs().max())
+      worst[name] = max(worst.get(name, (0.0, 0.0)), (rel, mx))
+      assert rel <= 6e-3 and mx <= 1.5e-2, (name, h, rel, mx)
+    del p, tq, tk, tv
+  print(f"usp backward folded={folded}: worst (rel-l2, max-abs/max|ref|) {worst}", flush=True)
+
+
 def test_autograd_function(dev):
   from maxdiffusion_amd import attention_op
 
