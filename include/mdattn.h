@@ -254,8 +254,12 @@ int mdattn_fwd_fp8_bias(void* stream, const void* q8, const void* k8, const void
  * kernels/splash_attention/splash_attention_kernel.py:1277-1600, with `scale` applied inside (logits = scale*q.k).
  *   dout, out    bf16 [B,Sq,H,D] by o_strides;  dq by q_strides;  dk by k_strides;  dv by v_strides
  *   lse          f32 [B,H,Sq] as written by the forward
- *   workspace    f32 device buffer of at least mdattn_bwd_workspace_floats(B,H,Sq) elements, 16-byte aligned
- * Requires D == 128 or D == 64 (LTX-2's audio stream).
+ *   workspace    f32 device buffer of at least mdattn_bwd_workspace_floats(B,H,Sq) elements, 16-byte aligned;
+ *                scratch of the call (per padded q row: -lse in log2 units and -rowsum(dout*out)), nothing to keep
+ * Two passes, no atomics: dq; then dk and dv together.  When scale * log2(e) == 1 (the caller's q carries the softmax
+ * scale, as for the forward) the logits need no multiply; dq is then the gradient for the q that was passed.
+ * Requires D == 128 or D == 64 (LTX-2's audio stream); sequence strides below 2^23 elements and
+ * B * H * ceil32(Sq) below 2^29 (MDATTN_E_UNSUPPORTED beyond).
  */
 int64_t mdattn_bwd_workspace_floats(int B, int H, int Sq);
 int mdattn_bwd_bf16(void* stream, const void* q, const void* k, const void* v, const void* out, const void* dout,
