@@ -67,3 +67,42 @@ def test_captured_step_replays_to_the_eager_result(dev):
     got = list(captured) + [o_run, l_run]
     for i, (g, w) in enumerate(zip(got, want)):
       assert torch.equal(g, w), f"replay {rep}: output {i} differs from the eager result"
+
+
+def test_captured_forward_and_static_backward_replay_to_the_eager_result(dev):
+  """A training step under capture: forward with lse, then the backward through the entry point that allocates nothing
+  (its scratch is the library's static device array; the per-device address lookup happens on the warm-up call)."""
+  B, H, Sq, Skv = 2, 3, 333, 500
+  q, do = (to_dev_bf16(O.normal_bf16((B, Sq, H, 128), s), dev) for s in (0, 3))
+  k, v = (to_dev_bf16(O.normal_bf16((B, Skv, H, 128), s), dev) for s in (1, 2))
+  out, lse = ops.flash_attention(q, k, v, return_lse=True)
+  want = [t.clone() for t in ops.flash_attention_backward(q, k, v, out, do, lse)]
+  grads = [torch.empty_like(t) for t in (q, k, v)]
+
+  def step():
+    o, l = ops.flash_attention(q, k, v, return_lse=True)  # torch's capture-time allocator; the library allocates nothing
+    ops.flash_attention_backward_static(q, k, v, o, do, l, *grads)
+    return o, l
+
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    step()
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    out_c, lse_c = step()
+  for rep in range(3):
+    for t in grads + [out_c, lse_c]:
+      t.fill_(float(rep) + 0.25)
+    # eager work between the replays, including a backward that uses the same static scratch with another shape
+    qq, kk = (to_dev_bf16(O.normal_bf16((1, 70 + rep, 2, 128), 40 + s), dev) for s in (0, 1))
+    oo, ll = ops.flash_attention(qq, kk, kk, return_lse=True)
+    ops.flash_attention_backward_static(qq, kk, kk, oo, oo, ll, torch.empty_like(qq), torch.empty_like(kk), torch.empty_like(kk))
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out_c, out) and torch.equal(lse_c, lse), f"replay {rep}: forward differs"
+    for i, (g, w) in enumerate(zip(grads, want)):
+      assert torch.equal(g, w), f"replay {rep}: gradient {i} differs from the eager result"
