@@ -99,18 +99,25 @@ def source_id() -> str:
   return h.hexdigest()[:16]
 
 
+def built_library_id(path: str | None = None) -> str | None:
+  """The source id a built library carries, read from the file (nothing is loaded), or None."""
+  path = path or LIB_PATH
+  marker = b"mdattn-build-id:"
+  try:
+    with open(path, "rb") as f:
+      data = f.read()
+  except OSError:
+    return None
+  i = data.find(marker)
+  if i < 0:
+    return None
+  j = data.find(b"\0", i)
+  return data[i + len(marker):j].decode(errors="replace")
+
+
 def library_is_current() -> bool:
   """True when libmdattn.so exists and was built from the sources in this tree."""
-  if not os.path.exists(LIB_PATH):
-    return False
-  import ctypes
-
-  try:
-    fn = ctypes.CDLL(LIB_PATH).mdattn_build_id
-  except (OSError, AttributeError):
-    return False
-  fn.restype = ctypes.c_char_p
-  return fn().decode() == source_id()
+  return built_library_id() == source_id()
 
 
 def ensure_built(verbose: bool = True) -> str:
@@ -123,14 +130,20 @@ def ensure_built(verbose: bool = True) -> str:
 
 def build_library(verbose: bool = True) -> str:
   """Compile every HIP source into maxdiffusion_amd/libmdattn.so.  Always recompiles."""
+  # Linked under another name and moved into place: a process that has the previous library mapped keeps its own
+  # file, and a later dlopen of the path finds the new one instead of the handle it already holds.
+  tmp = LIB_PATH + f".{os.getpid()}.tmp"
   cmd = [_hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", f'-DMDATTN_BUILD_ID="{source_id()}"',
-         f"-I{INCLUDE}", f"-I{CSRC}", "-o", LIB_PATH, *[os.path.join(CSRC, s) for s in SOURCES]]
+         f"-I{INCLUDE}", f"-I{CSRC}", "-o", tmp, *[os.path.join(CSRC, s) for s in SOURCES]]
   if verbose:
     print("[maxdiffusion_amd.build]", " ".join(cmd), flush=True)
   r = subprocess.run(cmd, capture_output=True, text=True)
   err = _filter(r.stderr)
   if r.returncode != 0:
+    if os.path.exists(tmp):
+      os.remove(tmp)
     raise RuntimeError(f"hipcc failed ({r.returncode}):\n{r.stdout}\n{err}")
+  os.replace(tmp, LIB_PATH)
   if verbose and err.strip():
     print(err, file=sys.stderr)
   if verbose:  # registers, spills and occupancy of every kernel: a spill in a hot loop shows here, not in a test

@@ -16,7 +16,10 @@ extern "C" int mdattn_set_fwd_schedule(int schedule) {
 #ifndef MDATTN_BUILD_ID
 #define MDATTN_BUILD_ID "unknown"
 #endif
-extern "C" const char* mdattn_build_id(void) { return MDATTN_BUILD_ID; }
+// The id sits behind a marker so that it can be read from the file without loading the library (a process that has
+// mapped a stale build cannot load the fresh one from the same path any more).
+static const char kBuildIdRecord[] = "mdattn-build-id:" MDATTN_BUILD_ID;
+extern "C" const char* mdattn_build_id(void) { return kBuildIdRecord + 16; }
 
 extern "C" int mdattn_version(void) { return MDATTN_VERSION; }
 

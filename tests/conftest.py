@@ -32,6 +32,15 @@ def pytest_collection_modifyitems(config, items):
       item.add_marker(skip)
 
 
+@pytest.fixture(scope="session", autouse=True)
+def _current_library():
+  """Before the first test of a session touches the library: make sure that what is built comes from the sources in the
+  tree (a test that loaded a stale library first would keep it mapped for the whole session)."""
+  from maxdiffusion_amd import build
+
+  build.ensure_built()
+
+
 @pytest.fixture(scope="session")
 def lib():
   """The built C-ABI library; built here only if nothing is built yet or what is built comes from other sources."""
