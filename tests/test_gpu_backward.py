@@ -222,3 +222,49 @@ def test_backward_with_key_mask(dev, D, sq, skv, kind):
     _check(hsd(dq[b:b + 1]), rq, f"masked {kind} D={D} dq b{b}")
     _check(hsd(dk[b:b + 1]), rk, f"masked {kind} D={D} dk b{b}")
     _check(hsd(dv[b:b + 1]), rv, f"masked {kind} D={D} dv b{b}")
+
+
+def test_backward_seeded_sweep_of_shapes_layouts_masks_and_scale_kinds(dev):
+  """Thirty seeded draws of (batch, heads, Sq, Skv, head dim, layout, sharpness, key mask or not, scale carried by q or
+  not) against torch's f32 autograd on the GPU (test harness only)."""
+  import math
+  import random
+  rnd = random.Random(21)
+  gen = torch.Generator(device=dev).manual_seed(21)
+  for it in range(30):
+    B, H, D = rnd.choice([1, 1, 2]), rnd.choice([1, 2, 3, 5]), rnd.choice([128, 128, 64])
+    sq = rnd.choice([1, 7, 31, 32, 33, 64, 100, 127, 128, 129, 255, 256, 257, 300, 513, 1000])
+    skv = rnd.choice([1, 2, 5, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 500, 1023, 1025, 2100])
+    layout, mult = rnd.choice(["bshd", "bhsd"]), rnd.choice([1.0, 1.0, 2.0, 4.0])
+    masked, folded = rnd.random() < 0.4, rnd.random() < 0.4
+    q, k, v, do = ((torch.randn((B, s_, H, D), generator=gen, device=dev) * m).to(torch.bfloat16)
+                   for s_, m in ((sq, mult), (skv, 1.0), (skv, 1.0), (sq, 1.0)))
+    scale = D**-0.5
+    if folded and not masked:
+      q = (q.float() * (scale * math.log2(math.e))).to(torch.bfloat16)
+      scale = math.log(2.0)
+    keep = None
+    if masked:
+      keep = torch.rand((B, skv), generator=gen, device=dev) < 0.7
+      keep[:, rnd.randrange(skv)] = True  # every batch element keeps a key
+    if layout == "bhsd":
+      q, k, v = (t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3) for t in (q, k, v))
+    bias = ops.key_mask_bias(keep) if masked else None
+    out, lse = ops.flash_attention(q, k, v, scale=scale, return_lse=True, out_layout=layout, key_bias=bias)
+    dq, dk, dv = ops.flash_attention_backward(q, k, v, out, do, lse, scale=scale, key_bias=bias)
+    tq, tk, tv = (x.float().permute(0, 2, 1, 3).detach().requires_grad_(True) for x in (q, k, v))  # [B,H,S,D]
+    s = (tq @ tk.transpose(2, 3)) * scale
+    if masked:
+      s = s.masked_fill(~keep[:, None, None, :], float("-inf"))
+    (torch.softmax(s, dim=-1) @ tv).backward(do.float().permute(0, 2, 1, 3))
+    what = f"draw {it}: B={B} H={H} D={D} Sq={sq} Skv={skv} {layout} x{mult} masked={masked} folded={folded and not masked}"
+    for name, got, t in (("dq", dq, tq), ("dk", dk, tk), ("dv", dv, tv)):
+      g, r = got.float(), t.grad.permute(0, 2, 1, 3)
+      assert bool(torch.isfinite(g).all()), f"{what} {name}"
+      den = float(r.norm())
+      if den < 1e-6:  # one key: the exact gradient is zero (see _check)
+        assert float(g.abs().max()) <= 0.25, f"{what} {name}"
+        continue
+      rel, mx = float((g - r).norm()) / den, float((g - r).abs().max() / r.abs().max())
+      # sharper logits (x2, x4) put more weight on fewer probabilities: the bf16 rounding of P and dS weighs more
+      assert rel <= (6e-3 if mult == 1.0 else 1e-2) and mx <= (1.5e-2 if mult == 1.0 else 3e-2), f"{what} {name}: rel-l2 {rel:.2e} max {mx:.2e}"
