@@ -268,7 +268,9 @@ def main():
     bms = e0.elapsed_time(e1) / 5
     # the five matrix products of the backward pass: S, dP, dV, dK, dQ (the two passes execute seven: S and dP are formed in both)
     bfl = 2.5 * O.attention_flops(1, H, S, Skv, D)
-    backward = {"Sq": S, "Skv": Skv, "ms": bms, "TFLOP/s": bfl / (bms * 1e-3) / 1e12,
+    btf = bfl / (bms * 1e-3) / 1e12
+    backward = {"Sq": S, "Skv": Skv, "ms": bms, "TFLOP/s": btf, "bound": "mfma", "peak": 2500.0, "frac": btf / 2500.0,
+                "frac_executed": btf * 7.0 / 5.0 / 2500.0,
                 "flop_counted": bfl, "note": "5 matrix products counted, 7 executed (two atomic-free passes: dq; dk and dv)"}
 
   flops = O.attention_flops(1, H, S, Skv * ring, D)
