@@ -422,9 +422,10 @@ __global__ __launch_bounds__((bwd_waves<HD>() * 64)) void attn_bwd_kernel(BwdArg
 }
 // The dk / dv pass at head dim 128 wants a few registers more than half the register file (128 accumulators, 64 of
 // entity fragments, 32 of S and dP): held to two waves per SIMD, which the schedule needs to overlap one wave's
-// exponentials with the other's MFMAs; at one wave per SIMD it measured 28 % slower.
+// exponentials with the other's MFMAs; at one wave per SIMD it measured 28 % slower.  Head dim 64 fits three waves
+// per SIMD (3 % faster than two).
 template <int HD, bool BIAS, bool PRE>
-__global__ __launch_bounds__((bwd_waves<HD>() * 64)) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_bwd_both_kernel(BwdArgs a) {
+__global__ __launch_bounds__((bwd_waves<HD>() * 64)) __attribute__((amdgpu_waves_per_eu(HD == 64 ? 3 : 2, HD == 64 ? 3 : 2))) void attn_bwd_both_kernel(BwdArgs a) {
   attn_bwd_body<3, HD, BIAS, PRE>(a);
 }
 
