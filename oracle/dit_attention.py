@@ -22,7 +22,14 @@ Pinning status of each function (what fixes it besides its own formula):
   ltx2_apply_split_rotary_emb    brute-force loop, norm preservation, and: split rotation of x equals
                                  the interleaved rotation of x with each head's halves interleaved
   norm_rope_fullrow / _perhead   compositions of rmsnorm and apply_rope_interleaved (both pinned above)
-  / _qkv                         plus, for _qkv, the bias add and the column split of the fused projection
+  norm_rope_qkv                  equals norm_rope_fullrow on the column blocks of the fused projection; the bias
+                                 add on a hand case (zero projection, constant bias blocks -> +-1 and the v bias)
+  norm_rope_wan_reference_flow   torch's CPU kernels on the same inputs: rms_norm in f32 cast to bf16, then the
+                                 rotation evaluated on bf16 tensors (every *, -, + returns bf16): >= 99.99 % of the
+                                 outputs bit-identical, while moving any single rounding point (table kept in f32,
+                                 products not rounded, norm output not rounded) drops the agreement below 95 %;
+                                 and inputs on which every rounding is exact, where it equals norm_rope_fullrow
+                                 bit for bit
   attention / attention_rows     scipy logsumexp, torch SDPA (fp32, CPU),
                                  invariants (K=0 -> mean(V), lse=ln Skv; ...),
                                  hand fixtures of tests/ltx2/test_attention_ltx2.py:38-116

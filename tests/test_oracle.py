@@ -190,6 +190,107 @@ def test_norm_rope_fused_vs_reference_rounding_flow():
   assert w.scale == 128**-0.5
 
 
+def _torch_bf16_wan_norm_rope(x, w, cos, sin, heads, eps=1e-6):
+  """The Wan prologue with a library deciding every rounding: torch's rms_norm in f32 cast to bf16 (the one rounding
+  flax's RMSNorm does, attention_flax.py:2529-2553), then the rotation as torch's CPU bf16 kernels evaluate
+  `y0*c - y1*s`, `y0*s + y1*c` on bf16 tensors: each `*`, `-` and `+` returns a bf16 tensor (attention_flax.py:2598-2613)."""
+  b, s, n = x.shape
+  y = torch.nn.functional.rms_norm(torch.from_numpy(x), (n,), torch.from_numpy(w), eps=eps).to(torch.bfloat16)
+  y = y.reshape(b, s, heads, n // heads // 2, 2)
+  c = torch.from_numpy(cos).to(torch.bfloat16)[None, :, None, :]
+  sn = torch.from_numpy(sin).to(torch.bfloat16)[None, :, None, :]
+  y0, y1 = y[..., 0], y[..., 1]
+  out = torch.stack([y0 * c - y1 * sn, y0 * sn + y1 * c], dim=-1)
+  assert out.dtype == torch.bfloat16
+  return out.reshape(b, s, heads, n // heads).float().numpy()
+
+
+def test_reference_rounding_flow_matches_torch_bf16_kernels():
+  """Pins norm_rope_wan_reference_flow to a library's bf16 arithmetic.  The elementwise bf16 kernels leave no freedom
+  (no summation order), so the two sides can differ only where the f32 normalised value sits within an f32 ulp of a
+  bf16 rounding boundary (x/sqrt(.)*w here, x*rsqrt(.)*w in the library): a stated, tiny fraction, one bf16 step of y.
+  Variants of the flow with one rounding point moved do not reach that agreement, so the test tells them apart."""
+  H, D, grid = 12, 128, (3, 5, 7)
+  S = grid[0] * grid[1] * grid[2]
+  cos, sin = O.wan_rope_table(grid, D)
+  for seed, mult in ((0, 1.0), (5, 4.0)):
+    x = O.bf16_round(O.normal_bf16((2, S, H * D), seed) * np.float32(mult))
+    w = O.norm_weight(H * D, 3)
+    flow = O.norm_rope_wan_reference_flow(x, w, cos, sin, H)
+    lib = _torch_bf16_wan_norm_rope(x, w, cos, sin, H)
+    same = float(np.mean(flow == lib))
+    assert same >= 0.9999, (seed, same)  # observed: 1.0 and 0.99998
+    # the rest: one bf16 step of y carried through the rotation (|y| < 8 here: a step is at most 2^-5, times |c|+|s|)
+    assert np.abs(flow - lib).max() <= 2.0**-5 * 1.5
+
+    def variant(round_y=True, round_table=True, round_products=True):
+      r = O.bf16_round
+      b = x.shape[0]
+      y = O.rmsnorm(x, w, 1e-6, np.float32)
+      y = (r(y) if round_y else y).reshape(b, S, H, D // 2, 2)
+      c = (r(cos) if round_table else cos)[None, :, None, :]
+      sn = (r(sin) if round_table else sin)[None, :, None, :]
+      p = r if round_products else (lambda t: t)
+      y0, y1 = y[..., 0], y[..., 1]
+      return np.stack([r(p(y0 * c) - p(y1 * sn)), r(p(y0 * sn) + p(y1 * c))], axis=-1).reshape(b, S, H, D)
+
+    np.testing.assert_array_equal(variant(), flow)
+    # (a third of the table entries are the identity rotation -- position 0 along an axis -- where the table and the
+    # products round exactly; the fractions below are over all entries)
+    assert float(np.mean(variant(round_table=False) == lib)) < 0.95     # table left in f32: observed 0.917
+    assert float(np.mean(variant(round_products=False) == lib)) < 0.95  # products not rounded: observed 0.887
+    assert float(np.mean(variant(round_y=False) == lib)) < 0.95         # norm output not rounded: observed 0.908
+    fused = O.bf16_round(O.norm_rope_fullrow(x, w, cos, sin, H).astype(np.float32))
+    assert float(np.mean(fused == lib)) < 0.85                          # the fused kernel's single rounding: 0.752
+
+
+def test_reference_rounding_flow_exact_case():
+  """Inputs on which every rounding of the bf16 flow is exact, so that it must equal the exact prologue bit for bit:
+  x = +-2 everywhere with eps = 0 (mean square 4, normalised values +-1), small power-of-two weights, and tables whose
+  entries are powers of two (the rotation formula is evaluated as given; nothing requires cos^2 + sin^2 = 1)."""
+  rng = np.random.default_rng(11)
+  H, D, S = 2, 16, 6
+  x = (2.0 * rng.choice([-1.0, 1.0], size=(1, S, H * D))).astype(np.float32)
+  w = rng.choice([0.5, 1.0, 2.0, 4.0], size=H * D).astype(np.float32)
+  cos = rng.choice([0.25, 0.5, 1.0, -0.5], size=(S, D // 2)).astype(np.float32)
+  sin = rng.choice([0.125, -0.25, 2.0, 0.0], size=(S, D // 2)).astype(np.float32)
+  flow = O.norm_rope_wan_reference_flow(x, w, cos, sin, H, eps=0.0)
+  exact = O.norm_rope_fullrow(x, w, cos, sin, H, eps=0.0)
+  np.testing.assert_array_equal(flow, exact.astype(np.float32))
+  # hand value: pair (y0, y1) = (w0*sgn0, w1*sgn1) -> (y0 c - y1 s, y0 s + y1 c)
+  y = (x[0, 3] / 2.0 * w).reshape(H, D // 2, 2)
+  want0 = y[1, 5, 0] * cos[3, 5] - y[1, 5, 1] * sin[3, 5]
+  want1 = y[1, 5, 0] * sin[3, 5] + y[1, 5, 1] * cos[3, 5]
+  assert flow[0, 3, 1, 10] == want0 and flow[0, 3, 1, 11] == want1
+
+
+def test_norm_rope_qkv_is_the_prologue_on_the_column_blocks():
+  """norm_rope_qkv: q and k blocks equal norm_rope_fullrow of the (biased) column slices, v is the biased value block;
+  the bias add is checked on a hand case (a zero projection output: every token row is the bias itself)."""
+  H, D, grid = 3, 32, (2, 3, 2)
+  S, n = 12, 3 * 32
+  cos, sin = O.wan_rope_table(grid, D)
+  rng = np.random.default_rng(12)
+  qkv = rng.standard_normal((2, S, 3 * n))
+  bias = rng.standard_normal(3 * n)
+  wq, wk = 1 + 0.1 * rng.standard_normal(n), 1 + 0.1 * rng.standard_normal(n)
+  q, k, v = O.norm_rope_qkv(qkv, wq, wk, cos, sin, H)
+  np.testing.assert_array_equal(q, O.norm_rope_fullrow(qkv[..., :n], wq, cos, sin, H))
+  np.testing.assert_array_equal(k, O.norm_rope_fullrow(qkv[..., n:2 * n], wk, cos, sin, H))
+  np.testing.assert_array_equal(v, qkv[..., 2 * n:].reshape(2, S, H, D))
+  qb, kb, vb = O.norm_rope_qkv(qkv, wq, wk, cos, sin, H, bias=bias)
+  shifted = qkv + bias
+  np.testing.assert_allclose(qb, O.norm_rope_fullrow(shifted[..., :n], wq, cos, sin, H), rtol=1e-13, atol=1e-13)
+  np.testing.assert_allclose(kb, O.norm_rope_fullrow(shifted[..., n:2 * n], wk, cos, sin, H), rtol=1e-13, atol=1e-13)
+  # hand case: zero projection, constant bias blocks c_q, c_k, c_v, unit weights, no rotation, eps = 0:
+  # every normalised element is sign(c) (a constant row has RMS |c|) and v is c_v
+  hb = np.concatenate([np.full(n, 3.0), np.full(n, -0.5), np.full(n, 7.0)])
+  q0, k0, v0 = O.norm_rope_qkv(np.zeros((1, 2, 3 * n)), np.ones(n), np.ones(n), None, None, H, bias=hb, eps=0.0)
+  np.testing.assert_allclose(q0, 1.0, rtol=1e-15)
+  np.testing.assert_allclose(k0, -1.0, rtol=1e-15)
+  np.testing.assert_array_equal(v0, np.full((1, 2, H, D), 7.0))
+
+
 # ----------------------------------------------------------------------------- attention + LSE
 def test_attention_lse_matches_scipy_and_out_matches_torch_sdpa():
   rng = np.random.default_rng(8)
