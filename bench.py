@@ -304,7 +304,10 @@ def main():
                                                              if fp8 else "bf16 flash-attention forward with LSE (softmax scale * log2 e carried by the prologue's q output)")},
       "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                    "frac": achieved / peak, "traffic": traffic.get(kname), "kernel": klabel,
-                   "kernel_ms": att_ms, "flop_per_launch": flops / ring},
+                   "kernel_ms": att_ms, "flop_per_launch": flops / ring,
+                   # spread over the timed steps: the shader clock under this kernel differs from box to box and drifts
+                   # within a run, so one average does not place the run; min / median / max do
+                   "kernel_ms_min": min(t_att), "kernel_ms_median": sorted(t_att)[len(t_att) // 2], "kernel_ms_max": max(t_att)},
       "roofline_norm_rope": {"bound": "hbm", "achieved": nr_bytes / (pro_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                              "frac": nr_bytes / (pro_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "traffic": traffic.get(f"norm_rope_{w.norm}_kernel"),
                              "kernel": f"norm_rope_{w.norm}_kernel" + (" (two launches: q, k)" if w.norm == "rows" else ""),

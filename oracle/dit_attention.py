@@ -34,6 +34,11 @@ Pinning status of each function (what fixes it besides its own formula):
                                  invariants (K=0 -> mean(V), lse=ln Skv; ...),
                                  hand fixtures of tests/ltx2/test_attention_ltx2.py:38-116
   attention_bwd                  torch autograd through torch SDPA (fp64, CPU), finite differences
+  rmsnorm_bwd / norm_rope_*_bwd  torch autograd (fp64, CPU) through torch.nn.functional.rms_norm and a rotation
+                                 written as a complex multiply (view_as_complex) or, for LTX-2's two forms, with
+                                 torch index arithmetic; central finite differences of the forward oracle; and the
+                                 closed-form facts: du is orthogonal to u when eps = 0 (the norm is scale-invariant),
+                                 and a rotation-only chain returns the inverse rotation of the gradient
   merge_lse / merge_mlo /        attention over a union of KV chunks equals the
   merge_scan_ring                merge of per-chunk results (brute force)
   attention_dot_product_bf16     torch's CPU bf16 kernels (matmul with bf16 result, bf16 scale multiply,
@@ -62,7 +67,8 @@ __all__ = [
     "flux_ids", "flux_rope_angles", "flux_rope_table", "flux_rope_table_matrix",
     "apply_rope_interleaved", "apply_rope_matrix_form", "norm_rope_fullrow", "norm_rope_qkv", "norm_rope_perhead",
     "norm_rope_wan_reference_flow", "attention", "attention_rows", "attention_dot_product_bf16",
-    "ltx2_apply_rotary_emb", "ltx2_apply_split_rotary_emb", "norm_rope_ltx2", "attention_bwd", "merge_lse", "merge_mlo", "merge_scan_ring", "ring_replay", "quant_e4m3", "attention_fp8_emulated",
+    "ltx2_apply_rotary_emb", "ltx2_apply_split_rotary_emb", "norm_rope_ltx2", "attention_bwd",
+    "rmsnorm_bwd", "norm_rope_fullrow_bwd", "norm_rope_perhead_bwd", "norm_rope_ltx2_bwd", "merge_lse", "merge_mlo", "merge_scan_ring", "ring_replay", "quant_e4m3", "attention_fp8_emulated",
     "LSE_INIT",
 ]
 
@@ -405,6 +411,72 @@ def attention_bwd(q, k, v, do, scale: float, dtype=np.float64, kv_mask=None):
   dq = np.matmul(ds, k) * dtype(scale)
   dk = np.matmul(np.swapaxes(ds, -1, -2), q) * dtype(scale)
   return dq, dk, dv
+
+
+# --------------------------------------------------------------------------- backward of the prologue
+def rmsnorm_bwd(x, w, dy, eps: float = 1e-6, dtype=np.float64):
+  """VJP of `rmsnorm`: (dx, dw) for an upstream gradient dy of y = x * r * w, r = rsqrt(mean(x^2) + eps).
+
+  dx = r * (w dy) - x * r^3 * mean(x w dy);  dw = sum over every leading axis of dy * x * r.  The reference has no
+  hand-written backward: q and k gradients flow through nnx.RMSNorm by JAX autodiff (attention_flax.py:2655-2677)."""
+  x, dy = np.asarray(x, dtype), np.asarray(dy, dtype)
+  w = np.asarray(w, dtype)
+  r = 1.0 / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + dtype(eps))
+  wdy = w * dy
+  dx = r * wdy - x * r**3 * np.mean(x * wdy, axis=-1, keepdims=True)
+  dw = (dy * x * r).reshape(-1, x.shape[-1]).sum(axis=0)
+  return dx, dw
+
+
+def _rope_interleaved_transposed(g, cos, sin, seq_axis: int = -3):
+  """Transpose (= inverse, for unit-modulus tables) of `apply_rope_interleaved`: the rotation by -angle."""
+  return apply_rope_interleaved(g, cos, -np.asarray(sin), seq_axis)
+
+
+def norm_rope_fullrow_bwd(x, w, cos, sin, heads: int, g, eps: float = 1e-6, q_mul: float = 1.0, bias=None, dtype=np.float64):
+  """VJP of q_mul * norm_rope_fullrow(x + bias): g [B,S,H,D] -> (dx [B,S,H*D], dw [H*D]) (d bias = dx summed over
+  tokens).  The gradient is rotated back (transposed rotation), then goes through the RMSNorm VJP."""
+  b, s, hd = x.shape
+  g = np.asarray(g, dtype) * dtype(q_mul)
+  if cos is not None:
+    g = _rope_interleaved_transposed(g, cos, sin, seq_axis=-3)
+  u = np.asarray(x, dtype) + (0.0 if bias is None else np.asarray(bias, dtype))
+  return rmsnorm_bwd(u, w, g.reshape(b, s, hd), eps, dtype)
+
+
+def norm_rope_perhead_bwd(x, w, cos, sin, g, eps: float = 1e-6, q_mul: float = 1.0, w_txt=None, n_txt: int = 0, dtype=np.float64):
+  """VJP of q_mul * norm_rope_perhead: x, g [B,L,H,D] -> (dx, dw [D], dw_txt [D] or None)."""
+  g = np.asarray(g, dtype) * dtype(q_mul)
+  if cos is not None:
+    g = _rope_interleaved_transposed(g, cos, sin, seq_axis=-3)
+  if w_txt is None or n_txt <= 0:
+    dx, dw = rmsnorm_bwd(x, w, g, eps, dtype)
+    return dx, dw, None
+  dx = np.empty(np.shape(x), dtype)
+  dx[:, :n_txt], dw_txt = rmsnorm_bwd(x[:, :n_txt], w_txt, g[:, :n_txt], eps, dtype)
+  dx[:, n_txt:], dw = rmsnorm_bwd(x[:, n_txt:], w, g[:, n_txt:], eps, dtype)
+  return dx, dw, dw_txt
+
+
+def norm_rope_ltx2_bwd(x, w, cos, sin, mode: str, g, eps: float = 1e-6, dtype=np.float64):
+  """VJP of `norm_rope_ltx2`: x, g [B,S,H*D] -> (dx, dw).  The tables are full-size and need not hold equal values for
+  the two members of a pair, so the transposed rotation is written out, not taken as the rotation by -angle."""
+  g = np.asarray(g, dtype)
+  if mode == "interleaved":
+    c, sn = np.asarray(cos, dtype), np.asarray(sin, dtype)
+    gs = (g * sn).reshape(*g.shape[:-1], -1, 2)
+    # out[2j] = y[2j] c[2j] - y[2j+1] s[2j];  out[2j+1] = y[2j+1] c[2j+1] + y[2j] s[2j+1]
+    g = g * c + np.stack([gs[..., 1], -gs[..., 0]], axis=-1).reshape(g.shape)
+  elif mode == "split":
+    c, sn = np.asarray(cos, dtype), np.asarray(sin, dtype)
+    b, s, n = g.shape
+    h, r = c.shape[1], c.shape[3]
+    gh = g.reshape(b, s, h, 2, r).transpose(0, 2, 1, 3, 4)
+    g1, g2 = gh[..., 0, :], gh[..., 1, :]
+    g = np.stack([g1 * c + g2 * sn, g2 * c - g1 * sn], axis=-2).transpose(0, 2, 1, 3, 4).reshape(b, s, n)
+  elif mode != "none":
+    raise ValueError(mode)
+  return rmsnorm_bwd(x, w, g, eps, dtype)
 
 
 # --------------------------------------------------------------------------- A6 merges

@@ -560,6 +560,104 @@ def test_attention_bwd_matches_torch_autograd_and_finite_differences():
   assert all(not g.any() for g in O.attention_bwd(q, k, v, do, scale, kv_mask=np.zeros(Skv, bool)))
 
 
+def _torch_rope_complex(y, cos, sin):
+  """Rotation of interleaved pairs as a complex multiply (torch): y [B,S,H,D] f64, cos/sin [S,D/2]."""
+  yc = torch.view_as_complex(y.reshape(*y.shape[:-1], -1, 2))
+  rot = torch.complex(torch.tensor(cos, dtype=torch.float64), torch.tensor(sin, dtype=torch.float64))[None, :, None, :]
+  return torch.view_as_real(yc * rot).reshape(y.shape)
+
+
+def test_prologue_bwd_matches_torch_autograd_and_finite_differences():
+  """norm_rope_fullrow_bwd / _perhead_bwd / rmsnorm_bwd against torch autograd (f64) through the library's rms_norm and
+  a complex-multiply rotation; a directional finite difference of the forward oracle; closed-form facts."""
+  rng = np.random.default_rng(41)
+  B, H, D, grid = 2, 3, 16, (2, 2, 3)
+  S, n = 12, 3 * 16
+  cos, sin = O.wan_rope_table(grid, D)
+  x, g = rng.standard_normal((B, S, n)), rng.standard_normal((B, S, H, D))
+  w, bias = 1 + 0.1 * rng.standard_normal(n), 0.3 * rng.standard_normal(n)
+  for use_rope, q_mul, use_bias in ((True, 1.0, False), (False, 1.0, False), (True, 0.1275, True)):
+    c_, s_ = (cos, sin) if use_rope else (None, None)
+    b_ = bias if use_bias else None
+    dx, dw = O.norm_rope_fullrow_bwd(x, w, c_, s_, H, g, q_mul=q_mul, bias=b_)
+    tx, tw, tb_ = (torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (x, w, bias))
+    y = torch.nn.functional.rms_norm(tx + (tb_ if use_bias else 0.0), (n,), tw, eps=1e-6).reshape(B, S, H, D)
+    if use_rope:
+      y = _torch_rope_complex(y, cos, sin)
+    (y * q_mul * torch.tensor(g)).sum().backward()
+    np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-9, atol=1e-12)
+    np.testing.assert_allclose(dw, tw.grad.numpy(), rtol=1e-9, atol=1e-12)
+    if use_bias:
+      np.testing.assert_allclose(dx.reshape(-1, n).sum(0), tb_.grad.numpy(), rtol=1e-9, atol=1e-12)
+    # finite differences of the forward oracle along random directions of x and w
+    f = lambda xx, ww: float((O.norm_rope_fullrow(xx + (0.0 if b_ is None else b_), ww, c_, s_, H) * q_mul * g).sum())
+    e = 1e-6
+    dxd, dwd = rng.standard_normal(x.shape), rng.standard_normal(w.shape)
+    fd = (f(x + e * dxd, w) - f(x - e * dxd, w)) / (2 * e)
+    assert abs(fd - float((dx * dxd).sum())) <= 1e-6 * max(1.0, abs(fd))
+    fd = (f(x, w + e * dwd) - f(x, w - e * dwd)) / (2 * e)
+    assert abs(fd - float((dw * dwd).sum())) <= 1e-6 * max(1.0, abs(fd))
+  # the norm is scale-invariant when eps = 0: the input gradient has no component along the input row
+  dx0, _ = O.rmsnorm_bwd(x, w, g.reshape(B, S, n), eps=0.0)
+  assert np.abs((dx0 * x).sum(-1)).max() <= 1e-12
+  # rotation-only chain (unit weights, a row of unit RMS kept fixed by projecting the gradient): d(rope)/dy is the
+  # rotation by the opposite angle
+  back = O.apply_rope_interleaved(O.apply_rope_interleaved(g, cos, sin), cos, -sin)
+  np.testing.assert_allclose(back, g, rtol=1e-6, atol=1e-6)  # f32 tables: unit modulus to f32 round-off
+
+  # per-head flavour with separate text-token weights
+  ids = O.flux_ids(3, 2, 3)
+  L = ids.shape[0]
+  cos, sin = O.flux_rope_table(ids, axes_dim=(4, 6, 6))
+  x, g = rng.standard_normal((B, L, H, D)), rng.standard_normal((B, L, H, D))
+  w, wt = 1 + 0.1 * rng.standard_normal(D), 1 + 0.1 * rng.standard_normal(D)
+  dx, dw, dwt = O.norm_rope_perhead_bwd(x, w, cos, sin, g, q_mul=0.5, w_txt=wt, n_txt=3)
+  tx, tw, twt = (torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (x, w, wt))
+  y = torch.cat([torch.nn.functional.rms_norm(tx[:, :3], (D,), twt, eps=1e-6), torch.nn.functional.rms_norm(tx[:, 3:], (D,), tw, eps=1e-6)], dim=1)
+  (_torch_rope_complex(y, cos, sin) * 0.5 * torch.tensor(g)).sum().backward()
+  np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-9, atol=1e-12)
+  np.testing.assert_allclose(dw, tw.grad.numpy(), rtol=1e-9, atol=1e-12)
+  np.testing.assert_allclose(dwt, twt.grad.numpy(), rtol=1e-9, atol=1e-12)
+  dx1, dw1, none = O.norm_rope_perhead_bwd(x, w, cos, sin, g)
+  tx, tw = (torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (x, w))
+  (_torch_rope_complex(torch.nn.functional.rms_norm(tx, (D,), tw, eps=1e-6), cos, sin) * torch.tensor(g)).sum().backward()
+  assert none is None
+  np.testing.assert_allclose(dx1, tx.grad.numpy(), rtol=1e-9, atol=1e-12)
+  np.testing.assert_allclose(dw1, tw.grad.numpy(), rtol=1e-9, atol=1e-12)
+
+
+def test_ltx2_prologue_bwd_matches_torch_autograd():
+  """norm_rope_ltx2_bwd against torch autograd through rms_norm and the two LTX-2 rotations written with torch index
+  arithmetic (attention_ltx2.py:33-102), with tables whose pair members differ (the general case the kernel handles)."""
+  rng = np.random.default_rng(42)
+  B, S, H, D = 2, 5, 3, 16
+  n = H * D
+  x, g = rng.standard_normal((B, S, n)), rng.standard_normal((B, S, n))
+  w = 1 + 0.1 * rng.standard_normal(n)
+  cos_i, sin_i = rng.standard_normal((B, S, n)), rng.standard_normal((B, S, n))
+  cos_s, sin_s = rng.standard_normal((B, H, S, D // 2)), rng.standard_normal((B, H, S, D // 2))
+  for mode, c_, s_ in (("none", None, None), ("interleaved", cos_i, sin_i), ("split", cos_s, sin_s)):
+    dx, dw = O.norm_rope_ltx2_bwd(x, w, c_, s_, mode, g)
+    tx, tw = (torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (x, w))
+    y = torch.nn.functional.rms_norm(tx, (n,), tw, eps=1e-6)
+    if mode == "interleaved":
+      yr = y.reshape(B, S, n // 2, 2)
+      rot = torch.stack([-yr[..., 1], yr[..., 0]], dim=-1).reshape(B, S, n)
+      y = y * torch.tensor(c_) + rot * torch.tensor(s_)
+    elif mode == "split":
+      yh = y.reshape(B, S, H, 2, D // 2).permute(0, 2, 1, 3, 4)
+      a1, a2 = yh[..., 0, :], yh[..., 1, :]
+      c, sn = torch.tensor(c_), torch.tensor(s_)
+      y = torch.stack([a1 * c - a2 * sn, a2 * c + a1 * sn], dim=-2).permute(0, 2, 1, 3, 4).reshape(B, S, n)
+    (y * torch.tensor(g)).sum().backward()
+    np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-9, atol=1e-12)
+    np.testing.assert_allclose(dw, tw.grad.numpy(), rtol=1e-9, atol=1e-12)
+    f = lambda xx: float((O.norm_rope_ltx2(xx, w, c_, s_, mode) * g).sum())
+    d = rng.standard_normal(x.shape)
+    fd = (f(x + 1e-6 * d) - f(x - 1e-6 * d)) / 2e-6
+    assert abs(fd - float((dx * d).sum())) <= 1e-6 * max(1.0, abs(fd))
+
+
 # ----------------------------------------------------------------------------- fp8 emulation
 def test_fp8_emulation_meets_cosine_bar():
   q = O.normal_bf16((2, 128, 128), 0)
