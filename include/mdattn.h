@@ -145,6 +145,68 @@ int mdattn_norm_rope_rows(void* stream, const void* x_in, int x_is_f32, void* x_
                           int64_t in_stride_batch, int64_t in_stride_seq, const mdattn_strides* out_strides);
 
 /*
+ * Backward of the fused prologues: input gradients and weight gradients from the saved inputs and the upstream
+ * gradients of the prologue's outputs (what the attention backward returns as dq, dk).  Replaces: JAX autodiff through
+ * norm_q / norm_k and _apply_rope (models/attention_flax.py:2655-2677, :2596-2620; Flux :2989-3020; LTX-2
+ * models/ltx2/attention_ltx2.py:556-585) -- the reference has no hand-written backward here, the trainer
+ * differentiates straight through these lines (trainers/wan_trainer.py:169).
+ *   forward  u = x (+ bias);  r = rsqrt(mean(u^2) + eps);  y = u r w;  out = q_mul * R(y)
+ *   backward dy = q_mul * R^T g;  du = r (w dy) - u r^3 mean(u w dy);  dw = sum over tokens of dy u r
+ * The row statistics are recomputed from the saved input; statistics, rotation and VJP in f32, ONE rounding of du to
+ * the input's dtype; dw in f32.  dw is reduced over tokens without atomics in two stages through `workspace` (every
+ * workgroup writes one partial row, a second kernel adds the rows in a fixed order: bit-reproducible).
+ *   workspace    f32 device scratch, 16-byte aligned; mdattn_norm_rope_bwd_workspace_floats(rows, columns) floats
+ *                give the kernels their full grid (1024 partial rows); a smaller one (>= columns floats) is accepted
+ *                and lowers the number of workgroups.  rows / columns: B*S and 2*H*D (one tensor: H*D; with bias
+ *                twice that) for the full-row form; B*S*H and 4*D for the per-head form; B*S and H*D for the rows form.
+ */
+int64_t mdattn_norm_rope_bwd_workspace_floats(int64_t rows, int64_t columns);
+
+/*
+ * Backward of mdattn_norm_rope_fullrow and, with `bias`, of mdattn_norm_rope_qkv's q and k blocks (its v block is a
+ * copy: dv is the attention backward's dv, summed over tokens for the v bias by the caller).
+ *   q_in, k_in   the saved inputs, bf16 rows of H*D by (in_stride_batch, in_stride_seq); k_in may be NULL, and then
+ *                gk, dk_in, wk, dwk are NULL too
+ *   bias         bf16 [2*H*D] (q | k blocks of the projection biases the forward added) or NULL; needs k_in
+ *   gq, gk       bf16 [B,S,H,D] by g_strides: gradients of q_out, k_out
+ *   dq_in, dk_in bf16 rows of H*D by (dx_stride_batch, dx_stride_seq): gradients of the inputs (with dx strides of
+ *                3*H*D and dk_in = dq_in + H*D they are the q | k blocks of a fused gradient buffer)
+ *   dwq, dwk     f32 [H*D];  dbias f32 [2*H*D] (with bias; = column sums of dq_in | dk_in) or NULL
+ *   wq, wk, cos, sin, eps, q_mul as given to the forward.  Requires D % 8 == 0, H*D <= 8192.
+ */
+int mdattn_norm_rope_fullrow_bwd(void* stream, const void* q_in, const void* k_in, const void* bias,
+                                 const void* gq, const void* gk, void* dq_in, void* dk_in,
+                                 const void* wq, const void* wk, float* dwq, float* dwk, float* dbias,
+                                 const float* cos, const float* sin, int B, int S, int H, int D, float eps, float q_mul,
+                                 int64_t in_stride_batch, int64_t in_stride_seq,
+                                 int64_t dx_stride_batch, int64_t dx_stride_seq, const mdattn_strides* g_strides,
+                                 float* workspace, int64_t workspace_floats);
+
+/*
+ * Backward of mdattn_norm_rope_perhead.  q_in, k_in bf16 [B,S,H,D] by in_strides (k_in may be NULL with gk, dk_in,
+ * wk, dwk); gq, gk by g_strides; dq_in, dk_in by dx_strides; dwq, dwk f32 [D]: weight gradients over the tokens that
+ * used wq / wk; dwq_txt, dwk_txt f32 [D] (given exactly when wq_txt / wk_txt are): over the tokens [0, n_txt).
+ */
+int mdattn_norm_rope_perhead_bwd(void* stream, const void* q_in, const void* k_in, const void* gq, const void* gk,
+                                 void* dq_in, void* dk_in, const void* wq, const void* wk, const void* wq_txt,
+                                 const void* wk_txt, int n_txt, float* dwq, float* dwk, float* dwq_txt, float* dwk_txt,
+                                 const float* cos, const float* sin, int B, int S, int H, int D, float eps, float q_mul,
+                                 const mdattn_strides* in_strides, const mdattn_strides* dx_strides,
+                                 const mdattn_strides* g_strides, float* workspace, int64_t workspace_floats);
+
+/*
+ * Backward of mdattn_norm_rope_rows (LTX-2): x_in [B,S,H*D] bf16 or f32 as given to the forward, g bf16 [B,S,H,D] by
+ * g_strides, dx in x_in's dtype by (dx_stride_batch, dx_stride_seq), dw f32 [H*D]; tables and rope_mode as for the
+ * forward (the two members of a pair may carry different table values: the transposed rotation is applied as written,
+ * not as the rotation by the opposite angle).
+ */
+int mdattn_norm_rope_rows_bwd(void* stream, const void* x_in, int x_is_f32, const void* g, void* dx, const float* w,
+                              float* dw, const float* cos, const float* sin, int rope_mode, int B, int S, int H, int D,
+                              float eps, int64_t in_stride_batch, int64_t in_stride_seq,
+                              int64_t dx_stride_batch, int64_t dx_stride_seq, const mdattn_strides* g_strides,
+                              float* workspace, int64_t workspace_floats);
+
+/*
  * Non-causal softmax attention forward, bf16 MFMA, online softmax in f32, optional LSE.
  * Replaces: the kernel a KERNEL_REGISTRY entry dispatches to (models/attention_flax.py:1589-1597,
  * :1965-1966), i.e. what _tpu_flash_attention (:563-809) / kernels/custom_splash_attention.py:69-320

@@ -106,6 +106,37 @@ int mdattn_xla_norm_rope_rows(void* stream, const mdattn_buffer* x, const mdattn
                               const mdattn_buffer* sin, const mdattn_buffer* x_out, float eps, int64_t heads,
                               int64_t mode, char* err, int err_len);
 
+/* "mdattn_norm_rope_fullrow_bwd": (q, k bf16 [B,S,H*D], gq, gk bf16 [B,S,H,D], wq, wk bf16 [H*D], cos, sin f32 [S,D/2],
+ * bias bf16 [2*H*D]) -> (dq, dk bf16 [B,S,H*D], dwq, dwk f32 [H*D], dbias f32 [2*H*D], workspace f32 [>= columns]).
+ * rope == 0: cos / sin ignored; has_k == 0: k, gk, wk, dk, dwk ignored; has_bias == 0: bias and dbias ignored.  XLA
+ * allocates the scratch of the two-stage weight-gradient reduction as the last result
+ * (mdattn_norm_rope_bwd_workspace_floats(B*S, columns) floats; columns = H*D x (2 with k) x (2 with bias)). */
+int mdattn_xla_norm_rope_fullrow_bwd(void* stream, const mdattn_buffer* q, const mdattn_buffer* k, const mdattn_buffer* gq,
+                                     const mdattn_buffer* gk, const mdattn_buffer* wq, const mdattn_buffer* wk,
+                                     const mdattn_buffer* cos, const mdattn_buffer* sin, const mdattn_buffer* bias,
+                                     const mdattn_buffer* dq, const mdattn_buffer* dk, const mdattn_buffer* dwq,
+                                     const mdattn_buffer* dwk, const mdattn_buffer* dbias, const mdattn_buffer* workspace,
+                                     float eps, float q_mul, int64_t heads, int64_t rope, int64_t has_k, int64_t has_bias,
+                                     char* err, int err_len);
+
+/* "mdattn_norm_rope_perhead_bwd": (q, k, gq, gk bf16 [B,S,H,D], wq, wk, wq_txt, wk_txt bf16 [D], cos, sin f32 [S,D/2]) ->
+ * (dq, dk bf16 [B,S,H,D], dwq, dwk, dwq_txt, dwk_txt f32 [D], workspace f32 [>= 4*D]).  n_txt == 0: the text weights and
+ * their gradients are ignored; has_k == 0: everything of k is ignored. */
+int mdattn_xla_norm_rope_perhead_bwd(void* stream, const mdattn_buffer* q, const mdattn_buffer* k, const mdattn_buffer* gq,
+                                     const mdattn_buffer* gk, const mdattn_buffer* wq, const mdattn_buffer* wk,
+                                     const mdattn_buffer* wq_txt, const mdattn_buffer* wk_txt, const mdattn_buffer* cos,
+                                     const mdattn_buffer* sin, const mdattn_buffer* dq, const mdattn_buffer* dk,
+                                     const mdattn_buffer* dwq, const mdattn_buffer* dwk, const mdattn_buffer* dwq_txt,
+                                     const mdattn_buffer* dwk_txt, const mdattn_buffer* workspace, float eps, float q_mul,
+                                     int64_t n_txt, int64_t rope, int64_t has_k, char* err, int err_len);
+
+/* "mdattn_norm_rope_rows_bwd": (x bf16|f32 [B,S,H*D], g bf16 [B,S,H,D], w f32 [H*D], cos, sin f32) -> (dx in x's dtype
+ * [B,S,H*D], dw f32 [H*D], workspace f32 [>= H*D]); mode as for mdattn_norm_rope_rows */
+int mdattn_xla_norm_rope_rows_bwd(void* stream, const mdattn_buffer* x, const mdattn_buffer* g, const mdattn_buffer* w,
+                                  const mdattn_buffer* cos, const mdattn_buffer* sin, const mdattn_buffer* dx,
+                                  const mdattn_buffer* dw, const mdattn_buffer* workspace, float eps, int64_t heads,
+                                  int64_t mode, char* err, int err_len);
+
 /* "mdattn_quant_e4m3": (x bf16, any shape) -> (x8 u8|f8e4m3fn same shape, scale f32 [2]) */
 int mdattn_xla_quant_e4m3(void* stream, const mdattn_buffer* x, const mdattn_buffer* x8, const mdattn_buffer* scale_out,
                           float premul, int64_t pow2_scale, char* err, int err_len);

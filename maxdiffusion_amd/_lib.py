@@ -39,6 +39,10 @@ SIGNATURES = {
     "mdattn_norm_rope_qkv": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _L, _L, _S], _I),
     "mdattn_norm_rope_perhead": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _F, _F, _S, _S], _I),
     "mdattn_norm_rope_rows": ([_P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _L, _L, _S], _I),
+    "mdattn_norm_rope_bwd_workspace_floats": ([_L, _L], _L),
+    "mdattn_norm_rope_fullrow_bwd": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _L, _L, _L, _L, _S, _P, _L], _I),
+    "mdattn_norm_rope_perhead_bwd": ([_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _S, _S, _S, _P, _L], _I),
+    "mdattn_norm_rope_rows_bwd": ([_P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _L, _L, _L, _L, _S, _P, _L], _I),
     "mdattn_fwd_bf16": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F], _I),
     "mdattn_fwd_bf16_bias": ([_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _S, _S, _S, _S, _F, _P, _L], _I),
     "mdattn_key_mask_bias": ([_P, _P, _P, _I, _I, _L, _F], _I),

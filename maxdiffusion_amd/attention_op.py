@@ -88,24 +88,62 @@ def _mask_bias(context, qv, kv):
   return ops.key_mask_bias(mask)
 
 
+def _dense(t: torch.Tensor) -> torch.Tensor:
+  """A view whose memory is dense in some axis order (the backward kernels write gradients with the operand's strides)."""
+  return t if t.is_contiguous() or t.permute(0, 2, 1, 3).is_contiguous() else t.contiguous()
+
+
+class _HipFlashAttention(torch.autograd.Function):
+  """Forward + backward through the HIP kernels: the registry entry carries its own VJP, as the reference's kernels do
+  (kernels/splash_attention/splash_attention_kernel.py:1166, :2067 define the custom_vjp the trainer differentiates
+  through, trainers/wan_trainer.py:169).  Saved for the backward: q, k, v, out, lse -- the residuals the reference
+  tags with `residual_checkpoint_name` for its remat policies; torch's checkpointing re-runs the forward instead, so
+  the name is carried in the context and not used here."""
+
+  @staticmethod
+  def forward(ctx, q, k, v, scale, key_bias):
+    out, lse = ops.flash_attention(q, k, v, scale=scale, return_lse=True, key_bias=key_bias)
+    ctx.save_for_backward(q, k, v, out, lse)
+    ctx.scale, ctx.key_bias = scale, key_bias
+    return out
+
+  @staticmethod
+  def backward(ctx, dout):
+    q, k, v, out, lse = ctx.saved_tensors
+    dq, dk, dv = ops.flash_attention_backward(q, k, v, out, dout.to(torch.bfloat16), lse, scale=ctx.scale, key_bias=ctx.key_bias)
+    return dq, dk, dv, None, None
+
+
+def hip_flash_attention_autograd(q, k, v, scale: float, key_bias=None):
+  """Differentiable attention on bf16 logical [B,S,H,D] views (torch autograd); key_bias as for ops.flash_attention."""
+  return _HipFlashAttention.apply(_dense(q), _dense(k), _dense(v), float(scale), key_bias)
+
+
 @register_kernel("hip_flash")
 def hip_flash_kernel(q, k, v, context):
   """KERNEL_REGISTRY entry: fn(q, k, v, context) -> [B, Sq, H*D] in q's dtype.
 
   Unlike the reference's flash entries, which pass k * scale (attention_flax.py:1783), the scale goes
   to the kernel and is folded into the exp2 argument; `flash_block_sizes`, `mesh` and the axis names
-  are accepted and ignored (one GPU, tiles fixed by the kernel).
+  are accepted and ignored (one GPU, tiles fixed by the kernel).  Differentiable: when autograd is recording and an
+  input requires a gradient, the call goes through `_HipFlashAttention` (forward with lse, HIP backward), in both
+  input layouts and with a key mask.
   """
   _reject_unsupported(context)
   heads = context["heads"]
   qv, kv, vv = _as_bshd(q, heads), _as_bshd(k, heads), _as_bshd(v, heads)
+  # LTX2 hands f32 q/k next to a v in the model dtype (norm dtype f32, attention_ltx2.py:415-432); the MFMA operands are
+  # bf16.  Each such cast is one more pass over the tensor in HBM: `hip_norm_rope_ltx2` in front of this entry emits
+  # bf16 q/k straight from the prologue kernel and leaves nothing to cast.
   cast = q.dtype != torch.bfloat16
-  if cast:  # LTX2 hands f32 q/k (attention_ltx2.py:415-432); the MFMA operands are bf16
-    qv, kv, vv = qv.to(torch.bfloat16), kv.to(torch.bfloat16), vv.to(torch.bfloat16)
+  qv, kv, vv = (t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16) for t in (qv, kv, vv))
   # [B,Skv] keep-mask (attention_flax.py:1926-1939): masked keys are excluded, as the flash wrappers do with
   # segment ids (:390-438); rows without a kept key return 0 (:1552-1554)
   bias = _mask_bias(context, qv, kv)
-  out = ops.flash_attention(qv, kv, vv, scale=context["scale"], key_bias=bias)
+  if torch.is_grad_enabled() and (qv.requires_grad or kv.requires_grad or vv.requires_grad):
+    out = hip_flash_attention_autograd(qv, kv, vv, context["scale"], bias)
+  else:
+    out = ops.flash_attention(qv, kv, vv, scale=context["scale"], key_bias=bias)
   b, s, h, d = out.shape
   out = out.reshape(b, s, h * d)
   return out.to(q.dtype) if cast else out
@@ -131,6 +169,74 @@ def hip_flash_fp8_kernel(q, k, v, context):
 
 
 
+def _wants_grad(*ts) -> bool:
+  return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in ts)
+
+
+class _HipNormRopeFullrow(torch.autograd.Function):
+  """The Wan prologue with its HIP backward: saved for the backward are the inputs only (the row statistics are
+  recomputed); the reference differentiates through these lines by JAX autodiff (attention_flax.py:2655-2677)."""
+
+  @staticmethod
+  def forward(ctx, q, k, wq, wk, cos, sin, heads, eps, out_layout, q_mul):
+    q_out, k_out = ops.norm_rope_fullrow(q, k, wq, wk, cos, sin, heads, eps, out_layout, q_mul)
+    ctx.save_for_backward(q, k, wq, wk, cos, sin)
+    ctx.cfg = (heads, eps, q_mul)
+    return q_out, k_out
+
+  @staticmethod
+  def backward(ctx, gq, gk):
+    q, k, wq, wk, cos, sin = ctx.saved_tensors
+    heads, eps, q_mul = ctx.cfg
+    dq, dk, dwq, dwk = ops.norm_rope_fullrow_backward(q, k, wq, wk, cos, sin, heads, gq.to(torch.bfloat16),
+                                                      gk.to(torch.bfloat16) if k is not None else None, eps, q_mul)
+    return dq, dk, dwq.to(wq.dtype), (dwk.to(wk.dtype) if k is not None else None), None, None, None, None, None, None
+
+
+class _HipNormRopePerhead(torch.autograd.Function):
+  """The Flux prologue with its HIP backward (attention_flax.py:2989-3020)."""
+
+  @staticmethod
+  def forward(ctx, q, k, wq, wk, wq_txt, wk_txt, cos, sin, eps, n_txt, out_layout, q_mul):
+    q_out, k_out = ops.norm_rope_perhead(q, k, wq, wk, cos, sin, eps, wq_txt, wk_txt, n_txt, out_layout, q_mul)
+    ctx.save_for_backward(q, k, wq, wk, wq_txt, wk_txt, cos, sin)
+    ctx.cfg = (eps, n_txt, q_mul)
+    return q_out, k_out
+
+  @staticmethod
+  def backward(ctx, gq, gk):
+    q, k, wq, wk, wq_txt, wk_txt, cos, sin = ctx.saved_tensors
+    eps, n_txt, q_mul = ctx.cfg
+    dq, dk, dwq, dwk, dwq_t, dwk_t = ops.norm_rope_perhead_backward(
+        q, k, wq, wk, cos, sin, gq.to(torch.bfloat16), gk.to(torch.bfloat16) if k is not None else None, eps, wq_txt, wk_txt, n_txt, q_mul)
+    cast = lambda g, w: None if g is None else g.to(w.dtype)
+    return dq, dk, cast(dwq, wq), cast(dwk, wk), cast(dwq_t, wq_txt), cast(dwk_t, wk_txt), None, None, None, None, None, None
+
+
+class _HipNormRopeRows(torch.autograd.Function):
+  """The LTX-2 prologue of one tensor with its HIP backward (models/ltx2/attention_ltx2.py:556-585)."""
+
+  @staticmethod
+  def forward(ctx, x, w, cos, sin, heads, mode, eps):
+    out = ops.norm_rope_rows(x, w, cos, sin, heads=heads, mode=mode, eps=eps)
+    ctx.save_for_backward(x, w, cos, sin)
+    ctx.cfg = (heads, mode, eps)
+    return out
+
+  @staticmethod
+  def backward(ctx, g):
+    x, w, cos, sin = ctx.saved_tensors
+    heads, mode, eps = ctx.cfg
+    dx, dw = ops.norm_rope_rows_backward(x, w, g.to(torch.bfloat16), cos, sin, heads=heads, mode=mode, eps=eps)
+    return dx, dw, None, None, None, None, None
+
+
+def _norm_rope_rows(x, w, cos, sin, heads, mode, eps):
+  if _wants_grad(x, w):
+    return _HipNormRopeRows.apply(x, w, cos, sin, heads, mode, eps)
+  return ops.norm_rope_rows(x, w, cos, sin, heads=heads, mode=mode, eps=eps)
+
+
 def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotary_emb=None, k_rotary_emb=None,
                        rope_type: str = "interleaved", is_self_attention: bool = True, eps: float = 1e-6,
                        q_mul: float = 1.0):
@@ -150,37 +256,14 @@ def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotar
 
   def run(x, scale, tab):
     if tab is None:
-      return ops.norm_rope_rows(x, scale, heads=heads, mode="none", eps=eps)
+      return _norm_rope_rows(x, scale, None, None, heads, "none", eps)
     cos, sin = (t.to(torch.float32).contiguous() for t in tab)
-    return ops.norm_rope_rows(x, scale, cos, sin, heads=heads, mode=rope_type, eps=eps)
+    return _norm_rope_rows(x, scale, cos, sin, heads, rope_type, eps)
 
   q = run(query, norm_q_scale if q_mul == 1.0 else norm_q_scale * q_mul, q_tab)
   k = run(key, norm_k_scale, k_tab) if key is not None else None
   return q, k
 
-
-
-class _HipFlashAttention(torch.autograd.Function):
-  """Forward + backward through the HIP kernels: what a trainer's custom_vjp around the attention kernel does in
-  the reference (kernels/splash_attention/splash_attention_kernel.py:1277-1600)."""
-
-  @staticmethod
-  def forward(ctx, q, k, v, scale):
-    out, lse = ops.flash_attention(q, k, v, scale=scale, return_lse=True)
-    ctx.save_for_backward(q, k, v, out, lse)
-    ctx.scale = scale
-    return out
-
-  @staticmethod
-  def backward(ctx, dout):
-    q, k, v, out, lse = ctx.saved_tensors
-    dq, dk, dv = ops.flash_attention_backward(q, k, v, out, dout.contiguous(), lse, scale=ctx.scale)
-    return dq, dk, dv, None
-
-
-def hip_flash_attention_autograd(q, k, v, scale: float):
-  """Differentiable attention on dense bf16 [B,S,H,D] tensors (torch autograd)."""
-  return _HipFlashAttention.apply(q, k, v, float(scale))
 
 
 def _apply_attention(
@@ -365,7 +448,8 @@ def hip_norm_rope(q, k, wq, wk, freqs_cis, heads: int, eps: float = 1e-6, per_he
   per_head=False: FlaxWanAttention.__call__ lines attention_flax.py:2655-2677 (q, k are [B,S,H*D]).
   per_head=True : FlaxFluxAttention.__call__ lines :2989-3020 (q, k are [B,S,H,D] views).
   freqs_cis=None is the norm-only mode of the cross-attention (:2671).  Returns logical [B,S,H,D]
-  views laid out as `out_layout`, ready for `hip_flash` with no transpose in between.
+  views laid out as `out_layout`, ready for `hip_flash` with no transpose in between.  Differentiable with respect to
+  q, k and the norm weights (torch autograd through the HIP backward kernels), so a trainer can keep the hook.
   `q_mul` is multiplied into the query before its single rounding: with q_mul=ops.folded_q_mul(D) and
   context["scale"]=ops.FOLDED_SCALE the softmax scale is carried by the prologue, where the reference carries it by
   two bf16 multiplies of k and q (:1783, :610), and the attention kernel saves its multiply per logit.
@@ -373,7 +457,11 @@ def hip_norm_rope(q, k, wq, wk, freqs_cis, heads: int, eps: float = 1e-6, per_he
   if per_head:
     b, s, h, d = q.shape
     cos, sin = _split_table(freqs_cis, s, d)
+    if _wants_grad(q, k, wq, wk, wq_txt, wk_txt):
+      return _HipNormRopePerhead.apply(q, k, wq, wk, wq_txt, wk_txt, cos, sin, eps, n_txt, out_layout, q_mul)
     return ops.norm_rope_perhead(q, k, wq, wk, cos, sin, eps, wq_txt, wk_txt, n_txt, out_layout, q_mul)
   b, s, n = q.shape
   cos, sin = _split_table(freqs_cis, s, n // heads)
+  if _wants_grad(q, k, wq, wk):
+    return _HipNormRopeFullrow.apply(q, k, wq, wk, cos, sin, heads, eps, out_layout, q_mul)
   return ops.norm_rope_fullrow(q, k, wq, wk, cos, sin, heads, eps, out_layout, q_mul)

@@ -42,7 +42,17 @@ mdattn_buffer Out(Res& r) {
 }
 struct Msg {
   char text[512] = {0};
-  ffi::Error done(int rc) const { return rc == MDATTN_OK ? ffi::Error::Success() : ffi::Error::InvalidArgument(std::string(text)); }
+  // argument errors stay InvalidArgument; a launch the runtime rejected, a request no kernel is built for and a request
+  // beyond the static scratch are not the caller's arguments being wrong, and say so
+  ffi::Error done(int rc) const {
+    switch (rc) {
+      case MDATTN_OK: return ffi::Error::Success();
+      case MDATTN_E_LAUNCH: return ffi::Error::Internal(std::string(text));
+      case MDATTN_E_UNSUPPORTED: return ffi::Error(ffi::ErrorCode::kUnimplemented, std::string(text));
+      case MDATTN_E_TOOBIG: return ffi::Error(ffi::ErrorCode::kResourceExhausted, std::string(text));
+      default: return ffi::Error::InvalidArgument(std::string(text));
+    }
+  }
 };
 
 ffi::Error FwdBf16(hipStream_t s, Buf q, Buf k, Buf v, Res out, Res lse, float scale, int64_t layout) {
@@ -102,6 +112,31 @@ ffi::Error NormRopeRows(hipStream_t s, Buf x, Buf w, Buf cos, Buf sin, Res x_out
   Msg m;
   const mdattn_buffer a = In(x), b = In(w), c = In(cos), d = In(sin), o = Out(x_out);
   return m.done(mdattn_xla_norm_rope_rows(s, &a, &b, &c, &d, &o, eps, heads, mode, m.text, sizeof m.text));
+}
+ffi::Error NormRopeFullrowBwd(hipStream_t s, Buf q, Buf k, Buf gq, Buf gk, Buf wq, Buf wk, Buf cos, Buf sin, Buf bias, Res dq, Res dk,
+                              Res dwq, Res dwk, Res dbias, Res workspace, float eps, float q_mul, int64_t heads, int64_t rope,
+                              int64_t has_k, int64_t has_bias) {
+  Msg m;
+  const mdattn_buffer a = In(q), b = In(k), c = In(gq), d = In(gk), e = In(wq), f = In(wk), g = In(cos), h = In(sin), i = In(bias),
+                      o0 = Out(dq), o1 = Out(dk), o2 = Out(dwq), o3 = Out(dwk), o4 = Out(dbias), ws = Out(workspace);
+  return m.done(mdattn_xla_norm_rope_fullrow_bwd(s, &a, &b, &c, &d, &e, &f, &g, &h, &i, &o0, &o1, &o2, &o3, &o4, &ws, eps, q_mul, heads, rope,
+                                                 has_k, has_bias, m.text, sizeof m.text));
+}
+ffi::Error NormRopePerheadBwd(hipStream_t s, Buf q, Buf k, Buf gq, Buf gk, Buf wq, Buf wk, Buf wq_txt, Buf wk_txt, Buf cos, Buf sin, Res dq,
+                              Res dk, Res dwq, Res dwk, Res dwq_txt, Res dwk_txt, Res workspace, float eps, float q_mul, int64_t n_txt,
+                              int64_t rope, int64_t has_k) {
+  Msg m;
+  const mdattn_buffer a = In(q), b = In(k), c = In(gq), d = In(gk), e = In(wq), f = In(wk), et = In(wq_txt), ft = In(wk_txt), g = In(cos),
+                      h = In(sin), o0 = Out(dq), o1 = Out(dk), o2 = Out(dwq), o3 = Out(dwk), o4 = Out(dwq_txt), o5 = Out(dwk_txt),
+                      ws = Out(workspace);
+  return m.done(mdattn_xla_norm_rope_perhead_bwd(s, &a, &b, &c, &d, &e, &f, &et, &ft, &g, &h, &o0, &o1, &o2, &o3, &o4, &o5, &ws, eps, q_mul,
+                                                 n_txt, rope, has_k, m.text, sizeof m.text));
+}
+ffi::Error NormRopeRowsBwd(hipStream_t s, Buf x, Buf g, Buf w, Buf cos, Buf sin, Res dx, Res dw, Res workspace, float eps, int64_t heads,
+                           int64_t mode) {
+  Msg m;
+  const mdattn_buffer a = In(x), b = In(g), c = In(w), d = In(cos), e = In(sin), o0 = Out(dx), o1 = Out(dw), ws = Out(workspace);
+  return m.done(mdattn_xla_norm_rope_rows_bwd(s, &a, &b, &c, &d, &e, &o0, &o1, &ws, eps, heads, mode, m.text, sizeof m.text));
 }
 ffi::Error QuantE4m3(hipStream_t s, Buf x, Res x8, Res scale_out, float premul, int64_t pow2_scale) {
   Msg m;
@@ -174,6 +209,19 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopePerhead, NormRopePerhead,
                                   .Attr<int64_t>("has_k"));
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopeRows, NormRopeRows,
                               MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Ret<Buf>()
+                                  .Attr<float>("eps").Attr<int64_t>("heads").Attr<int64_t>("mode"));
+XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopeFullrowBwd, NormRopeFullrowBwd,
+                              MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>()
+                                  .Ret<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>()
+                                  .Attr<float>("eps").Attr<float>("q_mul").Attr<int64_t>("heads").Attr<int64_t>("rope")
+                                  .Attr<int64_t>("has_k").Attr<int64_t>("has_bias"));
+XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopePerheadBwd, NormRopePerheadBwd,
+                              MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>()
+                                  .Arg<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>()
+                                  .Attr<float>("eps").Attr<float>("q_mul").Attr<int64_t>("n_txt").Attr<int64_t>("rope")
+                                  .Attr<int64_t>("has_k"));
+XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnNormRopeRowsBwd, NormRopeRowsBwd,
+                              MDATTN_BIND.Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>()
                                   .Attr<float>("eps").Attr<int64_t>("heads").Attr<int64_t>("mode"));
 XLA_FFI_DEFINE_HANDLER_SYMBOL(MdattnQuantE4m3, QuantE4m3,
                               MDATTN_BIND.Arg<Buf>().Ret<Buf>().Ret<Buf>().Attr<float>("premul").Attr<int64_t>("pow2_scale"));

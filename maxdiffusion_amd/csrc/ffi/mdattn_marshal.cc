@@ -370,6 +370,148 @@ extern "C" int mdattn_xla_norm_rope_rows(void* stream, const mdattn_buffer* x, c
                                       eps, S * N, N, &so));
 }
 
+namespace {
+bool same_dims(const mdattn_buffer* a, const mdattn_buffer* b) {
+  if (a->rank != b->rank) return false;
+  for (int i = 0; i < a->rank; ++i)
+    if (a->dims[i] != b->dims[i]) return false;
+  return true;
+}
+int check_workspace(const Err& e, const mdattn_buffer* ws, int64_t columns) {
+  CHECK_BUF(e, ws, "workspace");
+  CHECK_DT(e, ws, "workspace", MDATTN_DT_F32);
+  if (count(ws) < columns)
+    return e.fail(MDATTN_E_BADARG, "workspace must hold at least %lld floats (one partial row), got %lld", (long long)columns, (long long)count(ws));
+  return MDATTN_OK;
+}
+}  // namespace
+
+extern "C" int mdattn_xla_norm_rope_fullrow_bwd(void* stream, const mdattn_buffer* q, const mdattn_buffer* k, const mdattn_buffer* gq,
+                                                const mdattn_buffer* gk, const mdattn_buffer* wq, const mdattn_buffer* wk,
+                                                const mdattn_buffer* cos, const mdattn_buffer* sin, const mdattn_buffer* bias,
+                                                const mdattn_buffer* dq, const mdattn_buffer* dk, const mdattn_buffer* dwq,
+                                                const mdattn_buffer* dwk, const mdattn_buffer* dbias, const mdattn_buffer* workspace,
+                                                float eps, float q_mul, int64_t heads, int64_t rope, int64_t has_k, int64_t has_bias,
+                                                char* err, int err_len) {
+  const Err e{err, err_len, "mdattn_norm_rope_fullrow_bwd"};
+  CHECK_BUF(e, q, "q");
+  CHECK_DT(e, q, "q", MDATTN_DT_BF16);
+  if (q->rank != 3 || heads <= 0 || q->dims[2] % heads) return e.fail(MDATTN_E_BADARG, "q must be [B,S,H*D] with H = heads = %lld", (long long)heads);
+  const int64_t B = q->dims[0], S = q->dims[1], N = q->dims[2], D = N / heads;
+  if (!fits_int(B) || !fits_int(S) || !fits_int(N)) return e.fail(MDATTN_E_UNSUPPORTED, "dimensions beyond 2^31");
+  if (has_bias && !has_k) return e.fail(MDATTN_E_BADARG, "has_bias needs has_k (the fused q|k|v form carries both tensors)");
+  auto is_bshd = [&](const mdattn_buffer* b) {
+    return b->rank == 4 && b->dims[0] == B && b->dims[1] == S && b->dims[2] == heads && b->dims[3] == D;
+  };
+  auto check_side = [&](const mdattn_buffer* x, const mdattn_buffer* g, const mdattn_buffer* w, const mdattn_buffer* dx,
+                        const mdattn_buffer* dw, const char* nx, const char* ng, const char* nw, const char* ndx, const char* ndw) -> int {
+    CHECK_BUF(e, x, nx); CHECK_DT(e, x, nx, MDATTN_DT_BF16);
+    if (!same_dims(x, q)) return e.fail(MDATTN_E_BADARG, "%s must have q's shape", nx);
+    CHECK_BUF(e, g, ng); CHECK_DT(e, g, ng, MDATTN_DT_BF16);
+    if (!is_bshd(g)) return e.fail(MDATTN_E_BADARG, "%s must be [B,S,H,D] = [%lld,%lld,%lld,%lld]", ng, (long long)B, (long long)S, (long long)heads, (long long)D);
+    TRY(check_vec(e, w, nw, MDATTN_DT_BF16, N));
+    CHECK_BUF(e, dx, ndx); CHECK_DT(e, dx, ndx, MDATTN_DT_BF16);
+    if (!same_dims(dx, q)) return e.fail(MDATTN_E_BADARG, "%s must have q's shape", ndx);
+    TRY(check_vec(e, dw, ndw, MDATTN_DT_F32, N));
+    return MDATTN_OK;
+  };
+  TRY(check_side(q, gq, wq, dq, dwq, "q", "gq", "wq", "dq", "dwq"));
+  if (has_k) TRY(check_side(k, gk, wk, dk, dwk, "k", "gk", "wk", "dk", "dwk"));
+  if (rope) {
+    TRY(check_vec(e, cos, "cos", MDATTN_DT_F32, S * (D / 2)));
+    TRY(check_vec(e, sin, "sin", MDATTN_DT_F32, S * (D / 2)));
+  }
+  if (has_bias) {
+    TRY(check_vec(e, bias, "bias", MDATTN_DT_BF16, 2 * N));
+    TRY(check_vec(e, dbias, "dbias", MDATTN_DT_F32, 2 * N));
+  }
+  TRY(check_workspace(e, workspace, N * (has_k ? 2 : 1) * (has_bias ? 2 : 1)));
+  const mdattn_strides sg{S * N, N, D};
+  return e.from(mdattn_norm_rope_fullrow_bwd(
+      stream, q->data, has_k ? k->data : nullptr, has_bias ? bias->data : nullptr, gq->data, has_k ? gk->data : nullptr, dq->data,
+      has_k ? dk->data : nullptr, wq->data, has_k ? wk->data : nullptr, static_cast<float*>(dwq->data),
+      has_k ? static_cast<float*>(dwk->data) : nullptr, has_bias ? static_cast<float*>(dbias->data) : nullptr,
+      rope ? static_cast<const float*>(cos->data) : nullptr, rope ? static_cast<const float*>(sin->data) : nullptr, (int)B, (int)S,
+      (int)heads, (int)D, eps, q_mul, S * N, N, S * N, N, &sg, static_cast<float*>(workspace->data), count(workspace)));
+}
+
+extern "C" int mdattn_xla_norm_rope_perhead_bwd(void* stream, const mdattn_buffer* q, const mdattn_buffer* k, const mdattn_buffer* gq,
+                                                const mdattn_buffer* gk, const mdattn_buffer* wq, const mdattn_buffer* wk,
+                                                const mdattn_buffer* wq_txt, const mdattn_buffer* wk_txt, const mdattn_buffer* cos,
+                                                const mdattn_buffer* sin, const mdattn_buffer* dq, const mdattn_buffer* dk,
+                                                const mdattn_buffer* dwq, const mdattn_buffer* dwk, const mdattn_buffer* dwq_txt,
+                                                const mdattn_buffer* dwk_txt, const mdattn_buffer* workspace, float eps, float q_mul,
+                                                int64_t n_txt, int64_t rope, int64_t has_k, char* err, int err_len) {
+  const Err e{err, err_len, "mdattn_norm_rope_perhead_bwd"};
+  CHECK_BUF(e, q, "q");
+  CHECK_DT(e, q, "q", MDATTN_DT_BF16);
+  View4 vq;
+  if (!describe(q, 0, &vq)) return e.fail(MDATTN_E_BADARG, "q must be a rank-4 [B,S,H,D] buffer");
+  if (n_txt < 0 || n_txt > vq.S) return e.fail(MDATTN_E_BADARG, "n_txt = %lld is outside [0, S = %lld]", (long long)n_txt, (long long)vq.S);
+  auto check_side = [&](const mdattn_buffer* x, const mdattn_buffer* g, const mdattn_buffer* w, const mdattn_buffer* wt,
+                        const mdattn_buffer* dx, const mdattn_buffer* dw, const mdattn_buffer* dwt, const char* nx, const char* ng,
+                        const char* nw, const char* nwt, const char* ndx, const char* ndw, const char* ndwt) -> int {
+    View4 t;
+    CHECK_BUF(e, x, nx); CHECK_DT(e, x, nx, MDATTN_DT_BF16);
+    if (!same_dims(x, q)) return e.fail(MDATTN_E_BADARG, "%s must have q's shape", nx);
+    TRY(check_out_bshd(e, g, ng, MDATTN_DT_BF16, vq, &t));
+    TRY(check_out_bshd(e, dx, ndx, MDATTN_DT_BF16, vq, &t));
+    TRY(check_vec(e, w, nw, MDATTN_DT_BF16, vq.D));
+    TRY(check_vec(e, dw, ndw, MDATTN_DT_F32, vq.D));
+    if (n_txt > 0) {
+      TRY(check_vec(e, wt, nwt, MDATTN_DT_BF16, vq.D));
+      TRY(check_vec(e, dwt, ndwt, MDATTN_DT_F32, vq.D));
+    }
+    return MDATTN_OK;
+  };
+  TRY(check_side(q, gq, wq, wq_txt, dq, dwq, dwq_txt, "q", "gq", "wq", "wq_txt", "dq", "dwq", "dwq_txt"));
+  if (has_k) TRY(check_side(k, gk, wk, wk_txt, dk, dwk, dwk_txt, "k", "gk", "wk", "wk_txt", "dk", "dwk", "dwk_txt"));
+  if (rope) {
+    TRY(check_vec(e, cos, "cos", MDATTN_DT_F32, vq.S * (vq.D / 2)));
+    TRY(check_vec(e, sin, "sin", MDATTN_DT_F32, vq.S * (vq.D / 2)));
+  }
+  TRY(check_workspace(e, workspace, 4 * vq.D));
+  const bool txt = n_txt > 0;
+  return e.from(mdattn_norm_rope_perhead_bwd(
+      stream, q->data, has_k ? k->data : nullptr, gq->data, has_k ? gk->data : nullptr, dq->data, has_k ? dk->data : nullptr, wq->data,
+      has_k ? wk->data : nullptr, txt ? wq_txt->data : nullptr, (txt && has_k) ? wk_txt->data : nullptr, (int)n_txt,
+      static_cast<float*>(dwq->data), has_k ? static_cast<float*>(dwk->data) : nullptr, txt ? static_cast<float*>(dwq_txt->data) : nullptr,
+      (txt && has_k) ? static_cast<float*>(dwk_txt->data) : nullptr, rope ? static_cast<const float*>(cos->data) : nullptr,
+      rope ? static_cast<const float*>(sin->data) : nullptr, (int)vq.B, (int)vq.S, (int)vq.H, (int)vq.D, eps, q_mul, &vq.st, &vq.st, &vq.st,
+      static_cast<float*>(workspace->data), count(workspace)));
+}
+
+extern "C" int mdattn_xla_norm_rope_rows_bwd(void* stream, const mdattn_buffer* x, const mdattn_buffer* g, const mdattn_buffer* w,
+                                             const mdattn_buffer* cos, const mdattn_buffer* sin, const mdattn_buffer* dx,
+                                             const mdattn_buffer* dw, const mdattn_buffer* workspace, float eps, int64_t heads,
+                                             int64_t mode, char* err, int err_len) {
+  const Err e{err, err_len, "mdattn_norm_rope_rows_bwd"};
+  CHECK_BUF(e, x, "x");
+  if (x->dtype != MDATTN_DT_BF16 && x->dtype != MDATTN_DT_F32) return e.fail(MDATTN_E_BADARG, "x must be bf16 or f32, got %s", dt_name(x->dtype));
+  if (x->rank != 3 || heads <= 0 || x->dims[2] % heads) return e.fail(MDATTN_E_BADARG, "x must be [B,S,H*D] with H = heads = %lld", (long long)heads);
+  if (mode < 0 || mode > 2) return e.fail(MDATTN_E_BADARG, "mode must be 0 (norm only), 1 (interleaved) or 2 (split), got %lld", (long long)mode);
+  const int64_t B = x->dims[0], S = x->dims[1], N = x->dims[2], D = N / heads;
+  if (!fits_int(B) || !fits_int(S) || !fits_int(N)) return e.fail(MDATTN_E_UNSUPPORTED, "dimensions beyond 2^31");
+  CHECK_BUF(e, g, "g");
+  CHECK_DT(e, g, "g", MDATTN_DT_BF16);
+  if (g->rank != 4 || g->dims[0] != B || g->dims[1] != S || g->dims[2] != heads || g->dims[3] != D)
+    return e.fail(MDATTN_E_BADARG, "g must be [B,S,H,D] = [%lld,%lld,%lld,%lld]", (long long)B, (long long)S, (long long)heads, (long long)D);
+  TRY(check_vec(e, w, "w", MDATTN_DT_F32, N));
+  CHECK_BUF(e, dx, "dx");
+  if (dx->dtype != x->dtype || !same_dims(dx, x)) return e.fail(MDATTN_E_BADARG, "dx must have x's dtype and shape");
+  TRY(check_vec(e, dw, "dw", MDATTN_DT_F32, N));
+  if (mode) {
+    TRY(check_vec(e, cos, "cos", MDATTN_DT_F32, mode == 1 ? B * S * N : B * heads * S * (D / 2)));
+    TRY(check_vec(e, sin, "sin", MDATTN_DT_F32, mode == 1 ? B * S * N : B * heads * S * (D / 2)));
+  }
+  TRY(check_workspace(e, workspace, N));
+  const mdattn_strides sg{S * N, N, D};
+  return e.from(mdattn_norm_rope_rows_bwd(stream, x->data, x->dtype == MDATTN_DT_F32, g->data, dx->data, static_cast<const float*>(w->data),
+                                          static_cast<float*>(dw->data), mode ? static_cast<const float*>(cos->data) : nullptr,
+                                          mode ? static_cast<const float*>(sin->data) : nullptr, (int)mode, (int)B, (int)S, (int)heads, (int)D,
+                                          eps, S * N, N, S * N, N, &sg, static_cast<float*>(workspace->data), count(workspace)));
+}
+
 extern "C" int mdattn_xla_quant_e4m3(void* stream, const mdattn_buffer* x, const mdattn_buffer* x8, const mdattn_buffer* scale_out,
                                      float premul, int64_t pow2_scale, char* err, int err_len) {
   const Err e{err, err_len, "mdattn_quant_e4m3"};

@@ -32,6 +32,9 @@ FFI_TARGETS = {
     "mdattn_norm_rope_qkv": "MdattnNormRopeQkv",
     "mdattn_norm_rope_perhead": "MdattnNormRopePerhead",
     "mdattn_norm_rope_rows": "MdattnNormRopeRows",
+    "mdattn_norm_rope_fullrow_bwd": "MdattnNormRopeFullrowBwd",
+    "mdattn_norm_rope_perhead_bwd": "MdattnNormRopePerheadBwd",
+    "mdattn_norm_rope_rows_bwd": "MdattnNormRopeRowsBwd",
     "mdattn_quant_e4m3": "MdattnQuantE4m3",
     "mdattn_fwd_fp8": "MdattnFwdFp8",
     "mdattn_fwd_fp8_bias": "MdattnFwdFp8Bias",
@@ -41,7 +44,10 @@ FFI_TARGETS = {
 }
 # entry points of mdattn.h that are host-side helpers, not kernels: no custom call
 HOST_ONLY = ("mdattn_version", "mdattn_strerror", "mdattn_build_id", "mdattn_set_fwd_schedule",
-             "mdattn_bwd_workspace_floats", "mdattn_bwd_static_max_floats")
+             "mdattn_bwd_workspace_floats", "mdattn_bwd_static_max_floats", "mdattn_norm_rope_bwd_workspace_floats")
+
+BWD_STATIC_MAX_FLOATS = 8 * 1024 * 1024  # MDATTN_BWD_STATIC_MAX_FLOATS of include/mdattn.h
+NORM_ROPE_BWD_MAX_PARTIAL_ROWS = 1024    # mdattn_norm_rope_bwd_workspace_floats(rows, columns) = min(rows, 1024) * columns
 
 FOLDED_SCALE = math.log(2.0)  # see ops.FOLDED_SCALE: scale * log2(e) == 1, the softmax scale rides on q
 
@@ -182,21 +188,36 @@ def hip_finalize(o_run):
   return call(o_run)
 
 
-def hip_flash_attention_vjp(q, k, v, scale: float, static_scratch: bool = False, keep_mask=None):
-  """Differentiable attention on [B,S,H,D] bf16 arrays: jax.custom_vjp around the forward and backward custom calls
-  (what kernels/splash_attention/splash_attention_kernel.py:1277-1600 does for the Pallas kernel).  static_scratch:
-  the backward that needs no workspace result (its scratch is a static device array of the library); keep_mask: a
-  [B,Skv] key padding mask, honoured by the forward and the backward alike."""
+def hip_flash_attention_vjp(q, k, v, scale: float, static_scratch: bool = False, keep_mask=None, layout: int = 0,
+                            residual_checkpoint_name: str | None = None):
+  """Differentiable attention: jax.custom_vjp around the forward and backward custom calls (what
+  kernels/splash_attention/splash_attention_kernel.py:1166, :2067 do for the Pallas kernels), on [B,S,H,D] (layout 0) or
+  [B,H,S,D] (layout 1) bf16 arrays; returns out [B,Sq,H,D].  keep_mask: a [B,Skv] key padding mask, honoured by the
+  forward and the backward alike.  residual_checkpoint_name: the saved (out, lse) are tagged with
+  jax.ad_checkpoint.checkpoint_name, as the reference's wrappers tag their residuals for the remat policies
+  (models/attention_flax.py:1941-1962).  static_scratch: the backward whose scratch is a static device array of the
+  library (no workspace result); used only when the shape fits that array (decided here, at trace time), and it assumes
+  that XLA runs the custom calls of one GPU on one stream: two such calls overlapping on one GPU would race on the array."""
   jax, jnp = _require_jax()
   bias = hip_key_mask_bias(keep_mask) if keep_mask is not None else None
+  if keep_mask is not None:
+    skv = _bshd_dims(k, layout)[1]
+    if tuple(keep_mask.shape) != (q.shape[0], skv):
+      raise ValueError(f"attention_mask must have shape [batch, kv_length] = {(q.shape[0], skv)}, got {tuple(keep_mask.shape)}.")
+  b, sq, h, d = _bshd_dims(q, layout)
+  results = (jax.ShapeDtypeStruct((b, sq, h, d), jnp.bfloat16), jax.ShapeDtypeStruct((b, h, sq), jnp.float32))
+  nws = 2 * b * h * ((sq + 31) // 32 * 32)  # mdattn_bwd_workspace_floats
+  use_static = static_scratch and bias is None and nws <= BWD_STATIC_MAX_FLOATS
+  # the backward custom calls take [B,S,H,D] operands: layout 1 inputs are transposed for them (XLA fuses the copies
+  # into the producers where it can); the forward reads either layout in place
+  to_bshd = (lambda x: x) if layout == 0 else (lambda x: x.transpose(0, 2, 1, 3))
 
   def forward(q, k, v):
     if bias is None:
-      return hip_flash_attention(q, k, v, scale, 0)
-    b, sq, h, d = q.shape
-    call = jax.ffi.ffi_call("mdattn_fwd_bf16_bias", (jax.ShapeDtypeStruct((b, sq, h, d), jnp.bfloat16), jax.ShapeDtypeStruct((b, h, sq), jnp.float32)),
-                            vmap_method="sequential")
-    return call(q, k, v, bias, scale=_f32(scale), layout=_i64(0))
+      call = jax.ffi.ffi_call("mdattn_fwd_bf16", results, vmap_method="sequential")
+      return call(q, k, v, scale=_f32(scale), layout=_i64(layout))
+    call = jax.ffi.ffi_call("mdattn_fwd_bf16_bias", results, vmap_method="sequential")
+    return call(q, k, v, bias, scale=_f32(scale), layout=_i64(layout))
 
   @jax.custom_vjp
   def attn(q, k, v):
@@ -204,43 +225,81 @@ def hip_flash_attention_vjp(q, k, v, scale: float, static_scratch: bool = False,
 
   def fwd(q, k, v):
     out, lse = forward(q, k, v)
+    if residual_checkpoint_name is not None:
+      from jax.ad_checkpoint import checkpoint_name
+
+      out, lse = checkpoint_name(out, residual_checkpoint_name), checkpoint_name(lse, residual_checkpoint_name + "_lse")
     return out, (q, k, v, out, lse)
 
   def bwd(res, dout):
     q, k, v, out, lse = res
-    b, sq, h, d = q.shape
+    q, k, v = to_bshd(q), to_bshd(k), to_bshd(v)
     grads = (jax.ShapeDtypeStruct(q.shape, jnp.bfloat16), jax.ShapeDtypeStruct(k.shape, jnp.bfloat16), jax.ShapeDtypeStruct(v.shape, jnp.bfloat16))
-    if static_scratch and bias is None:
+    if use_static:
       call = jax.ffi.ffi_call("mdattn_bwd_bf16_static", grads, vmap_method="sequential")
-      return tuple(call(q, k, v, out, dout.astype(jnp.bfloat16), lse, scale=_f32(scale)))
-    nws = 2 * b * h * ((sq + 31) // 32 * 32)  # mdattn_bwd_workspace_floats
-    results = grads + (jax.ShapeDtypeStruct((nws,), jnp.float32),)
-    if bias is not None:
-      call = jax.ffi.ffi_call("mdattn_bwd_bf16_bias", results, vmap_method="sequential")
-      dq, dk, dv, _ = call(q, k, v, out, dout.astype(jnp.bfloat16), lse, bias, scale=_f32(scale))
+      dq, dk, dv = call(q, k, v, out, dout.astype(jnp.bfloat16), lse, scale=_f32(scale))
     else:
-      call = jax.ffi.ffi_call("mdattn_bwd_bf16", results, vmap_method="sequential")
-      dq, dk, dv, _ = call(q, k, v, out, dout.astype(jnp.bfloat16), lse, scale=_f32(scale))
-    return dq, dk, dv
+      results_b = grads + (jax.ShapeDtypeStruct((nws,), jnp.float32),)
+      if bias is not None:
+        call = jax.ffi.ffi_call("mdattn_bwd_bf16_bias", results_b, vmap_method="sequential")
+        dq, dk, dv, _ = call(q, k, v, out, dout.astype(jnp.bfloat16), lse, bias, scale=_f32(scale))
+      else:
+        call = jax.ffi.ffi_call("mdattn_bwd_bf16", results_b, vmap_method="sequential")
+        dq, dk, dv, _ = call(q, k, v, out, dout.astype(jnp.bfloat16), lse, scale=_f32(scale))
+    return to_bshd(dq), to_bshd(dk), to_bshd(dv)  # the transposition is its own inverse: back to the inputs' layout
 
   attn.defvjp(fwd, bwd)
   return attn(q, k, v)
 
 
+def _partial_rows_floats(rows: int, columns: int) -> int:
+  return min(rows, NORM_ROPE_BWD_MAX_PARTIAL_ROWS) * columns
+
+
 def hip_norm_rope_fullrow(q, k, wq, wk, cos, sin, heads: int, eps: float = 1e-6, q_mul: float = 1.0):
   """q, k [B,S,H*D] bf16 (k may be None: cached text K/V); cos/sin f32 [S,D/2] or None (norm only) -> (q_out, k_out)
   [B,S,H,D] bf16.  `q_mul` is multiplied into q_out before its rounding: D**-0.5 * log2(e) here and scale = ln 2 in
-  hip_flash_attention carry the softmax scale in the prologue.  FlaxWanAttention.__call__, attention_flax.py:2655-2677."""
+  hip_flash_attention carry the softmax scale in the prologue.  FlaxWanAttention.__call__, attention_flax.py:2655-2677.
+  Differentiable with respect to q, k, wq, wk (jax.custom_vjp around mdattn_norm_rope_fullrow_bwd; the reference
+  differentiates through these lines by autodiff)."""
   jax, jnp = _require_jax()
   b, s, n = q.shape
   d = n // heads
   rope, has_k = cos is not None, k is not None
   dummy = jnp.zeros((8,), jnp.float32)
-  out = jax.ShapeDtypeStruct((b, s, heads, d), jnp.bfloat16)
-  k_out = out if has_k else jax.ShapeDtypeStruct((8,), jnp.bfloat16)
-  call = jax.ffi.ffi_call("mdattn_norm_rope_fullrow", (out, k_out), vmap_method="sequential")
-  q_out, k_res = call(q, k if has_k else q, wq, wk if has_k else wq, cos if rope else dummy, sin if rope else dummy,
-                      eps=_f32(eps), q_mul=_f32(q_mul), heads=_i64(heads), rope=_i64(rope), has_k=_i64(has_k))
+  cos_, sin_ = (cos, sin) if rope else (dummy, dummy)
+  attrs = dict(eps=_f32(eps), q_mul=_f32(q_mul), heads=_i64(heads), rope=_i64(rope), has_k=_i64(has_k))
+
+  def forward(q, k, wq, wk):
+    out = jax.ShapeDtypeStruct((b, s, heads, d), jnp.bfloat16)
+    k_out = out if has_k else jax.ShapeDtypeStruct((8,), jnp.bfloat16)
+    call = jax.ffi.ffi_call("mdattn_norm_rope_fullrow", (out, k_out), vmap_method="sequential")
+    return call(q, k, wq, wk, cos_, sin_, **attrs)
+
+  @jax.custom_vjp
+  def prologue(q, k, wq, wk):
+    return forward(q, k, wq, wk)
+
+  def fwd(q, k, wq, wk):
+    return forward(q, k, wq, wk), (q, k, wq, wk)
+
+  def bwd(res, g):
+    q, k, wq, wk = res
+    gq, gk = g
+    cols = n * (2 if has_k else 1)
+    small = jax.ShapeDtypeStruct((8,), jnp.bfloat16)
+    small_f = jax.ShapeDtypeStruct((8,), jnp.float32)
+    results = (jax.ShapeDtypeStruct(q.shape, jnp.bfloat16), jax.ShapeDtypeStruct(q.shape, jnp.bfloat16) if has_k else small,
+               jax.ShapeDtypeStruct((n,), jnp.float32), jax.ShapeDtypeStruct((n,), jnp.float32) if has_k else small_f, small_f,
+               jax.ShapeDtypeStruct((_partial_rows_floats(b * s, cols),), jnp.float32))
+    call = jax.ffi.ffi_call("mdattn_norm_rope_fullrow_bwd", results, vmap_method="sequential")
+    dq, dk, dwq, dwk, _, _ = call(q, k, gq.astype(jnp.bfloat16), gk.astype(jnp.bfloat16) if has_k else gq.astype(jnp.bfloat16), wq, wk,
+                                  cos_, sin_, wq, has_bias=_i64(0), **attrs)
+    # without k the stand-in operands (q, wq) receive zero cotangents
+    return dq, (dk if has_k else jnp.zeros(k.shape, k.dtype)), dwq.astype(wq.dtype), (dwk.astype(wk.dtype) if has_k else jnp.zeros(wk.shape, wk.dtype))
+
+  prologue.defvjp(fwd, bwd)
+  q_out, k_res = prologue(q, k if has_k else q, wq, wk if has_k else wq)
   return q_out, (k_res if has_k else None)
 
 
@@ -267,18 +326,47 @@ def hip_norm_rope_qkv(qkv, wq, wk, cos, sin, heads: int, bias=None, eps: float =
 def hip_norm_rope_perhead(q, k, wq, wk, cos, sin, eps: float = 1e-6, wq_txt=None, wk_txt=None, n_txt: int = 0, q_mul: float = 1.0):
   """q, k [B,S,H,D] bf16 (k may be None); per-head RMSNorm with weights [D]; tokens [0, n_txt) take wq_txt / wk_txt
   (FlaxFluxAttention's encoder_*_norm on the text tokens of the joint sequence, attention_flax.py:3002-3003);
-  cos/sin f32 [S,D/2] or None -> (q_out, k_out) [B,S,H,D] bf16.  FlaxFluxAttention.__call__, :2989-3020."""
+  cos/sin f32 [S,D/2] or None -> (q_out, k_out) [B,S,H,D] bf16.  FlaxFluxAttention.__call__, :2989-3020.
+  Differentiable with respect to q, k and the four weights (jax.custom_vjp around mdattn_norm_rope_perhead_bwd)."""
   jax, jnp = _require_jax()
   rope, has_k = cos is not None, k is not None
   if n_txt and (wq_txt is None or (has_k and wk_txt is None)):
     raise ValueError("n_txt > 0 needs the text-token norm weights wq_txt (and wk_txt with k)")
   dummy = jnp.zeros((8,), jnp.float32)
-  out = jax.ShapeDtypeStruct(q.shape, jnp.bfloat16)
-  k_out = out if has_k else jax.ShapeDtypeStruct((8,), jnp.bfloat16)
-  call = jax.ffi.ffi_call("mdattn_norm_rope_perhead", (out, k_out), vmap_method="sequential")
-  q_out, k_res = call(q, k if has_k else q, wq, wk if has_k else wq, wq_txt if n_txt else wq, wk_txt if (n_txt and has_k) else wq,
-                      cos if rope else dummy, sin if rope else dummy,
-                      eps=_f32(eps), q_mul=_f32(q_mul), n_txt=_i64(n_txt), rope=_i64(rope), has_k=_i64(has_k))
+  cos_, sin_ = (cos, sin) if rope else (dummy, dummy)
+  d = q.shape[-1]
+  attrs = dict(eps=_f32(eps), q_mul=_f32(q_mul), n_txt=_i64(n_txt), rope=_i64(rope), has_k=_i64(has_k))
+
+  def forward(q, k, wq, wk, wqt, wkt):
+    out = jax.ShapeDtypeStruct(q.shape, jnp.bfloat16)
+    k_out = out if has_k else jax.ShapeDtypeStruct((8,), jnp.bfloat16)
+    call = jax.ffi.ffi_call("mdattn_norm_rope_perhead", (out, k_out), vmap_method="sequential")
+    return call(q, k, wq, wk, wqt, wkt, cos_, sin_, **attrs)
+
+  @jax.custom_vjp
+  def prologue(q, k, wq, wk, wqt, wkt):
+    return forward(q, k, wq, wk, wqt, wkt)
+
+  def fwd(q, k, wq, wk, wqt, wkt):
+    return forward(q, k, wq, wk, wqt, wkt), (q, k, wq, wk, wqt, wkt)
+
+  def bwd(res, g):
+    q, k, wq, wk, wqt, wkt = res
+    gq, gk = g
+    b, s, h, _ = q.shape
+    act, vec = jax.ShapeDtypeStruct(q.shape, jnp.bfloat16), jax.ShapeDtypeStruct((d,), jnp.float32)
+    small, small_f = jax.ShapeDtypeStruct((8,), jnp.bfloat16), jax.ShapeDtypeStruct((8,), jnp.float32)
+    results = (act, act if has_k else small, vec, vec if has_k else small_f, vec if n_txt else small_f,
+               vec if (n_txt and has_k) else small_f, jax.ShapeDtypeStruct((_partial_rows_floats(b * s * h, 4 * d),), jnp.float32))
+    call = jax.ffi.ffi_call("mdattn_norm_rope_perhead_bwd", results, vmap_method="sequential")
+    gq = gq.astype(jnp.bfloat16)
+    dq, dk, dwq, dwk, dwqt, dwkt, _ = call(q, k, gq, gk.astype(jnp.bfloat16) if has_k else gq, wq, wk, wqt, wkt, cos_, sin_, **attrs)
+    zero = lambda x: jnp.zeros(x.shape, x.dtype)
+    return (dq, dk if has_k else zero(k), dwq.astype(wq.dtype), dwk.astype(wk.dtype) if has_k else zero(wk),
+            dwqt.astype(wqt.dtype) if n_txt else zero(wqt), dwkt.astype(wkt.dtype) if (n_txt and has_k) else zero(wkt))
+
+  prologue.defvjp(fwd, bwd)
+  q_out, k_res = prologue(q, k if has_k else q, wq, wk if has_k else wq, wq_txt if n_txt else wq, wk_txt if (n_txt and has_k) else wq)
   return q_out, (k_res if has_k else None)
 
 
@@ -298,11 +386,30 @@ def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotar
 
   def run(x, scale, tab):
     b, s, n = x.shape
-    out = jax.ShapeDtypeStruct((b, s, heads, n // heads), jnp.bfloat16)
     mode = 0 if tab is None else (1 if rope_type == "interleaved" else 2)
     cos, sin = (dummy, dummy) if tab is None else (tab[0].astype(jnp.float32), tab[1].astype(jnp.float32))
-    call = jax.ffi.ffi_call("mdattn_norm_rope_rows", out, vmap_method="sequential")
-    return call(x, scale.astype(jnp.float32), cos, sin, eps=_f32(eps), heads=_i64(heads), mode=_i64(mode))
+    attrs = dict(eps=_f32(eps), heads=_i64(heads), mode=_i64(mode))
+
+    def forward(x, w):
+      out = jax.ShapeDtypeStruct((b, s, heads, n // heads), jnp.bfloat16)
+      return jax.ffi.ffi_call("mdattn_norm_rope_rows", out, vmap_method="sequential")(x, w, cos, sin, **attrs)
+
+    @jax.custom_vjp
+    def prologue(x, w):
+      return forward(x, w)
+
+    def fwd(x, w):
+      return forward(x, w), (x, w)
+
+    def bwd(res, g):
+      x, w = res
+      results = (jax.ShapeDtypeStruct(x.shape, x.dtype), jax.ShapeDtypeStruct((n,), jnp.float32),
+                 jax.ShapeDtypeStruct((_partial_rows_floats(b * s, n),), jnp.float32))
+      dx, dw, _ = jax.ffi.ffi_call("mdattn_norm_rope_rows_bwd", results, vmap_method="sequential")(x, g.astype(jnp.bfloat16), w, cos, sin, **attrs)
+      return dx, dw
+
+    prologue.defvjp(fwd, bwd)
+    return prologue(x, scale.astype(jnp.float32))
 
   q_scale = norm_q_scale if q_mul == 1.0 else norm_q_scale * q_mul
   return run(query, q_scale, q_tab), (run(key, norm_k_scale, k_tab) if key is not None else None)
@@ -318,14 +425,20 @@ def _as_rank4(q, k, v, heads: int):
 
 
 def hip_flash_kernel(q, k, v, context):
-  """The KERNEL_REGISTRY entry `hip_flash`: fn(q, k, v, context) -> [B, Sq, H*D] in q's dtype."""
+  """The KERNEL_REGISTRY entry `hip_flash`: fn(q, k, v, context) -> [B, Sq, H*D] in q's dtype.  The function is a
+  jax.custom_vjp (forward custom call with lse, backward custom calls): the trainer differentiates straight through
+  `apply_attention` (trainers/wan_trainer.py:169), as it does through the reference's own kernels
+  (kernels/splash_attention/splash_attention_kernel.py:1166, :2067).  Both input layouts, the key mask and
+  context["residual_checkpoint_name"] are honoured.  f32 inputs (LTX-2's q, k) are cast to bf16 by XLA, one more pass
+  over each; `hip_norm_rope_ltx2` in front of this entry emits bf16 and leaves nothing to cast."""
   _, jnp = _require_jax()
   if context.get("is_causal"):
     raise NotImplementedError("hip_flash is non-causal")
   q4, k4, v4, layout = _as_rank4(q, k, v, context["heads"])
   dt = q.dtype
-  out, _ = hip_flash_attention(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"], layout,
-                               keep_mask=context.get("attention_mask"))
+  out = hip_flash_attention_vjp(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"],
+                                keep_mask=context.get("attention_mask"), layout=layout,
+                                residual_checkpoint_name=context.get("residual_checkpoint_name"))
   b, sq, h, d = out.shape
   return out.reshape(b, sq, h * d).astype(dt)
 

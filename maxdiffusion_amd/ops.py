@@ -16,7 +16,8 @@ from . import _lib
 from ._lib import Strides
 
 __all__ = [
-    "norm_rope_fullrow", "norm_rope_qkv", "norm_rope_perhead", "norm_rope_rows", "flash_attention", "flash_attention_backward", "flash_attention_backward_static", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
+    "norm_rope_fullrow", "norm_rope_qkv", "norm_rope_perhead", "norm_rope_rows",
+    "norm_rope_fullrow_backward", "norm_rope_perhead_backward", "norm_rope_rows_backward", "flash_attention", "flash_attention_backward", "flash_attention_backward_static", "flash_attention_fp8", "quant_e4m3", "key_mask_bias",
     "merge_partial", "flash_attention_merge", "finalize", "new_merge_state", "LSE_INIT", "FOLDED_SCALE", "folded_q_mul", "set_fwd_schedule", "FWD_SCHEDULES", "FP8_SOFTMAX_MODES",
 ]
 
@@ -186,6 +187,136 @@ def norm_rope_perhead(q, k, wq, wk, cos, sin, eps: float = 1e-6, wq_txt=None, wk
       _ptr(cos), _ptr(sin), b, s, h, d, eps, q_mul, ctypes.byref(si), ctypes.byref(so))
   _lib.check(rc, "mdattn_norm_rope_perhead")
   return q_out, k_out
+
+
+def _bwd_workspace(rows: int, columns: int, device):
+  n = _lib.load().mdattn_norm_rope_bwd_workspace_floats(rows, columns)
+  return torch.empty(n, dtype=torch.float32, device=device), n
+
+
+def _grad_view(g, like_shape, name):
+  if g.dim() != 4 or tuple(g.shape) != tuple(like_shape) or g.dtype != torch.bfloat16:
+    raise ValueError(f"{name} must be a bf16 logical [B,S,H,D] = {tuple(like_shape)} view, got {tuple(g.shape)} {g.dtype}")
+  if g.stride(3) != 1:
+    g = g.contiguous()
+  return g
+
+
+def norm_rope_fullrow_backward(q, k, wq, wk, cos, sin, heads: int, gq, gk, eps: float = 1e-6, q_mul: float = 1.0, bias=None,
+                               dq=None, dk=None):
+  """Backward of `norm_rope_fullrow` (and, with `bias` bf16 [2*H*D], of the q | k blocks of `norm_rope_qkv`).
+
+  q, k: the saved bf16 [B,S,H*D] inputs (k may be None, then gk is None); gq, gk: bf16 logical [B,S,H,D] gradients of
+  the prologue's outputs.  Returns (dq, dk, dwq, dwk) -- dq, dk bf16 shaped and strided like q, k (or written into
+  the given dq / dk, which may be the column blocks of a fused gradient buffer), dwq, dwk f32 [H*D] -- plus dbias
+  f32 [2*H*D] when bias is given."""
+  _check_dev(q, k, wq, wk, cos, sin, gq, gk, bias, dq, dk)
+  if q.dim() != 3 or q.dtype != torch.bfloat16 or q.stride(2) != 1:
+    raise ValueError("q must be bf16 [B, S, H*D] with a contiguous last axis")
+  b, s, n = q.shape
+  if n % heads:
+    raise ValueError(f"inner dim {n} is not divisible by heads={heads}")
+  d = n // heads
+  has_k = k is not None
+  if has_k and (k.shape != q.shape or k.dtype != q.dtype or k.stride() != q.stride()):
+    raise ValueError("k must match q in shape, dtype and strides")
+  if has_k != (gk is not None):
+    raise ValueError("gk must be given exactly when k is")
+  cos, sin = _table(cos, s, d, "cos"), _table(sin, s, d, "sin")
+  gq = _grad_view(gq, (b, s, heads, d), "gq")
+  if has_k:
+    gk = _grad_view(gk, (b, s, heads, d), "gk")
+    if gk.stride() != gq.stride():
+      gk = torch.empty_strided(gq.shape, gq.stride(), dtype=gk.dtype, device=gk.device).copy_(gk)
+  if bias is not None and (not has_k or bias.dtype != torch.bfloat16 or bias.numel() != 2 * n or not bias.is_contiguous()):
+    raise ValueError("bias must be a contiguous bf16 [2*H*D] tensor (q | k blocks) and needs k")
+  if dq is None:
+    dq = torch.empty_strided(q.shape, q.stride(), dtype=torch.bfloat16, device=q.device)
+  if has_k and dk is None:
+    dk = torch.empty_strided(q.shape, q.stride(), dtype=torch.bfloat16, device=q.device)
+  for name, t in (("dq", dq), ("dk", dk)):
+    if t is not None and (t.shape != q.shape or t.dtype != torch.bfloat16 or t.stride(2) != 1 or (has_k and t.stride() != dq.stride())):
+      raise ValueError(f"{name} must be bf16 [B, S, H*D] with a contiguous last axis (dq and dk sharing their strides)")
+  dwq = torch.empty(n, dtype=torch.float32, device=q.device)
+  dwk = torch.empty(n, dtype=torch.float32, device=q.device) if has_k else None
+  dbias = torch.empty(2 * n, dtype=torch.float32, device=q.device) if bias is not None else None
+  ws, nws = _bwd_workspace(b * s, (2 if has_k else 1) * (2 if bias is not None else 1) * n, q.device)
+  st = _strides(gq)
+  rc = _lib.load().mdattn_norm_rope_fullrow_bwd(
+      _stream(), _ptr(q), _ptr(k), _ptr(bias), _ptr(gq), _ptr(gk), _ptr(dq), _ptr(dk), _ptr(wq), _ptr(wk), _ptr(dwq), _ptr(dwk),
+      _ptr(dbias), _ptr(cos), _ptr(sin), b, s, heads, d, eps, q_mul, q.stride(0), q.stride(1), dq.stride(0), dq.stride(1),
+      ctypes.byref(st), _ptr(ws), nws)
+  _lib.check(rc, "mdattn_norm_rope_fullrow_bwd")
+  return (dq, dk, dwq, dwk) if bias is None else (dq, dk, dwq, dwk, dbias)
+
+
+def norm_rope_perhead_backward(q, k, wq, wk, cos, sin, gq, gk, eps: float = 1e-6, wq_txt=None, wk_txt=None, n_txt: int = 0,
+                               q_mul: float = 1.0):
+  """Backward of `norm_rope_perhead`: q, k the saved bf16 logical [B,S,H,D] inputs (k may be None), gq, gk the
+  gradients of its outputs.  Returns (dq, dk, dwq, dwk, dwq_txt, dwk_txt): dq, dk bf16 laid out like q; the weight
+  gradients f32 [D] (the *_txt ones None when no text weights were given)."""
+  _check_dev(q, k, wq, wk, wq_txt, wk_txt, cos, sin, gq, gk)
+  if q.dtype != torch.bfloat16:
+    raise ValueError("q must be bf16")
+  b, s, h, d = q.shape
+  has_k = k is not None
+  if has_k and (k.shape != q.shape or k.stride() != q.stride() or k.dtype != q.dtype):
+    raise ValueError("k must match q in shape, dtype and strides")
+  if has_k != (gk is not None):
+    raise ValueError("gk must be given exactly when k is")
+  cos, sin = _table(cos, s, d, "cos"), _table(sin, s, d, "sin")
+  gq = _grad_view(gq, q.shape, "gq")
+  if has_k:
+    gk = _grad_view(gk, q.shape, "gk")
+    if gk.stride() != gq.stride():
+      gk = torch.empty_strided(gq.shape, gq.stride(), dtype=gk.dtype, device=gk.device).copy_(gk)
+  dq = torch.empty_strided(q.shape, q.stride(), dtype=torch.bfloat16, device=q.device)
+  dk = torch.empty_strided(q.shape, q.stride(), dtype=torch.bfloat16, device=q.device) if has_k else None
+  f32 = lambda: torch.empty(d, dtype=torch.float32, device=q.device)
+  dwq, dwk = f32(), (f32() if has_k else None)
+  dwq_t = f32() if wq_txt is not None else None
+  dwk_t = f32() if (wk_txt is not None and has_k) else None
+  ws, nws = _bwd_workspace(b * s * h, 4 * d, q.device)
+  si, sd, sg = _strides(q), _strides(dq), _strides(gq)
+  rc = _lib.load().mdattn_norm_rope_perhead_bwd(
+      _stream(), _ptr(q), _ptr(k), _ptr(gq), _ptr(gk), _ptr(dq), _ptr(dk), _ptr(wq), _ptr(wk), _ptr(wq_txt),
+      _ptr(wk_txt if has_k else None), n_txt, _ptr(dwq), _ptr(dwk), _ptr(dwq_t), _ptr(dwk_t), _ptr(cos), _ptr(sin), b, s, h, d, eps, q_mul,
+      ctypes.byref(si), ctypes.byref(sd), ctypes.byref(sg), _ptr(ws), nws)
+  _lib.check(rc, "mdattn_norm_rope_perhead_bwd")
+  return dq, dk, dwq, dwk, dwq_t, dwk_t
+
+
+def norm_rope_rows_backward(x, w, g, cos=None, sin=None, heads: int = 1, mode: str = "none", eps: float = 1e-6):
+  """Backward of `norm_rope_rows`: x the saved [B,S,H*D] input (bf16 or f32), g the bf16 logical [B,S,H,D] gradient of
+  its output.  Returns (dx in x's dtype and strides, dw f32 [H*D])."""
+  _check_dev(x, w, cos, sin, g)
+  if x.dim() != 3 or x.dtype not in (torch.bfloat16, torch.float32) or x.stride(2) != 1:
+    raise ValueError("x must be bf16 or f32 [B, S, H*D] with a contiguous last axis")
+  b, s, n = x.shape
+  if n % heads:
+    raise ValueError(f"inner dim {n} is not divisible by heads={heads}")
+  d = n // heads
+  modes = {"none": 0, "interleaved": 1, "split": 2}
+  if mode not in modes:
+    raise ValueError(f"mode={mode!r} not supported. Choose between 'none', 'interleaved' and 'split'.")
+  if w.dtype != torch.float32 or w.numel() != n or not w.is_contiguous():
+    raise ValueError("w must be a contiguous f32 [H*D] tensor")
+  if mode != "none":
+    want = (b, s, n) if mode == "interleaved" else (b, heads, s, d // 2)
+    for name, t in (("cos", cos), ("sin", sin)):
+      if t is None or tuple(t.shape) != want or t.dtype != torch.float32 or not t.is_contiguous():
+        raise ValueError(f"{name} must be a contiguous f32 tensor of shape {want} for mode={mode!r}")
+  g = _grad_view(g, (b, s, heads, d), "g")
+  dx = torch.empty_strided(x.shape, x.stride(), dtype=x.dtype, device=x.device)
+  dw = torch.empty(n, dtype=torch.float32, device=x.device)
+  ws, nws = _bwd_workspace(b * s, n, x.device)
+  st = _strides(g)
+  rc = _lib.load().mdattn_norm_rope_rows_bwd(
+      _stream(), _ptr(x), int(x.dtype == torch.float32), _ptr(g), _ptr(dx), _ptr(w), _ptr(dw), _ptr(cos if mode != "none" else None),
+      _ptr(sin if mode != "none" else None), modes[mode], b, s, heads, d, eps, x.stride(0), x.stride(1), dx.stride(0), dx.stride(1),
+      ctypes.byref(st), _ptr(ws), nws)
+  _lib.check(rc, "mdattn_norm_rope_rows_bwd")
+  return dx, dw
 
 
 def key_mask_bias(keep: torch.Tensor, masked_value: float = -math.inf) -> torch.Tensor:

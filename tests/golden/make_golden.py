@@ -103,7 +103,57 @@ def main():
   u = lambda a: a.transpose(1, 0, 2)[None].astype(np.float32)
   np.savez_compressed(os.path.join(HERE, "attention_bwd_small.npz"), q=bits(q), k=bits(k), v=bits(v), do=bits(do),
                       scale=128**-0.5, dq=u(dq), dk=u(dk), dv=u(dv))
+  prologue_bwd()
+
+
+def prologue_bwd():
+  """Backward of the three prologue forms on the shapes of the forward fixtures (norm_rope_wan/flux/ltx2.npz)."""
+  grid, H, D = (3, 4, 4), 4, 128
+  S = 3 * 4 * 4
+  q, k = O.normal_bf16((1, S, H * D), 0), O.normal_bf16((1, S, H * D), 1)
+  wq, wk = O.norm_weight(H * D, 3), O.norm_weight(H * D, 4)
+  gq, gk = O.normal_bf16((1, S, H, D), 7), O.normal_bf16((1, S, H, D), 8)
+  bias = O.bf16_round(0.5 * O.normal_bf16((2 * H * D,), 9))
+  cos, sin = O.wan_rope_table(grid, D)
+  f = lambda a: a.astype(np.float32)
+  dq, dwq = O.norm_rope_fullrow_bwd(q, wq, cos, sin, H, gq, q_mul=0.125)
+  dk, dwk = O.norm_rope_fullrow_bwd(k, wk, cos, sin, H, gk)
+  dqb, dwqb = O.norm_rope_fullrow_bwd(q, wq, cos, sin, H, gq, q_mul=0.125, bias=bias[:H * D])
+  dkb, dwkb = O.norm_rope_fullrow_bwd(k, wk, cos, sin, H, gk, bias=bias[H * D:])
+  dqn, dwqn = O.norm_rope_fullrow_bwd(q, wq, None, None, H, gq)
+  wan = dict(q=bits(q), k=bits(k), wq=bits(wq), wk=bits(wk), gq=bits(gq), gk=bits(gk), bias=bits(bias), cos=cos, sin=sin, heads=H,
+             q_mul=0.125, dq=f(dq), dk=f(dk), dwq=f(dwq), dwk=f(dwk), dq_bias=f(dqb), dk_bias=f(dkb), dwq_bias=f(dwqb),
+             dwk_bias=f(dwkb), dq_norm_only=f(dqn), dwq_norm_only=f(dwqn))
+
+  ids = O.flux_ids(5, 4, 6)
+  L = ids.shape[0]
+  q, k = O.normal_bf16((1, L, 3, 128), 0), O.normal_bf16((1, L, 3, 128), 1)
+  gq, gk = O.normal_bf16((1, L, 3, 128), 7), O.normal_bf16((1, L, 3, 128), 8)
+  wq, wk, wqt, wkt = (O.norm_weight(128, s) for s in (3, 4, 5, 6))
+  cos, sin = O.flux_rope_table(ids)
+  dq, dwq, dwqt = O.norm_rope_perhead_bwd(q, wq, cos, sin, gq, q_mul=0.125, w_txt=wqt, n_txt=5)
+  dk, dwk, dwkt = O.norm_rope_perhead_bwd(k, wk, cos, sin, gk, w_txt=wkt, n_txt=5)
+  flux = dict(q=bits(q), k=bits(k), gq=bits(gq), gk=bits(gk), wq=bits(wq), wk=bits(wk), wq_txt=bits(wqt), wk_txt=bits(wkt), cos=cos,
+              sin=sin, n_txt=5, q_mul=0.125, dq=f(dq), dk=f(dk), dwq=f(dwq), dwk=f(dwk), dwq_txt=f(dwqt), dwk_txt=f(dwkt))
+
+  rng = np.random.default_rng(40)
+  B, S, H, D = 2, 9, 4, 64
+  x = O.normal_bf16((B, S, H * D), 0)
+  g = O.normal_bf16((B, S, H, D), 7)
+  w = (1 + 0.1 * rng.standard_normal(H * D)).astype(np.float32)
+  # general full-size tables: the two members of a pair carry different values
+  cos_i, sin_i = (rng.uniform(-1, 1, (B, S, H * D)).astype(np.float32) for _ in range(2))
+  cos_s, sin_s = (rng.uniform(-1, 1, (B, H, S, D // 2)).astype(np.float32) for _ in range(2))
+  ltx = dict(x=bits(x), g=bits(g), w=w, heads=H, cos_i=cos_i, sin_i=sin_i, cos_s=cos_s, sin_s=sin_s)
+  for mode, c_, s_ in (("none", None, None), ("interleaved", cos_i, sin_i), ("split", cos_s, sin_s)):
+    dx, dw = O.norm_rope_ltx2_bwd(x, w, c_, s_, mode, g.reshape(B, S, H * D))
+    ltx["dx_" + mode], ltx["dw_" + mode] = f(dx), f(dw)
+  np.savez_compressed(os.path.join(HERE, "norm_rope_bwd.npz"), **{"wan_" + k_: v for k_, v in wan.items()},
+                      **{"flux_" + k_: v for k_, v in flux.items()}, **{"ltx2_" + k_: v for k_, v in ltx.items()})
 
 
 if __name__ == "__main__":
-  main()
+  if len(sys.argv) > 1 and sys.argv[1] == "prologue_bwd":
+    prologue_bwd()
+  else:
+    main()

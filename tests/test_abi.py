@@ -22,6 +22,7 @@ def test_header_declares_the_expected_entry_points():
       "mdattn_quant_e4m3", "mdattn_fwd_fp8", "mdattn_merge", "mdattn_finalize", "mdattn_fwd_bf16_bias", "mdattn_key_mask_bias", "mdattn_norm_rope_rows", "mdattn_bwd_bf16", "mdattn_bwd_workspace_floats",
       "mdattn_fwd_bf16_merge", "mdattn_bwd_bf16_static", "mdattn_bwd_static_max_floats",
       "mdattn_build_id", "mdattn_set_fwd_schedule", "mdattn_norm_rope_qkv", "mdattn_bwd_bf16_bias", "mdattn_fwd_fp8_bias",
+      "mdattn_norm_rope_bwd_workspace_floats", "mdattn_norm_rope_fullrow_bwd", "mdattn_norm_rope_perhead_bwd", "mdattn_norm_rope_rows_bwd",
   ])
 
 

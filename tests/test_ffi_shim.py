@@ -96,6 +96,9 @@ class _FakeArray:
   def __mul__(self, other):
     return _FakeArray(self.shape, self.dtype)
 
+  def transpose(self, *axes):
+    return _FakeArray(tuple(self.shape[a] for a in axes), self.dtype)
+
   def __getitem__(self, idx):  # slicing of the last axis only: x[:, :, a:]
     a = idx[-1].start or 0
     return _FakeArray(self.shape[:-1] + (self.shape[-1] - a,), self.dtype)
@@ -136,8 +139,15 @@ def fake_jax(monkeypatch):
       return out
 
   jax.custom_vjp = _CustomVjp
-  jax.ffi, jax.numpy = ffi, jnp
-  for name, mod in (("jax", jax), ("jax.ffi", ffi), ("jax.numpy", jnp)):
+  adc = types.ModuleType("jax.ad_checkpoint")
+
+  def checkpoint_name(x, name):
+    calls.append({"checkpoint_name": name, "shape": x.shape})
+    return x
+
+  adc.checkpoint_name = checkpoint_name
+  jax.ffi, jax.numpy, jax.ad_checkpoint = ffi, jnp, adc
+  for name, mod in (("jax", jax), ("jax.ffi", ffi), ("jax.numpy", jnp), ("jax.ad_checkpoint", adc)):
     monkeypatch.setitem(sys.modules, name, mod)
   return calls
 
@@ -173,6 +183,8 @@ def test_python_wrappers_follow_the_bind_lines(fake_jax):
   binds = _bind_lines()
   seen = set()
   for c in fake_jax:
+    if "target" not in c:
+      continue
     impl, n_arg, n_ret, attrs = binds[P.FFI_TARGETS[c["target"]]]
     seen.add(c["target"])
     n_results = len(c["results"]) if isinstance(c["results"], tuple) else 1
@@ -199,6 +211,51 @@ def test_python_wrappers_follow_the_bind_lines(fake_jax):
     P.hip_flash_kernel(q3, k3, k3, dict(ctx, is_causal=True))
   with pytest.raises(ValueError, match=r"\[batch, kv_length\]"):
     P.hip_flash_attention(q, k, v, 0.1, 0, keep_mask=_FakeArray((B, 40), "bool_"))
+
+
+def test_registered_entry_is_differentiable(fake_jax):
+  """The function `install()` registers as `hip_flash` is a custom_vjp: forward custom call with lse, backward custom
+  calls, in both input layouts, with a key mask, with the residuals tagged by context["residual_checkpoint_name"];
+  the prologue hooks are custom_vjps too; the static-scratch backward is used only for shapes that fit its array."""
+  from maxdiffusion_amd import jax_plugin as P
+
+  bf = "bfloat16"
+  B, S, Skv, H, D = 2, 40, 60, 3, 128
+  ctx = {"heads": H, "scale": 0.1, "attention_mask": None, "is_causal": False, "residual_checkpoint_name": "attn_res"}
+  targets = lambda: [c["target"] for c in fake_jax if "target" in c]
+  # rank 3 ([B,S,H*D], layout 0)
+  q3, k3 = _FakeArray((B, S, H * D), bf), _FakeArray((B, Skv, H * D), bf)
+  assert P.hip_flash_kernel(q3, k3, k3, ctx).shape == (B, S, H * D)
+  assert targets() == ["mdattn_fwd_bf16", "mdattn_bwd_bf16"]      # the fake custom_vjp runs fwd and bwd
+  assert [c["checkpoint_name"] for c in fake_jax if "checkpoint_name" in c] == ["attn_res", "attn_res_lse"]
+  fwd, bwd = [c for c in fake_jax if "target" in c]
+  assert fwd["attrs"]["layout"] == 0 and [r.shape for r in bwd["results"][:3]] == [(B, S, H, D), (B, Skv, H, D), (B, Skv, H, D)]
+  # rank 4 ([B,H,S,D], layout 1): the forward reads it in place, the backward's operands are transposed to [B,S,H,D]
+  fake_jax.clear()
+  q4, k4 = _FakeArray((B, H, S, D), bf), _FakeArray((B, H, Skv, D), bf)
+  assert P.hip_flash_kernel(q4, k4, k4, ctx).shape == (B, S, H * D)
+  fwd, bwd = [c for c in fake_jax if "target" in c]
+  assert fwd["attrs"]["layout"] == 1 and fwd["operands"][0].shape == (B, H, S, D)
+  assert [o.shape for o in bwd["operands"][:3]] == [(B, S, H, D), (B, Skv, H, D), (B, Skv, H, D)]
+  # with a key mask: the biased forward and the biased backward
+  fake_jax.clear()
+  P.hip_flash_kernel(q3, k3, k3, dict(ctx, attention_mask=_FakeArray((B, Skv), "bool_")))
+  assert targets() == ["mdattn_key_mask_bias", "mdattn_fwd_bf16_bias", "mdattn_bwd_bf16_bias"]
+  # the static-scratch backward only where 2*B*H*ceil32(Sq) fits its array; beyond, the workspace form
+  fake_jax.clear()
+  P.hip_flash_attention_vjp(_FakeArray((B, S, H, D), bf), _FakeArray((B, Skv, H, D), bf), _FakeArray((B, Skv, H, D), bf), 0.1, static_scratch=True)
+  big = _FakeArray((1, 1 << 21, 4, D), bf)  # 2 * 4 * 2^21 = 16 Mi floats > 8 Mi
+  P.hip_flash_attention_vjp(big, big, big, 0.1, static_scratch=True)
+  assert targets() == ["mdattn_fwd_bf16", "mdattn_bwd_bf16_static", "mdattn_fwd_bf16", "mdattn_bwd_bf16"]
+  m = re.search(r"#define MDATTN_BWD_STATIC_MAX_FLOATS \(([\d\s*]+)\)", open(os.path.join(INCLUDE, "mdattn.h")).read())
+  assert P.BWD_STATIC_MAX_FLOATS == eval(m.group(1))  # digits, blanks and '*' only
+  # the prologue hooks: forward and backward custom calls, workspace result sized min(rows, 1024) * columns
+  fake_jax.clear()
+  w, tab = _FakeArray((H * D,), bf), _FakeArray((S, D // 2), "float32")
+  P.hip_norm_rope_fullrow(q3, q3, w, w, tab, tab, H)
+  assert targets() == ["mdattn_norm_rope_fullrow", "mdattn_norm_rope_fullrow_bwd"]
+  ws = [c for c in fake_jax if c.get("target") == "mdattn_norm_rope_fullrow_bwd"][0]["results"][-1]
+  assert ws.shape == (min(B * S, P.NORM_ROPE_BWD_MAX_PARTIAL_ROWS) * 2 * H * D,)
 
 
 def test_install_registers_both_kernel_names(fake_jax, monkeypatch, tmp_path):
@@ -257,6 +314,8 @@ def test_marshalling_rejects_bad_buffers_by_name(lib):
   B, S, Skv, H, D = 2, 40, 60, 3, 128
   q, k, v = buf((B, S, H, D), BF16), buf((B, Skv, H, D), BF16), buf((B, Skv, H, D), BF16)
   out, lse = buf((B, S, H, D), BF16), buf((B, H, S), F32)
+  q3, wN, wD, tabh = buf((B, S, H * D), BF16), buf((H * D,), BF16), buf((D,), BF16), buf((S, D // 2), F32)
+  fN, fD = buf((H * D,), F32), buf((D,), F32)
   cases = [
       (("fwd_bf16", buf((B, S, H * D), BF16), k, v, out, lse, f(0.1), i(0)), "rank-4"),
       (("fwd_bf16", buf((B, S, H, D), F32), k, v, out, lse, f(0.1), i(0)), "q must be bf16, got f32"),
@@ -294,6 +353,18 @@ def test_marshalling_rejects_bad_buffers_by_name(lib):
         f(1e-6), i(H), i(3)), "mode must be"),
       (("norm_rope_rows", buf((B, S, H * D), BF16), buf((H * D,), BF16), buf((B, S, H * D), F32), buf((B, S, H * D), F32), out,
         f(1e-6), i(H), i(1)), "w must be f32"),
+      (("norm_rope_fullrow_bwd", q3, q3, out, out, wN, wN, tabh, tabh, wN, q3, q3, fN, fN, fN, buf((10,), F32), f(1e-6), f(1.0), i(H), i(1), i(1), i(0)),
+       "workspace must hold at least 768"),
+      (("norm_rope_fullrow_bwd", q3, q3, buf((B, H, S, D), BF16), out, wN, wN, tabh, tabh, wN, q3, q3, fN, fN, fN, buf((768,), F32), f(1e-6), f(1.0), i(H), i(1), i(1), i(0)),
+       "gq must be [B,S,H,D]"),
+      (("norm_rope_fullrow_bwd", q3, q3, out, out, wN, wN, tabh, tabh, wN, q3, q3, buf((H * D,), BF16), fN, fN, buf((768,), F32), f(1e-6), f(1.0), i(H), i(1), i(1), i(0)),
+       "dwq must be f32"),
+      (("norm_rope_fullrow_bwd", q3, q3, out, out, wN, wN, tabh, tabh, wN, q3, q3, fN, fN, fN, buf((768,), F32), f(1e-6), f(1.0), i(H), i(1), i(0), i(1)),
+       "has_bias needs has_k"),
+      (("norm_rope_perhead_bwd", q, q, out, out, wD, wD, wD, wD, tabh, tabh, out, out, fD, fD, fD, buf((2 * D,), F32), buf((4 * D,), F32), f(1e-6), f(1.0), i(5), i(1), i(1)),
+       "dwk_txt must hold 128"),
+      (("norm_rope_rows_bwd", q3, out, buf((H * D,), F32), tabh, tabh, buf((B, S, H * D), F32), fN, buf((H * D,), F32), f(1e-6), i(H), i(0)),
+       "dx must have x's dtype and shape"),
       (("quant_e4m3", q, buf((B, S, H, D), BF16), buf((2,), F32), f(1.0), i(0)), "x8 must be a u8 or f8e4m3fn"),
       (("quant_e4m3", q, buf((B, S, H, D), F8), buf((1,), F32), f(1.0), i(0)), "scale_out must hold 2"),
       (("fwd_fp8", q, k, v, buf((2,), F32), buf((2,), F32), buf((2,), F32), out, lse, f(0.1), i(0), i(0)), "q8, k8, v8 must be u8 or f8e4m3fn"),

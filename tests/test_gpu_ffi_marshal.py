@@ -171,3 +171,52 @@ def test_backward_handlers(dev, lib):
   want = ops.flash_attention_backward(q, k, v, out, dout, lse, scale=0.08, key_bias=bias)
   xla(lib, "bwd_bf16_bias", q, k, v, out, dout, lse, bias, dq, dk, dv, ws, f(0.08))
   assert all(torch.equal(a, b) for a, b in zip((dq, dk, dv), want))
+
+
+def test_prologue_backward_handlers(dev, lib):
+  """The three prologue-backward targets on XLA-shaped buffers (dense, the workspace as a result), bit for bit against the
+  torch-side operators; absent-k and no-text-weight forms pass small stand-in buffers, as the Python wrappers do."""
+  B, S, H, D = 2, 45, 4, 128
+  N = H * D
+  gen = torch.Generator(device=dev).manual_seed(5)
+  rnd = lambda *s: torch.randn(s, generator=gen, device=dev).to(torch.bfloat16)
+  q, k, gq, gk = rnd(B, S, N), rnd(B, S, N), rnd(B, S, H, D), rnd(B, S, H, D)
+  wq, wk = (1 + 0.1 * rnd(N).float()).to(torch.bfloat16), (1 + 0.1 * rnd(N).float()).to(torch.bfloat16)
+  ang = torch.rand((S, D // 2), generator=gen, device=dev) * 6.28
+  cos, sin = torch.cos(ang), torch.sin(ang)
+  bias = (0.5 * rnd(2 * N).float()).to(torch.bfloat16)
+  e = lambda *s, dt=torch.float32: torch.empty(s, dtype=dt, device=dev)
+  small_b, small_f = e(8, dt=torch.bfloat16), e(8)
+  # full row, q and k, with the projection biases
+  dq, dk, dwq, dwk, db = e(B, S, N, dt=torch.bfloat16), e(B, S, N, dt=torch.bfloat16), e(N), e(N), e(2 * N)
+  ws = e(min(B * S, 1024) * 4 * N)
+  xla(lib, "norm_rope_fullrow_bwd", q, k, gq, gk, wq, wk, cos, sin, bias, dq, dk, dwq, dwk, db, ws, f(1e-6), f(0.5), i(H), i(1), i(1), i(1))
+  want = ops.norm_rope_fullrow_backward(q, k, wq, wk, cos, sin, H, gq, gk, q_mul=0.5, bias=bias)
+  for got, w_ in zip((dq, dk, dwq, dwk, db), want):
+    assert torch.equal(got, w_)
+  # q alone, norm only: stand-ins for everything of k, for the tables and for the bias
+  ws1 = e(min(B * S, 1024) * N)
+  xla(lib, "norm_rope_fullrow_bwd", q, q, gq, gq, wq, wq, small_f, small_f, wq, dq, small_b, dwq, small_f, small_f, ws1, f(1e-6), f(1.0), i(H),
+      i(0), i(0), i(0))
+  want = ops.norm_rope_fullrow_backward(q, None, wq, None, None, None, H, gq, None)
+  assert torch.equal(dq, want[0]) and torch.equal(dwq, want[2])
+  # per head, text weights on the first 7 tokens
+  q4, k4 = q.view(B, S, H, D), k.view(B, S, H, D)
+  wd = [(1 + 0.1 * rnd(D).float()).to(torch.bfloat16) for _ in range(4)]
+  dq4, dk4 = e(B, S, H, D, dt=torch.bfloat16), e(B, S, H, D, dt=torch.bfloat16)
+  dws = [e(D) for _ in range(4)]
+  wsh = e(min(B * S * H, 1024) * 4 * D)
+  xla(lib, "norm_rope_perhead_bwd", q4, k4, gq, gk, wd[0], wd[1], wd[2], wd[3], cos, sin, dq4, dk4, dws[0], dws[1], dws[2], dws[3], wsh,
+      f(1e-6), f(1.0), i(7), i(1), i(1))
+  want = ops.norm_rope_perhead_backward(q4, k4, wd[0], wd[1], cos, sin, gq, gk, wq_txt=wd[2], wk_txt=wd[3], n_txt=7)
+  for got, w_ in zip((dq4, dk4, *dws), want):
+    assert torch.equal(got, w_)
+  # rows (LTX-2), f32 input, split tables
+  x = torch.randn((B, S, N), generator=gen, device=dev)
+  w32 = 1 + 0.1 * torch.randn(N, generator=gen, device=dev)
+  angs = torch.rand((B, H, S, D // 2), generator=gen, device=dev) * 6.28
+  cs, sn = torch.cos(angs), torch.sin(angs)
+  dx, dw, wsr = e(B, S, N), e(N), e(min(B * S, 1024) * N)
+  xla(lib, "norm_rope_rows_bwd", x, gq, w32, cs, sn, dx, dw, wsr, f(1e-6), i(H), i(2))
+  want = ops.norm_rope_rows_backward(x, w32, gq, cs, sn, heads=H, mode="split")
+  assert torch.equal(dx, want[0]) and torch.equal(dw, want[1])

@@ -61,20 +61,21 @@ class Result {
   T value_;
 };
 
+enum class ErrorCode { kOk = 0, kInvalidArgument = 3, kResourceExhausted = 8, kUnimplemented = 12, kInternal = 13 };
+
 class Error {
  public:
+  Error() = default;
+  Error(ErrorCode code, std::string message) : code_(code), message_(std::move(message)) {}
   static Error Success() { return Error(); }
-  static Error InvalidArgument(std::string message) {
-    Error e;
-    e.message_ = std::move(message);
-    e.ok_ = false;
-    return e;
-  }
-  bool success() const { return ok_; }
+  static Error InvalidArgument(std::string message) { return Error(ErrorCode::kInvalidArgument, std::move(message)); }
+  static Error Internal(std::string message) { return Error(ErrorCode::kInternal, std::move(message)); }
+  bool success() const { return code_ == ErrorCode::kOk; }
+  ErrorCode code() const { return code_; }
   const std::string& message() const { return message_; }
 
  private:
-  bool ok_ = true;
+  ErrorCode code_ = ErrorCode::kOk;
   std::string message_;
 };
 
