@@ -273,6 +273,38 @@ def main():
                 "frac_executed": btf * 7.0 / 5.0 / 2500.0,
                 "flop_counted": bfl, "note": "5 matrix products counted, 7 executed (two atomic-free passes: dq; dk and dv)"}
 
+  # backward of the prologue (input and weight gradients from the saved inputs and the gradients of its outputs)
+  prologue_backward = None
+  if args.with_backward:
+    gq, gk = randn(1, S, H, D), randn(1, S, H, D)
+    if w.norm == "fullrow":
+      runb = lambda: ops.norm_rope_fullrow_backward(q_in, k_in, wq, wk, cos, sin, H, gq, gk, q_mul=q_mul)
+      nlaunch, pb_bytes = 1, 6 * S * H * D * 2 + 2 * S * (D // 2) * 4 + 2 * H * D * (2 + 4)
+      kname_b = "norm_rope_fullrow_bwd_kernel"
+    elif w.norm == "rows":
+      runb = lambda: (ops.norm_rope_rows_backward(q_in, wq, gq, cos, sin, heads=H, mode="interleaved"),
+                      ops.norm_rope_rows_backward(k_in, wk, gk, cos, sin, heads=H, mode="interleaved"))
+      nlaunch, pb_bytes = 2, 6 * S * H * D * 2 + 2 * 2 * S * H * D * 4 + 2 * H * D * (4 + 4)
+      kname_b = "norm_rope_rows_bwd_kernel (two launches: q, k)"
+    else:
+      runb = lambda: ops.norm_rope_perhead_backward(q4, k4, wq, wk, cos, sin, gq, gk, q_mul=q_mul)
+      nlaunch, pb_bytes = 1, 6 * S * H * D * 2 + 2 * S * (D // 2) * 4 + 2 * D * (2 + 4)
+      kname_b = "norm_rope_perhead_bwd_kernel"
+    for _ in range(2):
+      runb()
+    e0, e1 = ev(), ev()
+    e0.record()
+    for _ in range(reps):
+      runb()
+    e1.record()
+    torch.cuda.synchronize()
+    pbms = e0.elapsed_time(e1) / reps
+    prologue_backward = {"bound": "hbm", "achieved": pb_bytes / (pbms * 1e-3) / 1e9, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                         "frac": pb_bytes / (pbms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "traffic": None, "kernel": kname_b,
+                         "ms": pbms, "bytes_per_call": pb_bytes,
+                         "note": "saved inputs and output gradients read once, input gradients written once (bf16), tables, weights and "
+                                 "f32 weight gradients; the time includes the second-stage column sum and the workspace allocation"}
+
   flops = O.attention_flops(1, H, S, Skv * ring, D)
   att_ms = sum(t_att) / len(t_att)
   nr_bytes = O.normrope_bytes(1, S, H, D, with_table=True, per_element_table=w.norm == "rows")
@@ -323,6 +355,8 @@ def main():
     out["cross_attention"] = cross
   if backward:
     out["backward"] = backward
+  if prologue_backward:
+    out["prologue_backward"] = prologue_backward
   if args.cpu_rows > 0:
     out["cpu_baseline"] = cpu_baseline(w, args.cpu_rows)
   print(json.dumps(out), flush=True)

@@ -36,127 +36,204 @@ struct NormRopeBwdFullArgs {
   int64_t in_sb, in_ss, dx_sb, dx_ss, g_sb, g_ss, g_sh;
 };
 
-// One workgroup (256 lanes) per token row at a time, blockIdx.y = tensor (q, k); lane t owns the 16-byte chunks
-// t, t+256, ... (<= MAXC) of every row it sees, so its weight-gradient accumulators are per-lane registers.
-template <int MAXC, bool BIAS>
-__global__ __launch_bounds__(256) void norm_rope_fullrow_bwd_kernel(NormRopeBwdFullArgs a) {
-  const int tid = threadIdx.x, t = blockIdx.y;
+// One workgroup per token row at a time, blockIdx.y = tensor (q, k).  The workgroup has NT = blockDim.x lanes, chosen
+// by the host so that the row's 16-byte chunks divide evenly among them (5120 channels: 640 chunks = 320 lanes x 2);
+// lane t owns the chunks t, t+NT, ... (<= MAXC) of every row it sees, so its weight-gradient accumulators are per-lane
+// registers.
+// Vector ALU: the kernel is as much an ALU load as a memory stream (two passes over a row, three tensors to unpack),
+// so the rotated gradient is kept as f32 between the passes, the weights are unpacked once per workgroup, and q_mul
+// rides on the per-row scalars instead of on every element.
+// Memory: three register buffers rotate (the loop is unrolled three times by hand): while one row is worked on, the
+// raw rows of the next two tokens are in flight.  Vector-memory loads return in order, so whatever a row needs must
+// have been requested before the rows that are still to fly: a row's slice of the rotary table travels in its buffer,
+// and all loads are unconditional (indices clamped) so that the count of loads in flight is the same on every path.
+// Registers: what bounds the kernel is the number of row bytes in flight per CU, i.e. how many workgroups fit next to
+// their row buffers.  The unpacked weights and the weight-gradient accumulators (8 floats per chunk each) therefore
+// live in LDS, each lane reading and writing only its own chunks (no synchronisation; LDS traffic returns on its own
+// counter and does not queue behind the global loads): three workgroups of five waves per CU at 5120 channels.
+// TAB1: every chunk of a lane uses the same table slice (NT a multiple of D/8, true for power-of-two head dims).
+template <int MAXC, bool BIAS, bool TAB1>
+__global__ __launch_bounds__(512) void norm_rope_fullrow_bwd_kernel(NormRopeBwdFullArgs a) {
+  const int tid = threadIdx.x, t = blockIdx.y, NT = blockDim.x;
+  const int wave = tid >> 6, nwaves = NT >> 6;
   const int nchunks = a.N >> 3;
-  __shared__ float red[2][2][16];
+  __shared__ float red[2][2][8];
   const float mul = t == 0 ? a.q_mul : 1.0f;
   const bool rope = a.cos != nullptr;
   const int halfd4 = a.D >> 3;
+  constexpr int TC = TAB1 ? 1 : MAXC;
 
-  uint4 wraw[MAXC];
-  int goff[MAXC], tofs[MAXC];
-  float accw[MAXC][8];
+  // LDS: [MAXC * NT] chunks of 8 floats each for the weights, then the same for the weight-gradient accumulators;
+  // chunk (i, tid) belongs to lane tid alone
+  extern __shared__ __attribute__((aligned(16))) float lds_full[];
+  float4* wl = reinterpret_cast<float4*>(lds_full);
+  float4* al = wl + 2 * MAXC * NT;
+  int goff[MAXC], coff[MAXC], tofs[TC];
   [[maybe_unused]] float accb[MAXC][8];
+  [[maybe_unused]] float bf[MAXC][8];
 #pragma unroll
   for (int i = 0; i < MAXC; ++i) {
-    const int c = tid + i * 256;
-    const int cc = c < nchunks ? c : 0;
+    const int c = tid + i * NT;
+    const int cc = c < nchunks ? c : nchunks - 1;  // lanes past the row's end shadow its last chunk and never store
     const int e = cc << 3;
     const int h = e / a.D, d = e - h * a.D;
-    wraw[i] = a.w[t][cc];
+    float w8[8];
+    unpack8(a.w[t][cc], w8);
+    wl[2 * (i * NT + tid)] = make_float4(w8[0], w8[1], w8[2], w8[3]);
+    wl[2 * (i * NT + tid) + 1] = make_float4(w8[4], w8[5], w8[6], w8[7]);
+    al[2 * (i * NT + tid)] = make_float4(0.f, 0.f, 0.f, 0.f);
+    al[2 * (i * NT + tid) + 1] = make_float4(0.f, 0.f, 0.f, 0.f);
+    coff[i] = cc;
     goff[i] = (int)(h * a.g_sh) + d;
-    tofs[i] = d >> 3;
+    if (i < TC) tofs[i] = d >> 3;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) { accw[i][j] = 0.f; if constexpr (BIAS) accb[i][j] = 0.f; }
+    for (int j = 0; j < 8; ++j) { if constexpr (BIAS) { accb[i][j] = 0.f; bf[i][j] = 0.f; } }
+    if constexpr (BIAS) {
+      if (a.bias[t]) unpack8(a.bias[t][cc], bf[i]);
+    }
   }
+  auto lds8 = [&](const float4* base, int i, float* f) __attribute__((always_inline)) {
+    const float4 v0 = base[2 * (i * NT + tid)], v1 = base[2 * (i * NT + tid) + 1];
+    f[0] = v0.x; f[1] = v0.y; f[2] = v0.z; f[3] = v0.w; f[4] = v1.x; f[5] = v1.y; f[6] = v1.z; f[7] = v1.w;
+  };
+  const float4* cosp = rope ? a.cos : reinterpret_cast<const float4*>(a.w[t]);  // norm only: any readable address, unused
+  const float4* sinp = rope ? a.sin : reinterpret_cast<const float4*>(a.w[t]);
+  const int64_t tstride = rope ? halfd4 : 0;
 
-  int par = 0;
-  for (int tok = blockIdx.x; tok < a.ntok; tok += a.nb, par ^= 1) {
+  struct RowBuf {
+    uint4 x[MAXC], g[MAXC];
+    float4 cs[TC], sn[TC];
+  };
+  const int last = a.ntok - 1;
+  auto load_row = [&](int tok, RowBuf& r) __attribute__((always_inline)) {
+    tok = min(tok, last);
     const int b = tok / a.S, s = tok - b * a.S;
     const uint4* xrow = a.x_in[t] + ((b * a.in_sb + s * a.in_ss) >> 3);
     const __bf16* grow = a.g[t] + b * a.g_sb + s * a.g_ss;
-    uint4 xr[MAXC], gr[MAXC];
+    // (the empty asm statements keep the compiler from moving loads of one row across those of another: the order
+    // of issue is what the waits depend on)
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < TC; ++i) {
+      r.cs[i] = cosp[(int64_t)s * tstride + (rope ? tofs[i] : 0)];
+      r.sn[i] = sinp[(int64_t)s * tstride + (rope ? tofs[i] : 0)];
+    }
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
-      const int c = tid + i * 256;
-      if (c < nchunks) {
-        xr[i] = ld_nt(xrow + c);
-        gr[i] = ld_nt(reinterpret_cast<const uint4*>(grow + goff[i]));
-      }
+      r.x[i] = ld_nt(xrow + coff[i]);
+      r.g[i] = ld_nt(reinterpret_cast<const uint4*>(grow + goff[i]));
     }
-    auto chunk_u = [&](int i, int c, float* u) __attribute__((always_inline)) {
-      unpack8(xr[i], u);
-      if constexpr (BIAS) {
-        if (a.bias[t]) {
-          float bb[8];
-          unpack8(a.bias[t][c], bb);
-#pragma unroll
-          for (int j = 0; j < 8; ++j) u[j] += bb[j];
-        }
-      }
-    };
+    asm volatile("" ::: "memory");
+  };
+
+  int par = 0;
+  // one row: consumes `r` (the row of token tok), then refills it with the row three steps ahead
+  auto step = [&](int tok_, RowBuf& r) __attribute__((always_inline)) {
+    // past the end (the last trip of the three-step loop): the buffer holds the clamped last row; it goes through the
+    // same code with its stores and accumulation switched off, so that the loop has no exit in its middle
+    const bool valid = tok_ < a.ntok;
+    const int tok = min(tok_, last);
+    const int b = tok / a.S, s = tok - b * a.S;
+    // dy0 = R^T g (transposed rotation: dy0 = g0 c + g1 s, dy1 = g1 c - g0 s), without q_mul
     float dy[MAXC][8];
     float ss = 0.f, sd = 0.f;
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
-      const int c = tid + i * 256;
-      if (c < nchunks) {
-        float u[8], gf[8], w[8];
-        chunk_u(i, c, u);
-        unpack8(gr[i], gf);
-        unpack8(wraw[i], w);
-        if (rope) {  // transposed rotation: dy0 = g0 c + g1 s, dy1 = g1 c - g0 s
-          const float4 cs = a.cos[(int64_t)s * halfd4 + tofs[i]], sn = a.sin[(int64_t)s * halfd4 + tofs[i]];
-          const float cc[4] = {cs.x, cs.y, cs.z, cs.w}, sv[4] = {sn.x, sn.y, sn.z, sn.w};
+      float u[8], gf[8];
+      unpack8(r.x[i], u);
+      unpack8(r.g[i], gf);
+      if constexpr (BIAS) {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            dy[i][2 * j] = (gf[2 * j] * cc[j] + gf[2 * j + 1] * sv[j]) * mul;
-            dy[i][2 * j + 1] = (gf[2 * j + 1] * cc[j] - gf[2 * j] * sv[j]) * mul;
-          }
-        } else {
+        for (int j = 0; j < 8; ++j) u[j] += bf[i][j];
+      }
+      if (rope) {
+        const float4 cs = r.cs[TAB1 ? 0 : i], sn = r.sn[TAB1 ? 0 : i];
+        const float cc[4] = {cs.x, cs.y, cs.z, cs.w}, sv[4] = {sn.x, sn.y, sn.z, sn.w};
 #pragma unroll
-          for (int j = 0; j < 8; ++j) dy[i][j] = gf[j] * mul;
+        for (int j = 0; j < 4; ++j) {
+          dy[i][2 * j] = __builtin_fmaf(gf[2 * j], cc[j], gf[2 * j + 1] * sv[j]);
+          dy[i][2 * j + 1] = __builtin_fmaf(gf[2 * j + 1], cc[j], -(gf[2 * j] * sv[j]));
         }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dy[i][j] = gf[j];
+      }
+      if (tid + i * NT < nchunks) {
+        float w8[8];
+        lds8(wl, i, w8);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           ss = __builtin_fmaf(u[j], u[j], ss);
-          sd = __builtin_fmaf(u[j], w[j] * dy[i][j], sd);
+          sd = __builtin_fmaf(u[j], w8[j] * dy[i][j], sd);
         }
       }
     }
     ss = row16_sum(ss);
     sd = row16_sum(sd);
-    if ((tid & 15) == 0) { red[par][0][tid >> 4] = ss; red[par][1][tid >> 4] = sd; }
+    ss += __shfl_xor(ss, 16); sd += __shfl_xor(sd, 16);
+    ss = xhalf_sum(ss); sd = xhalf_sum(sd);
+    if ((tid & 63) == 0) { red[par][0][wave] = ss; red[par][1][wave] = sd; }
     // one barrier per row: the next row writes the other half of `red`, and the row after that comes after the next
     // barrier, which no lane passes before every lane has read this half
     __syncthreads();
     float tss = 0.f, tsd = 0.f;
-#pragma unroll
-    for (int j = 0; j < 16; ++j) { tss += red[par][0][j]; tsd += red[par][1][j]; }
-    const float r = rsqrt_newton(tss * a.inv_n + a.eps);
-    const float coef = r * r * r * tsd * a.inv_n;
+    for (int j = 0; j < nwaves; ++j) { tss += red[par][0][j]; tsd += red[par][1][j]; }
+    par ^= 1;
+    const float r_ = rsqrt_newton(tss * a.inv_n + a.eps);
+    const float rm = r_ * mul;                         // q_mul folded into the row scalars
+    const float coef = r_ * r_ * rm * tsd * a.inv_n;
     uint4* drow = a.dx[t] + ((b * a.dx_sb + s * a.dx_ss) >> 3);
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
-      const int c = tid + i * 256;
-      if (c < nchunks) {
-        float u[8], w[8], du[8];
-        chunk_u(i, c, u);
-        unpack8(wraw[i], w);
+      float u[8], du[8];
+      unpack8(r.x[i], u);  // unpacked again rather than kept: eight registers per chunk for one instruction per element
+      if constexpr (BIAS) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) u[j] += bf[i][j];
+      }
+      if (valid && tid + i * NT < nchunks) {
+        float w8[8], acc[8];
+        lds8(wl, i, w8);
+        lds8(al, i, acc);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          du[j] = r * w[j] * dy[i][j] - coef * u[j];
-          accw[i][j] = __builtin_fmaf(dy[i][j] * r, u[j], accw[i][j]);
+          const float dyr = dy[i][j] * rm;
+          du[j] = __builtin_fmaf(-coef, u[j], w8[j] * dyr);
+          acc[j] = __builtin_fmaf(dyr, u[j], acc[j]);
           if constexpr (BIAS) accb[i][j] += du[j];
         }
-        st_nt(drow + c, pack8(du));
+        al[2 * (i * NT + tid)] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        al[2 * (i * NT + tid) + 1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+        st_nt(drow + coff[i], pack8(du));
       }
     }
+    load_row(tok_ + 3 * a.nb, r);
+  };
+
+  // the three initial requests in the order the loop keeps them in (oldest first): the waits inside the loop are
+  // derived from the order of issue on every path into it
+  RowBuf r0, r1, r2;
+  load_row(blockIdx.x, r0);
+  __builtin_amdgcn_sched_barrier(0);
+  load_row(blockIdx.x + a.nb, r1);
+  __builtin_amdgcn_sched_barrier(0);
+  load_row(blockIdx.x + 2 * a.nb, r2);
+  __builtin_amdgcn_sched_barrier(0);
+  for (int tok = blockIdx.x; tok < a.ntok; tok += 3 * a.nb) {
+    step(tok, r0);
+    step(tok + a.nb, r1);
+    step(tok + 2 * a.nb, r2);
   }
 
   // partial row of this workgroup: [tensor][dw | db][N]
   float* prow = a.part + (int64_t)blockIdx.x * a.ncols + (int64_t)t * (BIAS ? 2 : 1) * a.N;
 #pragma unroll
   for (int i = 0; i < MAXC; ++i) {
-    const int c = tid + i * 256;
+    const int c = tid + i * NT;
     if (c < nchunks) {
       float4* p = reinterpret_cast<float4*>(prow + c * 8);
-      p[0] = make_float4(accw[i][0], accw[i][1], accw[i][2], accw[i][3]);
-      p[1] = make_float4(accw[i][4], accw[i][5], accw[i][6], accw[i][7]);
+      p[0] = al[2 * (i * NT + tid)];
+      p[1] = al[2 * (i * NT + tid) + 1];
       if constexpr (BIAS) {
         float4* pb = reinterpret_cast<float4*>(prow + a.N + c * 8);
         pb[0] = make_float4(accb[i][0], accb[i][1], accb[i][2], accb[i][3]);
@@ -480,6 +557,34 @@ __global__ __launch_bounds__(256) void norm_rope_rows_bwd_kernel(NormRopeBwdRows
   }
 }
 
+// Workgroups of `kernel` (block size nt, dynamic LDS lds) that the current device holds at once.  The backward kernels
+// are persistent loops over token rows: a grid of exactly that many workgroups (or fewer) runs as one even wave, where
+// a fixed grid of 1024 would run as one full round plus a partly filled one.  Asked of the runtime once per kernel,
+// block size and device.
+struct ResidentCache {
+  std::atomic<int> value[8][16];  // [block size / 64 - 1][device]
+};
+static int resident_blocks(ResidentCache& cache, const void* kernel, int nt, int lds) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) return 0;
+  const int slot = nt / 64 - 1;
+  const bool cached = slot >= 0 && slot < 8 && dev < 16;
+  if (cached) {
+    const int v = cache.value[slot][dev].load(std::memory_order_acquire);
+    if (v > 0) return v;
+  }
+  // registers and wave slots from the runtime (asked without LDS: its LDS rule assumes 64 KB per CU), LDS by hand:
+  // a gfx950 CU has 160 KB
+  int per_cu = 0, cus = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, nt, 0) != hipSuccess || per_cu < 1) return 0;
+  if (lds > 0 && (160 * 1024 - 1024) / lds < per_cu) per_cu = (160 * 1024 - 1024) / lds;
+  if (per_cu < 1) per_cu = 1;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) return 0;
+  const int v = per_cu * cus;
+  if (cached) cache.value[slot][dev].store(v, std::memory_order_release);
+  return v;
+}
+
 static int launch_colsum(hipStream_t st, const float* part, int nb, int ncols, int seglen, float* o0, float* o1, float* o2, float* o3) {
   ColsumArgs c;
   c.part = part; c.nb = nb; c.ncols = ncols; c.seglen = seglen;
@@ -498,8 +603,9 @@ extern "C" int64_t mdattn_norm_rope_bwd_workspace_floats(int64_t rows, int64_t c
 }
 
 // number of partial rows a workspace of `floats` allows for `units` independent row units and `ncols` columns
-static int partial_rows(int64_t units, int64_t ncols, int64_t floats) {
+static int partial_rows(int64_t units, int64_t ncols, int64_t floats, int resident = 0) {
   int64_t nb = units < kBwdMaxBlocks ? units : kBwdMaxBlocks;
+  if (resident > 0 && resident < nb) nb = resident;  // one even wave of workgroups
   if (floats / ncols < nb) nb = floats / ncols;
   return (int)nb;
 }
@@ -530,7 +636,20 @@ extern "C" int mdattn_norm_rope_fullrow_bwd(void* stream, const void* q_in, cons
   if (in_stride_batch % 8 || in_stride_seq % 8 || dx_stride_batch % 8 || dx_stride_seq % 8 || !strides_ok(g_strides, 8)) return MDATTN_E_ALIGN;
   const int ntens = has_k ? 2 : 1;
   const int64_t ncols = (int64_t)ntens * (bias ? 2 : 1) * N;
-  const int nb = partial_rows(ntok, ncols, workspace_floats);
+  // lanes per workgroup: the row's chunks split evenly over whole waves, at most two chunks per lane up to 8192 channels
+  const int nchunks = (int)(N / 8);
+  const int maxc = (nchunks + 511) / 512;
+  const int nt = ((nchunks + maxc - 1) / maxc + 63) / 64 * 64;
+  const int lds_bytes = 2 * maxc * nt * 8 * (int)sizeof(float);  // unpacked weights + accumulators, <= 64 KB
+  const bool tab1 = nt % (D / 8) == 0;  // every chunk of a lane then sits at the same offset inside its head
+  void (*kern)(NormRopeBwdFullArgs);
+  if (tab1) kern = maxc == 1 ? (bias ? norm_rope_fullrow_bwd_kernel<1, true, true> : norm_rope_fullrow_bwd_kernel<1, false, true>)
+                             : (bias ? norm_rope_fullrow_bwd_kernel<2, true, true> : norm_rope_fullrow_bwd_kernel<2, false, true>);
+  else kern = maxc == 1 ? (bias ? norm_rope_fullrow_bwd_kernel<1, true, false> : norm_rope_fullrow_bwd_kernel<1, false, false>)
+                        : (bias ? norm_rope_fullrow_bwd_kernel<2, true, false> : norm_rope_fullrow_bwd_kernel<2, false, false>);
+  static ResidentCache resident[2][2][2];
+  const int nb = partial_rows(ntok, ncols, workspace_floats,
+                              resident_blocks(resident[maxc - 1][bias ? 1 : 0][tab1 ? 1 : 0], reinterpret_cast<const void*>(kern), nt, lds_bytes) / ntens);
   if (nb < 1) return MDATTN_E_BADARG;
 
   NormRopeBwdFullArgs a;
@@ -546,19 +665,8 @@ extern "C" int mdattn_norm_rope_fullrow_bwd(void* stream, const void* q_in, cons
   a.eps = eps; a.inv_n = 1.0f / (float)N; a.q_mul = q_mul;
   a.in_sb = in_stride_batch; a.in_ss = in_stride_seq; a.dx_sb = dx_stride_batch; a.dx_ss = dx_stride_seq;
   a.g_sb = g_strides->batch; a.g_ss = g_strides->seq; a.g_sh = g_strides->head;
-  dim3 grid(nb, ntens), block(256);
   hipStream_t st = (hipStream_t)stream;
-  const int nchunks = (int)(N / 8);
-#define MDATTN_LAUNCH_FULL_BWD(MAXC)                                                                             \
-  do {                                                                                                           \
-    if (bias) hipLaunchKernelGGL((norm_rope_fullrow_bwd_kernel<MAXC, true>), grid, block, 0, st, a);             \
-    else hipLaunchKernelGGL((norm_rope_fullrow_bwd_kernel<MAXC, false>), grid, block, 0, st, a);                 \
-  } while (0)
-  if (nchunks <= 256) MDATTN_LAUNCH_FULL_BWD(1);
-  else if (nchunks <= 512) MDATTN_LAUNCH_FULL_BWD(2);
-  else if (nchunks <= 768) MDATTN_LAUNCH_FULL_BWD(3);
-  else MDATTN_LAUNCH_FULL_BWD(4);
-#undef MDATTN_LAUNCH_FULL_BWD
+  hipLaunchKernelGGL(kern, dim3(nb, ntens), dim3(nt), lds_bytes, st, a);
   int rc = launch_status();
   if (rc != MDATTN_OK) return rc;
   // columns: [q: dw (, db)] [k: dw (, db)], each N wide
@@ -588,7 +696,11 @@ extern "C" int mdattn_norm_rope_perhead_bwd(void* stream, const void* q_in, cons
   const int lpr = D / 8, groups = 256 / lpr;
   const int64_t rows = (int64_t)B * S * H;
   const int64_t ncols = 4 * (int64_t)D;
-  const int nb = partial_rows((rows + groups - 1) / groups, ncols, workspace_floats);
+  const int lds = groups * 4 * D * (int)sizeof(float);  // 32 KB for every supported D
+  void (*kern)(NormRopeBwdHeadArgs) = lpr == 8 ? norm_rope_perhead_bwd_kernel<8> : lpr == 16 ? norm_rope_perhead_bwd_kernel<16> : norm_rope_perhead_bwd_kernel<32>;
+  static ResidentCache resident[3];
+  const int nb = partial_rows((rows + groups - 1) / groups, ncols, workspace_floats,
+                              resident_blocks(resident[lpr == 8 ? 0 : lpr == 16 ? 1 : 2], reinterpret_cast<const void*>(kern), 256, lds));
   if (nb < 1) return MDATTN_E_BADARG;
 
   NormRopeBwdHeadArgs a;
@@ -603,12 +715,8 @@ extern "C" int mdattn_norm_rope_perhead_bwd(void* stream, const void* q_in, cons
   a.in_sb = in_strides->batch; a.in_ss = in_strides->seq; a.in_sh = in_strides->head;
   a.dx_sb = dx_strides->batch; a.dx_ss = dx_strides->seq; a.dx_sh = dx_strides->head;
   a.g_sb = g_strides->batch; a.g_ss = g_strides->seq; a.g_sh = g_strides->head;
-  dim3 grid(nb), block(256);
   hipStream_t st = (hipStream_t)stream;
-  const int lds = groups * 4 * D * (int)sizeof(float);  // 32 KB for every supported D
-  if (lpr == 8) hipLaunchKernelGGL((norm_rope_perhead_bwd_kernel<8>), grid, block, lds, st, a);
-  else if (lpr == 16) hipLaunchKernelGGL((norm_rope_perhead_bwd_kernel<16>), grid, block, lds, st, a);
-  else hipLaunchKernelGGL((norm_rope_perhead_bwd_kernel<32>), grid, block, lds, st, a);
+  hipLaunchKernelGGL(kern, dim3(nb), dim3(256), lds, st, a);
   int rc = launch_status();
   if (rc != MDATTN_OK) return rc;
   // columns: [q image][q text][k image][k text], each D wide; outputs that do not exist are skipped
@@ -635,7 +743,11 @@ extern "C" int mdattn_norm_rope_rows_bwd(void* stream, const void* x_in, int x_i
       dx_stride_seq % in_mult || dx_stride_seq < N || !strides_ok(g_strides, 8))
     return MDATTN_E_ALIGN;
   if (g_strides->head < D) return MDATTN_E_BADARG;
-  const int nb = partial_rows(ntok, N, workspace_floats);
+  const bool two = N / 16 > 256;
+  void (*kern)(NormRopeBwdRowsArgs) = x_is_f32 ? (two ? norm_rope_rows_bwd_kernel<2, true> : norm_rope_rows_bwd_kernel<1, true>)
+                                               : (two ? norm_rope_rows_bwd_kernel<2, false> : norm_rope_rows_bwd_kernel<1, false>);
+  static ResidentCache resident[2][2];
+  const int nb = partial_rows(ntok, N, workspace_floats, resident_blocks(resident[x_is_f32 ? 1 : 0][two ? 1 : 0], reinterpret_cast<const void*>(kern), 256, 0));
   if (nb < 1) return MDATTN_E_BADARG;
   NormRopeBwdRowsArgs a;
   a.x_in = x_in; a.g = (const __bf16*)g; a.dx = dx; a.w = w; a.cos = cos; a.sin = sin; a.part = workspace;
@@ -643,16 +755,8 @@ extern "C" int mdattn_norm_rope_rows_bwd(void* stream, const void* x_in, int x_i
   a.eps = eps; a.inv_n = 1.0f / (float)N;
   a.in_sb = in_stride_batch; a.in_ss = in_stride_seq; a.dx_sb = dx_stride_batch; a.dx_ss = dx_stride_seq;
   a.g_sb = g_strides->batch; a.g_ss = g_strides->seq; a.g_sh = g_strides->head;
-  dim3 grid(nb), block(256);
   hipStream_t st = (hipStream_t)stream;
-  const bool two = N / 16 > 256;
-  if (x_is_f32) {
-    if (two) hipLaunchKernelGGL((norm_rope_rows_bwd_kernel<2, true>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((norm_rope_rows_bwd_kernel<1, true>), grid, block, 0, st, a);
-  } else {
-    if (two) hipLaunchKernelGGL((norm_rope_rows_bwd_kernel<2, false>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((norm_rope_rows_bwd_kernel<1, false>), grid, block, 0, st, a);
-  }
+  hipLaunchKernelGGL(kern, dim3(nb), dim3(256), 0, st, a);
   int rc = launch_status();
   if (rc != MDATTN_OK) return rc;
   return launch_colsum(st, workspace, nb, (int)N, (int)N, dw, nullptr, nullptr, nullptr);
