@@ -275,8 +275,8 @@ int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, float* scal
  * bf16 out; lse as above.  Requires D == 128, or D == 64 (LTX-2's audio stream).
  * When scale * log2(e) * q_scale * k_scale is a power of two (see mdattn_quant_e4m3: premul, pow2_scale, and
  * scale = ln 2 here) the logit scale is applied inside the MFMAs and the softmax needs no multiply; the scales are
- * read on the device, so nothing has to be declared: two instances of the kernel are launched and the one whose
- * case it is not returns at once.
+ * read on the device, so nothing has to be declared: the one kernel that is launched holds both code paths and every
+ * wave takes the branch that the scales call for.
  *   softmax_mode  MDATTN_FP8_SOFTMAX_EXP2: P = e4m3(exp2(.)), the row sum over the unrounded P; lse is the exact
  *                 logsumexp of the quantised logits (usable as a partial for mdattn_merge).
  *                 MDATTN_FP8_SOFTMAX_BYTE_GRID: in the power-of-two case only (otherwise as EXP2), P is formed without
@@ -298,9 +298,10 @@ int mdattn_fwd_fp8(void* stream, const void* q8, const void* k8, const void* v8,
 /*
  * mdattn_fwd_fp8 with the additive per-key bias of mdattn_fwd_bf16_bias (a key padding mask,
  * models/attention_flax.py:1926-1939): logits = scale * q.k (de-quantised) + key_bias[b, key]; rows without any kept
- * key give out = 0 and lse = -inf.  The bias joins the products before the multiply per logit, so this entry point
- * always runs the exact-exponential softmax with that multiply, whatever the scales (MDATTN_FP8_SOFTMAX_EXP2
- * semantics).  key_bias as for mdattn_fwd_bf16_bias.
+ * key give out = 0 and lse = -inf.  Always the exact-exponential softmax (MDATTN_FP8_SOFTMAX_EXP2 semantics), on the
+ * path without a multiply per logit when the scales allow it, as for mdattn_fwd_fp8.  The tile's bias values travel
+ * with the K/V tile, and key tiles whose bias is all zero (all but the last few, for a padding mask) skip the bias
+ * arithmetic: a masked call costs a few per cent over an unmasked one.  key_bias as for mdattn_fwd_bf16_bias.
  */
 int mdattn_fwd_fp8_bias(void* stream, const void* q8, const void* k8, const void* v8, void* out, float* lse,
                         int B, int H, int Sq, int Skv, int D,

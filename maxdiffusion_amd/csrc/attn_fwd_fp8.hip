@@ -3,25 +3,35 @@
 //
 // Same decomposition as the bf16 kernel, on v_mfma_f32_32x32x64_f8f6f4 (K = 64 per instruction, twice
 // the bf16 rate):
-//   workgroup  = NW waves x 32 query rows; keys walked in tiles of 64, double-buffered in LDS with the
-//                next tile's global loads in flight in registers.
-//   S^T = K.Q^T  two 32-key blocks per tile, two MFMAs each (d = 0..63, 64..127).  A = K rows from LDS
-//                (row stride 144 B), B = the wave's Q fragment, resident in registers.  A and B use the
-//                same k-slot order, so a lane simply holds 32 contiguous bytes of its row.
-//   softmax      in f32 on the 32 logits a lane holds for its query row; q_scale*k_scale*scale*log2(e)
-//                is folded into the exp2 argument.  P is kept 2^4 above the usual normalisation
-//                (reference point = a row maximum - 4) so that e4m3's normal range [2^-6, 448] covers
-//                probabilities down to 2^-10 of the row max; the reference point only moves when
-//                some P may have passed 2^8, which the partial row sums reveal (no row maximum in the
-//                hot path).  The row sum uses the f32 P.
+//   workgroup  = NW waves x 32 query rows, three workgroups per CU (three waves per SIMD overlap each other's MFMA
+//                and softmax phases); keys walked in tiles of 64 through a 3-slot LDS ring filled by direct
+//                global->LDS loads (no staging registers), the loads of tile t+2 issued at the top of iteration t.
+//   S^T = K.Q^T  two 32-key blocks per tile, two MFMAs each (d = 0..63, 64..127).  A = K rows from LDS (unpadded
+//                rows of head_dim bytes, 16-byte chunks XOR-permuted by the row), B = the wave's Q fragment,
+//                resident in registers.  A and B use the same k-slot order, so a lane simply holds 32 contiguous
+//                bytes of its row.
+//   softmax      in f32 on the logits a lane holds for its query row, against a per-row reference point that is not
+//                the running maximum: it moves (cold branch: tile maximum - kPOff = 3, so that e4m3's normal range
+//                covers probabilities down to 2^-9 of the maximum) only when a lane's partial sum of P over the
+//                tile passes 448, e4m3's largest value.  MODE 0: q_scale*k_scale*scale*log2(e) folded into the
+//                exp2 argument, one multiply-add per logit.  MODE 1 (that product is a power of two): the scale
+//                rides in the MFMAs' block-scale operand and the chains start at minus the reference, P is one
+//                exp2 away.  MODE 2: no exponentials either (see kCodeOne).  Which of MODE 0 and MODE 1/2 applies
+//                depends on scales that live in device memory: one kernel holds both bodies and takes a
+//                wave-uniform branch on the scales it reads.
 //   O^T += V^T.P^T  one MFMA per 32-wide slab of d with all 64 keys of the tile as K.  P goes from the
 //                accumulator layout to the B operand by the e4m3 convert alone (operand byte s = value
 //                s%16 of block s/16).  V^T comes from the row-major V tile through ds_read_b64_tr_b8:
 //                within 16 lanes, lane i receives as byte e the element i%8 of the 8-byte chunk whose
 //                address lane 2e + i/8 supplies, so each lane points at one key row and one 8-byte
-//                column chunk, and every lane ends up with 8 keys of its own d.  The V tile has no row
-//                padding (128 B rows); its 8-byte chunks are XOR-swizzled by row bits 1 and 3, which
-//                makes the 8 rows x 32 B a half-wave reads hit 64 distinct banks.
+//                column chunk, and every lane ends up with 8 keys of its own d.  The V tile's 16-byte chunks are
+//                XOR-permuted by row bits 1 and 3, which makes the 8 rows x 32 B a half-wave reads hit 64
+//                distinct banks.
+//   key bias     (BIAS) the tile's 64 bias values ride through the LDS ring with the tile (a register load inside
+//                the loop would be waited for in issue order, behind the loads of the tile after next); tiles whose
+//                bias is all zero (every tile but the last few, for a padding mask) skip the bias code.  The bias
+//                joins the logits right after the MFMAs: divided by the logit scale in MODE 0 (the multiply per
+//                logit then carries it), in log2 units in MODE 1.
 //   epilogue     O * v_scale / l, bf16; lse = ln2 * (reference + log2 l).
 #include <type_traits>
 
@@ -70,19 +80,18 @@ struct Fp8Args {
 
 // Register budget: three waves per SIMD (<= 168 VGPRs); four at head dim 64 (<= 128 VGPRs, 24 KB of LDS: 1-4 % faster).  The kernel is bound by the vector ALU (softmax)
 // and by latencies a single wave cannot hide, so the third wave per SIMD is worth more than registers.
-// BIAS (MODE 0 only): an additive per-key bias (a key padding mask) joins the raw products right after the MFMAs,
-// divided by the logit scale so that the multiply per logit carries it; this instance serves every kind of scale.
-template <int NW, int MODE, bool BIAS = false, int HD = 128>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 64 ? 4 : 3, HD == 64 ? 4 : 3))) void attn_fwd_fp8_kernel(Fp8Args a) {
-  static_assert(!BIAS || MODE == 0, "the key bias lives in the path with a multiply per logit");
+// BIAS (MODE 0 and 1): an additive per-key bias (a key padding mask), see the header.
+template <int NW, int MODE, bool BIAS, int HD>
+__device__ __forceinline__ void fp8_body(const Fp8Args& a, const float c, char* smem8) {
+  static_assert(!BIAS || MODE != 2, "the key bias keeps exact exponentials");
   static_assert(HD == 128 || HD == 64, "head dim");
   constexpr int kKS8 = HD, kVS8 = HD;                 // row strides in LDS, bytes
-  constexpr int kStage8 = kBN8 * kKS8 + kBN8 * kVS8;  // bytes per LDS stage
+  constexpr int kTiles8 = kBN8 * kKS8 + kBN8 * kVS8;  // the K and the V tile of a stage
+  constexpr int kStage8 = kTiles8 + (BIAS ? 4 * kBN8 : 0);  // bytes per LDS stage; BIAS: + the tile's 64 bias values (f32)
   constexpr int NJ = HD / 64;                         // QK MFMAs (K = 64) per 32-key block
   constexpr int NSL = HD / 32;                        // 32-wide slabs of d = O accumulators
   constexpr bool PRE = MODE != 0;    // the logit scale is a power of two and rides in the MFMAs' block scale
   constexpr bool CODE = MODE == 2;   // ... and P is formed without exp2: see kCodeOne
-  extern __shared__ __attribute__((aligned(16))) char smem8[];
   constexpr int NT = NW * 64;
   constexpr int BM = NW * 32;
 
@@ -101,17 +110,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
   const uint8_t* vp = a.v + b * a.v_sb + h * a.v_sh;
   const int q0 = qt * BM + wave * 32;
   const int nt = (a.Skv + kBN8 - 1) / kBN8;
-  const float c = a.c * a.q_scale[0] * a.k_scale[0];
-  // The scales live in device memory, so the host cannot know which of the two instances of this kernel applies:
-  // it launches both, and the one whose case this is not ends here.
-  if constexpr (!BIAS) {
-    const unsigned cbits = __float_as_uint(c);
-    const bool c_pow2 = (cbits & 0x007FFFFFu) == 0u && cbits > 0x00800000u && cbits < 0x7F000000u;
-    if (c_pow2 != PRE) return;
-  }
-  [[maybe_unused]] const float* bias_row = BIAS ? a.bias + b * a.bias_sb + 4 * hh : nullptr;
-  [[maybe_unused]] const float bias_mul = kLog2e / c;            // natural-log bias -> units of the raw products
-  [[maybe_unused]] const int bias_cols = (a.Skv + 31) / 32 * 32;  // entries the caller's bias rows are sure to hold
+  [[maybe_unused]] const float* bias_row = BIAS ? a.bias + b * a.bias_sb : nullptr;
+  [[maybe_unused]] const float bias_mul = PRE ? kLog2e : kLog2e / c;  // natural-log bias -> log2 units (MODE 1) or units of the raw products
+  [[maybe_unused]] const int bias_cols = (a.Skv + 31) / 32 * 32;      // entries the caller's bias rows are sure to hold
 
   // ---- Q fragments: lane (row l32, half hh) holds bytes 64*j + 32*hh .. +31 of its row
   i32x8 qf[NJ];
@@ -149,6 +150,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
   auto dma = [&](int slot, int kt) __attribute__((always_inline)) {
     const unsigned Ks = smem_addr + (unsigned)(slot * kStage8);
     const unsigned Vs = Ks + kBN8 * kKS8;
+    if constexpr (BIAS) {
+      // every wave fetches the same 64 values to the same place (one load more per wave and tile, counted in the loop's
+      // s_waitcnt); the ring runs up to two tiles past the end, and a tile may reach past the padded bias row
+      int col = (kt < nt ? kt : nt - 1) * kBN8 + lane;
+      col = col < bias_cols ? col : bias_cols - 1;
+      lds_dma4(bias_row, (unsigned)col * 4u, Ks + kTiles8);
+    }
     if (kt * kBN8 + kBN8 <= a.Skv) {
       const uint8_t* kt0 = kp + (int64_t)(kt * kBN8 + RPI * wave) * a.k_ss;
       const uint8_t* vt0 = vp + (int64_t)(kt * kBN8 + RPI * wave) * a.v_ss;
@@ -180,6 +188,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
   // multiply.  The reference then starts at 0 and the first tile always takes the branch that sets it.
   const int sexp = (int)(__float_as_uint(c) >> 23) + (CODE ? 3 : 0);  // E8M0 code of c (of 8 c when the logits come in code units)
   float ref = PRE ? 0.f : -1e30f, l = 0.f;           // reference point of P (log2 units), per-lane partial row sum
+  [[maybe_unused]] bool fresh = true;                // PRE with a key bias: the row has not met a finite logit yet
   f32x16 negref;
 #pragma unroll
   for (int i = 0; i < 16; ++i) negref[i] = CODE ? kCodeOne : 0.f;
@@ -205,6 +214,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
 
   auto tile = [&](int t, int slot, auto masked) __attribute__((always_inline)) {
     const char* Ks = smem8 + slot * kStage8;
+    // A key padding mask is zero on all but the last tiles: lane l looks at the bias of key l of the tile, and a tile
+    // without any non-zero bias (one LDS read, one compare, one wave-uniform branch per block) skips the bias code.
+    [[maybe_unused]] bool has_bias = false;
+    if constexpr (BIAS) has_bias = __builtin_amdgcn_ballot_w64(reinterpret_cast<const float*>(Ks + kTiles8)[lane] != 0.f) != 0;
     // ---- S^T = K.Q^T for one 32-key block
     auto qk = [&](f32x16& S, int blk, const char* Kb) __attribute__((always_inline)) {
       i32x8 kf[NJ];
@@ -224,14 +237,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
         S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[0], qf[0], z, 0, 0, 0, 0, 0, 0);
         if constexpr (NJ == 2) S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[1], qf[1], S, 0, 0, 0, 0, 0, 0);
       }
-      if constexpr (BIAS) {
-        if (t * kBN8 + 32 * blk < bias_cols) {  // a block wholly past the keys (last tile) is masked below anyway
+      // the keys' bias joins the products after the MFMAs: in log2 units (MODE 1) or divided by the logit scale (MODE 0)
+      if (BIAS && has_bias) {
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const f32x4 bv = *reinterpret_cast<const f32x4*>(bias_row + t * kBN8 + 32 * blk + 8 * g);
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 bv = *reinterpret_cast<const f32x4*>(Kb + kTiles8 + (32 * blk + 8 * g + 4 * hh) * 4);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) S[4 * g + e] = __builtin_fmaf(bv[e], bias_mul, S[4 * g + e]);
-          }
+          for (int e = 0; e < 4; ++e) S[4 * g + e] = __builtin_fmaf(bv[e], bias_mul, S[4 * g + e]);
         }
       }
       if constexpr (decltype(masked)::value) {
@@ -296,7 +308,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
     };
     if constexpr (CODE) ls = rowsum();
     // (a byte 0x7F decodes to NaN and poisons the sum; bytes above it are caught by their top bit)
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(ls <= (CODE ? 3.0e38f : kPTrig)) || (hib & 0x80808080u) != 0u) != 0 || (PRE && t == 0), 0)) {
+    // PRE: a row's reference is set by the first tile in which it meets a finite logit: tile 0, unless a key bias
+    // excludes all of that tile's keys (`fresh` then stays set and the row tries again on the next tile)
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(ls <= (CODE ? 3.0e38f : kPTrig)) || (hib & 0x80808080u) != 0u || (PRE && BIAS && fresh)) != 0 ||
+                         (PRE && !BIAS && t == 0), 0)) {
       // The logits are recomputed rather than kept: the hot path holds them only while it forms P.
       int zero = 0;
       asm volatile("" : "+s"(zero));  // an address the compiler cannot match with the hot path's: no reuse of its logits
@@ -312,8 +327,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
       if constexpr (PRE) {  // the logits are relative to the old reference (MODE 2: in code units, 56 at the reference)
         mx = xhalf_max(mx);
         if constexpr (CODE) mx = (mx - kCodeOne) * 0.125f;
-        const float dm = t == 0 ? mx - kPOff : fmaxf(mx - kPOff, 0.f);
-        alpha = t == 0 ? 0.f : __builtin_amdgcn_exp2f(-dm);
+        float dm;
+        if constexpr (BIAS) {
+          const bool first = fresh && mx > -INFINITY;
+          dm = first ? mx - kPOff : (fresh ? 0.f : fmaxf(mx - kPOff, 0.f));
+          alpha = fresh ? 0.f : __builtin_amdgcn_exp2f(-dm);
+          fresh = fresh && !first;
+        } else {
+          dm = t == 0 ? mx - kPOff : fmaxf(mx - kPOff, 0.f);
+          alpha = t == 0 ? 0.f : __builtin_amdgcn_exp2f(-dm);
+        }
         ref += dm;
 #pragma unroll
         for (int i = 0; i < 16; ++i) negref[i] = CODE ? kCodeOne - 8.0f * ref : -ref;
@@ -361,7 +384,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
   dma(1, 1);
   int slot = 0, fill = 2;
   for (int t = 0; t < nt - 1; ++t) {
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * GPW));  // vmcnt: this wave's share of tile t has landed
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * GPW + (BIAS ? 1 : 0)));  // vmcnt: this wave's share of tile t has landed
     __syncthreads();                                  // ... and everyone's; slot `fill` (tile t-1) is free
     dma(fill, t + 2);
     tile(t, slot, std::false_type{});
@@ -392,26 +415,33 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
   }
 }
 
+// One kernel for both kinds of logit scale: c = scale * log2(e) * q_scale * k_scale is read on the device (the scales
+// are results of the quantiser, the host never sees them), and every wave takes the same branch: the body without a
+// multiply per logit when c is a power of two (PMODE 1: exp2; 2: the byte-grid softmax), the general body otherwise.
+// The two bodies are never live together, so the kernel's register count is the larger of the two.
+template <int NW, int PMODE, bool BIAS, int HD>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 64 ? 4 : 3, HD == 64 ? 4 : 3))) void attn_fwd_fp8_kernel(Fp8Args a) {
+  extern __shared__ __attribute__((aligned(16))) char smem8[];
+  const float c = a.c * a.q_scale[0] * a.k_scale[0];
+  const unsigned cbits = __builtin_amdgcn_readfirstlane(__float_as_uint(c));
+  const bool c_pow2 = (cbits & 0x007FFFFFu) == 0u && cbits > 0x00800000u && cbits < 0x7F000000u;
+  if (c_pow2) fp8_body<NW, PMODE, BIAS, HD>(a, c, smem8);
+  else fp8_body<NW, 0, BIAS, HD>(a, c, smem8);
+}
+
 template <int NW, int HD>
 int launch_fwd8(hipStream_t st, Fp8Args a, int B, int softmax_mode) {
   constexpr int BM = NW * 32;
-  constexpr int lds_bytes = kSlots8 * 2 * kBN8 * HD;
+  const int lds_bytes = kSlots8 * (2 * kBN8 * HD + (a.bias ? 4 * kBN8 : 0));
   a.nqt = (a.Sq + BM - 1) / BM;
   const int64_t total = (int64_t)B * a.H * a.nqt;
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
-  if (a.bias) {  // one instance for every kind of scale
-    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 0, true, HD>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
-    return launch_status();
-  }
-  hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 0, false, HD>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
-  // Power-of-two logit scale (the instance above then returns at once, this one otherwise): exp2, or the
-  // exponential-free softmax when the caller asked for it.
-  if (softmax_mode == MDATTN_FP8_SOFTMAX_BYTE_GRID)
-    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 2, false, HD>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
-  else
-    hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 1, false, HD>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  const dim3 grid(a.chunk * 8), block(NW * 64);
+  if (a.bias) hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 1, true, HD>), grid, block, lds_bytes, st, a);
+  else if (softmax_mode == MDATTN_FP8_SOFTMAX_BYTE_GRID) hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 2, false, HD>), grid, block, lds_bytes, st, a);
+  else hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 1, false, HD>), grid, block, lds_bytes, st, a);
   return launch_status();
 }
 
