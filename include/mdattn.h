@@ -6,7 +6,12 @@
  *   - only enqueues work on that stream: never synchronises, never allocates,
  *   - validates its arguments on the host BEFORE any launch and returns a negative
  *     MDATTN_E_* code instead of launching a kernel that could fault,
- *   - is re-entrant (no mutable global state).
+ *   - is re-entrant: no mutable global state, with two documented exceptions -- the test hook
+ *     mdattn_set_fwd_schedule (a process-wide switch read once per forward call) and the static scratch of
+ *     mdattn_bwd_bf16_static (shared by all calls on one GPU).  Once-initialised read-only caches (a kernel's LDS
+ *     opt-in, the resident-workgroup count of a persistent kernel, the scratch address) are filled under atomics.
+ *   - reads and clears a HIP error left pending on the calling thread before each launch, so that MDATTN_E_LAUNCH
+ *     always means one of its own launches was rejected.
  * All pointers are device pointers owned by the caller.  "bf16" tensors hold
  * bfloat16 bit patterns (uint16_t); the innermost (head_dim) axis is contiguous and
  * every other axis is described by an element stride, so [B,S,H,D] (= the
@@ -354,6 +359,11 @@ int mdattn_bwd_bf16_bias(void* stream, const void* q, const void* k, const void*
  * allocates nothing and frees nothing.  All calls on one GPU share the array: calls that may overlap on one GPU (two
  * streams, two threads) race on it and must be serialised by the caller; calls on different GPUs are independent.
  * The device that `stream` belongs to must be the current device.
+ * Warm-up: the first use on a device looks up the array's device address (hipGetSymbolAddress), which can make the
+ * runtime load the library's code object and place the 32 MiB array -- not something to happen under graph capture or
+ * in a no-allocation region.  Call mdattn_bwd_static_max_floats() once per device beforehand, with that device
+ * current (it performs the lookup), or make one un-captured call of the entry point; after that the entry point only
+ * enqueues kernels.
  */
 #define MDATTN_BWD_STATIC_MAX_FLOATS (8 * 1024 * 1024)
 int64_t mdattn_bwd_static_max_floats(void);

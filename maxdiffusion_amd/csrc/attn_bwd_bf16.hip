@@ -474,7 +474,7 @@ int launch_bwd_as(hipStream_t st, BwdArgs a, int B) {
   else kern = attn_bwd_kernel<MODE, HD, BIAS, PRE>;
   static LdsOptIn opted;
   if (lds_opt_in(opted, reinterpret_cast<const void*>(kern), lds_bytes) != MDATTN_OK) return MDATTN_E_LAUNCH;
-  hipLaunchKernelGGL(kern, dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  MDATTN_LAUNCH(kern, dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   return launch_status();
 }
 
@@ -536,7 +536,7 @@ static int bwd_run(hipStream_t st, const void* q, const void* k, const void* v, 
   float* delta = workspace + (int64_t)B * H * Sp;
   const int64_t rows = (int64_t)B * H * Sp;
   if ((rows + 15) / 16 > 0x7FFFFFFF || rows >= (1 << 29)) return MDATTN_E_UNSUPPORTED;  // delta - lse2 as a 32-bit byte offset
-  hipLaunchKernelGGL(bwd_prep_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const __bf16*)out,
+  MDATTN_LAUNCH(bwd_prep_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const __bf16*)out,
                      (const __bf16*)dout, lse, lse2, delta, H, Sq, Sp, D, rows, o_strides->batch, o_strides->seq, o_strides->head);
   if (launch_status() != MDATTN_OK) return MDATTN_E_LAUNCH;
 
@@ -618,7 +618,13 @@ float* scratch_on_current_device() {
 }
 }  // namespace
 
-extern "C" int64_t mdattn_bwd_static_max_floats(void) { return MDATTN_BWD_STATIC_MAX_FLOATS; }
+// Also the warm-up of the static entry point: looks the array's address up for the current device (which may make the
+// runtime load the code object and place the array), so that a later mdattn_bwd_bf16_static call -- under graph
+// capture, say -- finds it resolved.  Without a GPU the lookup fails quietly.
+extern "C" int64_t mdattn_bwd_static_max_floats(void) {
+  (void)scratch_on_current_device();
+  return MDATTN_BWD_STATIC_MAX_FLOATS;
+}
 
 extern "C" int mdattn_bwd_bf16_static(void* stream, const void* q, const void* k, const void* v, const void* out,
                                       const void* dout, const float* lse, void* dq, void* dk, void* dv,

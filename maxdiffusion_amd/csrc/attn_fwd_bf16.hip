@@ -686,8 +686,8 @@ static int launch_flat(hipStream_t st, AttnArgs a, int B) {
   // scale * log2(e) == 1 (to f32 round-off): the caller folded the factor into q; the logits need no multiply.
   // With a key bias the logits are touched after the MFMAs anyway, so that variant keeps its FMA.
   const bool pre = !BIAS && a.c > 1.0f - 1e-6f && a.c < 1.0f + 1e-6f;
-  if (pre) hipLaunchKernelGGL((attn_fwd_bf16_flat_kernel<NW, BIAS, HD, !BIAS>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
-  else hipLaunchKernelGGL((attn_fwd_bf16_flat_kernel<NW, BIAS, HD, false>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  if (pre) MDATTN_LAUNCH((attn_fwd_bf16_flat_kernel<NW, BIAS, HD, !BIAS>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  else MDATTN_LAUNCH((attn_fwd_bf16_flat_kernel<NW, BIAS, HD, false>), dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   return launch_status();
 }
 
@@ -705,7 +705,7 @@ static int launch_fwd(hipStream_t st, AttnArgs a, int B) {
   auto kern = pre ? attn_fwd_bf16_kernel<NW, true> : attn_fwd_bf16_kernel<NW, false>;
   static LdsOptIn opted[2];
   if (lds_opt_in(opted[pre], reinterpret_cast<const void*>(kern), lds_bytes) != MDATTN_OK) return MDATTN_E_LAUNCH;
-  hipLaunchKernelGGL(kern, dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
+  MDATTN_LAUNCH(kern, dim3(a.chunk * 8), dim3(NW * 64), lds_bytes, st, a);
   return launch_status();
 }
 

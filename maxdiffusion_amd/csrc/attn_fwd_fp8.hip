@@ -439,9 +439,9 @@ int launch_fwd8(hipStream_t st, Fp8Args a, int B, int softmax_mode) {
   a.total = (int)total;
   a.chunk = (a.total + 7) / 8;
   const dim3 grid(a.chunk * 8), block(NW * 64);
-  if (a.bias) hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 1, true, HD>), grid, block, lds_bytes, st, a);
-  else if (softmax_mode == MDATTN_FP8_SOFTMAX_BYTE_GRID) hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 2, false, HD>), grid, block, lds_bytes, st, a);
-  else hipLaunchKernelGGL((attn_fwd_fp8_kernel<NW, 1, false, HD>), grid, block, lds_bytes, st, a);
+  if (a.bias) MDATTN_LAUNCH((attn_fwd_fp8_kernel<NW, 1, true, HD>), grid, block, lds_bytes, st, a);
+  else if (softmax_mode == MDATTN_FP8_SOFTMAX_BYTE_GRID) MDATTN_LAUNCH((attn_fwd_fp8_kernel<NW, 2, false, HD>), grid, block, lds_bytes, st, a);
+  else MDATTN_LAUNCH((attn_fwd_fp8_kernel<NW, 1, false, HD>), grid, block, lds_bytes, st, a);
   return launch_status();
 }
 

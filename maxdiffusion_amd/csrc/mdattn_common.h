@@ -124,6 +124,16 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 inline bool strides_ok(const mdattn_strides* s, int64_t mult) {
   return s && s->batch % mult == 0 && s->seq % mult == 0 && s->head % mult == 0 && s->seq > 0 && s->head > 0 && s->batch >= 0;
 }
+// Every kernel launch of the library goes through MDATTN_LAUNCH and is followed by launch_status().  hipGetLastError()
+// returns (and clears) the last error of ANY earlier HIP call on the calling thread, so an error that the caller's own
+// code left pending would otherwise surface here as MDATTN_E_LAUNCH of a launch that went fine: MDATTN_LAUNCH reads
+// the pending error first.  That clears it: a caller who wants to see its own sticky error has to read it before
+// calling into the library.
+#define MDATTN_LAUNCH(...)         \
+  do {                             \
+    (void)hipGetLastError();       \
+    hipLaunchKernelGGL(__VA_ARGS__); \
+  } while (0)
 inline int launch_status() { return hipGetLastError() == hipSuccess ? MDATTN_OK : MDATTN_E_LAUNCH; }
 
 // A kernel that needs more dynamic LDS than the default limit has to opt in with hipFuncSetAttribute, once per

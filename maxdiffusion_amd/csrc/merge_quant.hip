@@ -162,8 +162,8 @@ extern "C" int mdattn_merge(void* stream, float* o_run, float* lse_run, const vo
   hipStream_t st = (hipStream_t)stream;
 #define MDATTN_MERGE_CASE(L)                                                          \
   if (lpr == L) {                                                                     \
-    if (cur_is_f32) hipLaunchKernelGGL((merge_kernel<L, true>), grid, block, 0, st, a); \
-    else hipLaunchKernelGGL((merge_kernel<L, false>), grid, block, 0, st, a);           \
+    if (cur_is_f32) MDATTN_LAUNCH((merge_kernel<L, true>), grid, block, 0, st, a); \
+    else MDATTN_LAUNCH((merge_kernel<L, false>), grid, block, 0, st, a);           \
   }
   MDATTN_MERGE_CASE(8) MDATTN_MERGE_CASE(16) MDATTN_MERGE_CASE(32)
 #undef MDATTN_MERGE_CASE
@@ -176,7 +176,7 @@ extern "C" int mdattn_finalize(void* stream, const float* o_run, void* out_bf16,
   if (!aligned16(o_run) || !aligned16(out_bf16)) return MDATTN_E_ALIGN;
   const int64_t n8 = n / 8;
   const unsigned grid = (unsigned)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536);
-  hipLaunchKernelGGL(finalize_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const float4*)o_run, (uint4*)out_bf16, n8);
+  MDATTN_LAUNCH(finalize_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const float4*)o_run, (uint4*)out_bf16, n8);
   return launch_status();
 }
 
@@ -190,9 +190,11 @@ extern "C" int mdattn_quant_e4m3(void* stream, const void* x_bf16, void* x_fp8, 
   const int64_t n8 = n / 8, n16 = n / 16;
   const unsigned g1 = (unsigned)((n8 + 255) / 256 < 2048 ? (n8 + 255) / 256 : 2048);
   const unsigned g2 = (unsigned)((n16 + 255) / 256 < 16384 ? (n16 + 255) / 256 : 16384);
-  hipLaunchKernelGGL(zero2_kernel, dim3(1), dim3(64), 0, st, scale_out);
-  hipLaunchKernelGGL(absmax_kernel, dim3(g1), dim3(256), 0, st, (const uint4*)x_bf16, n8, (unsigned*)(scale_out + 1));
-  hipLaunchKernelGGL(quant_kernel, dim3(g2), dim3(256), 0, st, (const uint4*)x_bf16, (uint4*)x_fp8, n16, scale_out,
+  MDATTN_LAUNCH(zero2_kernel, dim3(1), dim3(64), 0, st, scale_out);
+  if (launch_status() != MDATTN_OK) return MDATTN_E_LAUNCH;
+  MDATTN_LAUNCH(absmax_kernel, dim3(g1), dim3(256), 0, st, (const uint4*)x_bf16, n8, (unsigned*)(scale_out + 1));
+  if (launch_status() != MDATTN_OK) return MDATTN_E_LAUNCH;
+  MDATTN_LAUNCH(quant_kernel, dim3(g2), dim3(256), 0, st, (const uint4*)x_bf16, (uint4*)x_fp8, n16, scale_out,
                      premul, pow2_scale);
   return launch_status();
 }
@@ -212,7 +214,7 @@ extern "C" int mdattn_key_mask_bias(void* stream, const void* keep, float* bias,
   if (!keep || !bias || B <= 0 || Skv <= 0 || bias_stride < Skv) return MDATTN_E_BADARG;
   if (B > 65535) return MDATTN_E_UNSUPPORTED;
   const unsigned gx = (unsigned)((bias_stride + 255) / 256 < 1024 ? (bias_stride + 255) / 256 : 1024);
-  hipLaunchKernelGGL(mdattn::key_mask_bias_kernel, dim3(gx, B), dim3(256), 0, (hipStream_t)stream,
+  MDATTN_LAUNCH(mdattn::key_mask_bias_kernel, dim3(gx, B), dim3(256), 0, (hipStream_t)stream,
                      (const uint8_t*)keep, bias, Skv, bias_stride, masked_value);
   return mdattn::launch_status();
 }

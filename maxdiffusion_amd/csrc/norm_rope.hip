@@ -384,10 +384,10 @@ extern "C" int mdattn_norm_rope_fullrow(void* stream, const void* q_in, const vo
   dim3 grid(S, B), block(256);
   hipStream_t st = (hipStream_t)stream;
   const int nchunks = (int)(N / 8);
-  if (nchunks <= 256) hipLaunchKernelGGL(norm_rope_fullrow_kernel<1>, grid, block, 0, st, a);
-  else if (nchunks <= 512) hipLaunchKernelGGL(norm_rope_fullrow_kernel<2>, grid, block, 0, st, a);
-  else if (nchunks <= 768) hipLaunchKernelGGL(norm_rope_fullrow_kernel<3>, grid, block, 0, st, a);
-  else hipLaunchKernelGGL(norm_rope_fullrow_kernel<4>, grid, block, 0, st, a);
+  if (nchunks <= 256) MDATTN_LAUNCH(norm_rope_fullrow_kernel<1>, grid, block, 0, st, a);
+  else if (nchunks <= 512) MDATTN_LAUNCH(norm_rope_fullrow_kernel<2>, grid, block, 0, st, a);
+  else if (nchunks <= 768) MDATTN_LAUNCH(norm_rope_fullrow_kernel<3>, grid, block, 0, st, a);
+  else MDATTN_LAUNCH(norm_rope_fullrow_kernel<4>, grid, block, 0, st, a);
   return launch_status();
 }
 
@@ -422,10 +422,10 @@ extern "C" int mdattn_norm_rope_qkv(void* stream, const void* qkv, const void* b
   dim3 grid(S, B), block(256);
   hipStream_t st = (hipStream_t)stream;
   const int nchunks = (int)(N / 8);
-  if (nchunks <= 256) hipLaunchKernelGGL((norm_rope_fullrow_kernel<1, true>), grid, block, 0, st, a);
-  else if (nchunks <= 512) hipLaunchKernelGGL((norm_rope_fullrow_kernel<2, true>), grid, block, 0, st, a);
-  else if (nchunks <= 768) hipLaunchKernelGGL((norm_rope_fullrow_kernel<3, true>), grid, block, 0, st, a);
-  else hipLaunchKernelGGL((norm_rope_fullrow_kernel<4, true>), grid, block, 0, st, a);
+  if (nchunks <= 256) MDATTN_LAUNCH((norm_rope_fullrow_kernel<1, true>), grid, block, 0, st, a);
+  else if (nchunks <= 512) MDATTN_LAUNCH((norm_rope_fullrow_kernel<2, true>), grid, block, 0, st, a);
+  else if (nchunks <= 768) MDATTN_LAUNCH((norm_rope_fullrow_kernel<3, true>), grid, block, 0, st, a);
+  else MDATTN_LAUNCH((norm_rope_fullrow_kernel<4, true>), grid, block, 0, st, a);
   return launch_status();
 }
 
@@ -460,9 +460,9 @@ extern "C" int mdattn_norm_rope_perhead(void* stream, const void* q_in, const vo
   if (nblocks > 0x7FFFFFFF) return MDATTN_E_UNSUPPORTED;
   dim3 grid((unsigned)nblocks), block(256);
   hipStream_t st = (hipStream_t)stream;
-  if (lpr == 8) hipLaunchKernelGGL((norm_rope_perhead_kernel<8, RPT>), grid, block, 0, st, a);
-  else if (lpr == 16) hipLaunchKernelGGL((norm_rope_perhead_kernel<16, RPT>), grid, block, 0, st, a);
-  else hipLaunchKernelGGL((norm_rope_perhead_kernel<32, RPT>), grid, block, 0, st, a);
+  if (lpr == 8) MDATTN_LAUNCH((norm_rope_perhead_kernel<8, RPT>), grid, block, 0, st, a);
+  else if (lpr == 16) MDATTN_LAUNCH((norm_rope_perhead_kernel<16, RPT>), grid, block, 0, st, a);
+  else MDATTN_LAUNCH((norm_rope_perhead_kernel<32, RPT>), grid, block, 0, st, a);
   return launch_status();
 }
 
@@ -489,11 +489,11 @@ extern "C" int mdattn_norm_rope_rows(void* stream, const void* x_in, int x_is_f3
   hipStream_t st = (hipStream_t)stream;
   const bool two = N / 16 > 256;
   if (x_is_f32) {
-    if (two) hipLaunchKernelGGL((norm_rope_rows_kernel<2, true>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((norm_rope_rows_kernel<1, true>), grid, block, 0, st, a);
+    if (two) MDATTN_LAUNCH((norm_rope_rows_kernel<2, true>), grid, block, 0, st, a);
+    else MDATTN_LAUNCH((norm_rope_rows_kernel<1, true>), grid, block, 0, st, a);
   } else {
-    if (two) hipLaunchKernelGGL((norm_rope_rows_kernel<2, false>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((norm_rope_rows_kernel<1, false>), grid, block, 0, st, a);
+    if (two) MDATTN_LAUNCH((norm_rope_rows_kernel<2, false>), grid, block, 0, st, a);
+    else MDATTN_LAUNCH((norm_rope_rows_kernel<1, false>), grid, block, 0, st, a);
   }
   return launch_status();
 }

@@ -589,7 +589,7 @@ static int launch_colsum(hipStream_t st, const float* part, int nb, int ncols, i
   ColsumArgs c;
   c.part = part; c.nb = nb; c.ncols = ncols; c.seglen = seglen;
   c.outs[0] = o0; c.outs[1] = o1; c.outs[2] = o2; c.outs[3] = o3;
-  hipLaunchKernelGGL(colsum_kernel, dim3((ncols + 63) / 64), dim3(256), 0, st, c);
+  MDATTN_LAUNCH(colsum_kernel, dim3((ncols + 63) / 64), dim3(256), 0, st, c);
   return launch_status();
 }
 
@@ -666,7 +666,7 @@ extern "C" int mdattn_norm_rope_fullrow_bwd(void* stream, const void* q_in, cons
   a.in_sb = in_stride_batch; a.in_ss = in_stride_seq; a.dx_sb = dx_stride_batch; a.dx_ss = dx_stride_seq;
   a.g_sb = g_strides->batch; a.g_ss = g_strides->seq; a.g_sh = g_strides->head;
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(kern, dim3(nb, ntens), dim3(nt), lds_bytes, st, a);
+  MDATTN_LAUNCH(kern, dim3(nb, ntens), dim3(nt), lds_bytes, st, a);
   int rc = launch_status();
   if (rc != MDATTN_OK) return rc;
   // columns: [q: dw (, db)] [k: dw (, db)], each N wide
@@ -716,7 +716,7 @@ extern "C" int mdattn_norm_rope_perhead_bwd(void* stream, const void* q_in, cons
   a.dx_sb = dx_strides->batch; a.dx_ss = dx_strides->seq; a.dx_sh = dx_strides->head;
   a.g_sb = g_strides->batch; a.g_ss = g_strides->seq; a.g_sh = g_strides->head;
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(kern, dim3(nb), dim3(256), lds, st, a);
+  MDATTN_LAUNCH(kern, dim3(nb), dim3(256), lds, st, a);
   int rc = launch_status();
   if (rc != MDATTN_OK) return rc;
   // columns: [q image][q text][k image][k text], each D wide; outputs that do not exist are skipped
@@ -756,7 +756,7 @@ extern "C" int mdattn_norm_rope_rows_bwd(void* stream, const void* x_in, int x_i
   a.in_sb = in_stride_batch; a.in_ss = in_stride_seq; a.dx_sb = dx_stride_batch; a.dx_ss = dx_stride_seq;
   a.g_sb = g_strides->batch; a.g_ss = g_strides->seq; a.g_sh = g_strides->head;
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(kern, dim3(nb), dim3(256), 0, st, a);
+  MDATTN_LAUNCH(kern, dim3(nb), dim3(256), 0, st, a);
   int rc = launch_status();
   if (rc != MDATTN_OK) return rc;
   return launch_colsum(st, workspace, nb, (int)N, (int)N, dw, nullptr, nullptr, nullptr);

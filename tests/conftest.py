@@ -38,7 +38,13 @@ def _current_library():
   tree (a test that loaded a stale library first would keep it mapped for the whole session)."""
   from maxdiffusion_amd import build
 
-  build.ensure_built()
+  try:
+    build.ensure_built()
+  except RuntimeError as e:
+    if "hipcc not found" not in str(e):
+      raise
+    # no compiler on this machine: tests of the oracle and of the host logic still run; the `lib` fixture below
+    # fails the ones that need the library
 
 
 @pytest.fixture(scope="session")

@@ -23,8 +23,10 @@ def _case(dev, lib, B, H, sq, skv, seed, layout="bshd"):
   want = ops.flash_attention_backward(q, k, v, out, dout, lse)  # mdattn_bwd_bf16, workspace from torch
   # everything the static entry point touches exists before the call: it must not allocate
   got = tuple(torch.full_like(t, float("nan")) for t in (q, k, v))
+  assert lib.mdattn_bwd_static_max_floats() == 8 * 1024 * 1024  # the documented warm-up: resolves the array's address
   torch.cuda.synchronize()
   before = torch.cuda.memory_allocated(dev)
+  free_before = torch.cuda.mem_get_info(dev)[0]  # the driver's own count: sees a hipMalloc that torch's allocator would not
   P, S = ctypes.c_void_p, _lib.Strides
   st = lambda t: ctypes.byref(S(t.stride(0), t.stride(1), t.stride(2)))
   rc = lib.mdattn_bwd_bf16_static(
@@ -34,6 +36,7 @@ def _case(dev, lib, B, H, sq, skv, seed, layout="bshd"):
   assert rc == _lib.E_OK, _lib.strerror(rc)
   torch.cuda.synchronize()
   assert torch.cuda.memory_allocated(dev) == before
+  assert torch.cuda.mem_get_info(dev)[0] == free_before
   for name, g, w in zip(("dq", "dk", "dv"), got, want):
     assert bool(torch.isfinite(g.float()).all()), f"{name} B={B} H={H} Sq={sq} Skv={skv}"
     assert torch.equal(g, w), f"{name} differs from mdattn_bwd_bf16: B={B} H={H} Sq={sq} Skv={skv} {layout}"
