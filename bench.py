@@ -65,6 +65,17 @@ def main():
   ap.add_argument("--fused-qkv", action="store_true",
                   help="also time the prologue over a fused q|k|v projection output [1,S,3*H*D] with the three Linear biases "
                        "(mdattn_norm_rope_qkv, in place), outside the timed steps; reported as `roofline_norm_rope_qkv`")
+  ap.add_argument("--key-split", type=int, default=0, metavar="F",
+                  help="also time the self-attention with its key range split F ways inside ONE launch (the splits ride as batch "
+                       "entries: q with batch stride 0, k / v viewed [F, Skv/F, H, D]), followed by F merges and the finalize; "
+                       "reported as `key_split` beside the headline.  Skv must be divisible by F")
+  ap.add_argument("--hbm-probe", action="store_true",
+                  help="also time the runtime's own streaming kernels on tensors of the prologue's size (copy, two-input add, "
+                       "fill, sum): what this machine's memory system gives plain kernels, for scale; reported as `hbm_probe`")
+  ap.add_argument("--atomic-probe", action="store_true",
+                  help="with --with-backward: also time the f32 atomic adds that a single-pass backward (five matrix products "
+                       "instead of seven) would issue for dq at this shape, per wave and reduced per workgroup; reported inside "
+                       "the `backward` object")
   ap.add_argument("--with-backward", action="store_true",
                   help="also time the backward pass (dq, dk, dv) of the workload's attention, outside the timed steps; "
                        "reported as a `backward` object beside the headline")
@@ -269,9 +280,93 @@ def main():
     # the five matrix products of the backward pass: S, dP, dV, dK, dQ (the two passes execute seven: S and dP are formed in both)
     bfl = 2.5 * O.attention_flops(1, H, S, Skv, D)
     btf = bfl / (bms * 1e-3) / 1e12
+    probe = None
+    if args.atomic_probe:
+      import ctypes
+
+      fn = _lib.load().mdattn_probe_dq_atomics
+      fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 5
+      fn.restype = ctypes.c_int
+      dqf = torch.zeros((H, S // 32 * 32, D), dtype=torch.float32, device=dev)
+      probe = {}
+      for per_wave, key in ((1, "per_wave_ms"), (0, "per_workgroup_ms")):
+        run = lambda: _lib.check(fn(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), ctypes.c_void_p(dqf.data_ptr()), H, S, Skv, D, per_wave), "probe")
+        run()
+        e0, e1 = ev(), ev()
+        e0.record()
+        for _ in range(3):
+          run()
+        e1.record()
+        torch.cuda.synchronize()
+        probe[key] = e0.elapsed_time(e1) / 3
+      n_add = H * (Skv // 256) * (S // 32) * 32 * D  # per workgroup and query tile: one 32 x D partial
+      probe.update({"atomic_adds_per_workgroup_mode": n_add, "atomic_adds_per_wave_mode": 8 * n_add,
+                    "note": "f32 atomic adds of the dq partials of a key-outer single pass, nothing else in the launch"})
+      del dqf
     backward = {"Sq": S, "Skv": Skv, "ms": bms, "TFLOP/s": btf, "bound": "mfma", "peak": 2500.0, "frac": btf / 2500.0,
                 "frac_executed": btf * 7.0 / 5.0 / 2500.0,
                 "flop_counted": bfl, "note": "5 matrix products counted, 7 executed (two atomic-free passes: dq; dk and dv)"}
+    if probe:
+      backward["single_pass_dq_atomics_probe"] = probe
+
+  # the key range split F ways inside one launch, then merged: what a key split could buy small grids
+  key_split = None
+  if args.key_split > 1 and not fp8 and ring == 1:
+    F = args.key_split
+    if Skv % F:
+      raise SystemExit(f"--key-split: Skv={Skv} is not divisible by {F}")
+    qn, kn = prologue()
+    one = lambda: ops.flash_attention(qn, kn, v, scale=att_scale, return_lse=True)
+    qv, kv, vv = qn.expand(F, S, H, D), kn.reshape(F, Skv // F, H, D), v.reshape(F, Skv // F, H, D)
+
+    def split_attention():
+      return ops.flash_attention(qv, kv, vv, scale=att_scale, return_lse=True)
+
+    def split_step():
+      o, l = split_attention()
+      o_run, l_run = ops.new_merge_state(1, S, H, D, dev)
+      for i in range(F):
+        ops.merge_partial(o_run, l_run, o[i:i + 1], l[i:i + 1])
+      return ops.finalize(o_run)
+
+    def timed(fn, n=reps):
+      for _ in range(2):
+        fn()
+      e0, e1 = ev(), ev()
+      e0.record()
+      for _ in range(n):
+        fn()
+      e1.record()
+      torch.cuda.synchronize()
+      return e0.elapsed_time(e1) / n
+
+    ks_one, ks_att, ks_all = timed(one), timed(split_attention), timed(split_step)
+    err = float((split_step().float() - one()[0].float()).abs().max())
+    key_split = {"splits": F, "one_launch_ms": ks_one, "split_attention_launch_ms": ks_att, "split_with_merges_and_finalize_ms": ks_all,
+                 "max_abs_diff_vs_one_launch": err}
+
+  hbm_probe = None
+  if args.hbm_probe:
+    n = S * H * D * 2  # elements of q and k together
+    a_, b_ = torch.randn(n, device=dev).to(torch.bfloat16), torch.randn(n, device=dev).to(torch.bfloat16)
+    c_ = torch.empty_like(a_)
+
+    def rate(fn, nbytes):
+      for _ in range(3):
+        fn()
+      e0, e1 = ev(), ev()
+      e0.record()
+      for _ in range(reps):
+        fn()
+      e1.record()
+      torch.cuda.synchronize()
+      return nbytes / (e0.elapsed_time(e1) / reps * 1e-3) / 1e9
+
+    hbm_probe = {"unit": "GB/s", "bytes_per_tensor": n * 2,
+                 "copy_1r_1w": rate(lambda: c_.copy_(a_), 2 * n * 2), "add_2r_1w": rate(lambda: torch.add(a_, b_, out=c_), 3 * n * 2),
+                 "fill_1w": rate(lambda: c_.zero_(), n * 2), "sum_1r": rate(lambda: a_.sum(), n * 2),
+                 "note": "torch's own elementwise / reduction kernels on bf16 tensors of the prologue's size"}
+    del a_, b_, c_
 
   # backward of the prologue (input and weight gradients from the saved inputs and the gradients of its outputs)
   prologue_backward = None
@@ -357,6 +452,10 @@ def main():
     out["backward"] = backward
   if prologue_backward:
     out["prologue_backward"] = prologue_backward
+  if key_split:
+    out["key_split"] = key_split
+  if hbm_probe:
+    out["hbm_probe"] = hbm_probe
   if args.cpu_rows > 0:
     out["cpu_baseline"] = cpu_baseline(w, args.cpu_rows)
   print(json.dumps(out), flush=True)

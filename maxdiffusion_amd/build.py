@@ -16,7 +16,7 @@ INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "libmdattn.so")
 FFI_LIB_PATH = os.path.join(PKG_DIR, "libmdattn_ffi.so")
 
-SOURCES = ["mdattn_api.hip", "norm_rope.hip", "norm_rope_bwd.hip", "attn_fwd_bf16.hip", "attn_fwd_fp8.hip", "attn_bwd_bf16.hip", "merge_quant.hip",
+SOURCES = ["mdattn_api.hip", "norm_rope.hip", "norm_rope_bwd.hip", "attn_fwd_bf16.hip", "attn_fwd_fp8.hip", "attn_bwd_bf16.hip", "merge_quant.hip", "probes.hip",
            # the bodies of the XLA custom-call handlers on plain structs (no XLA header): part of the library
            os.path.join("ffi", "mdattn_marshal.cc")]
 

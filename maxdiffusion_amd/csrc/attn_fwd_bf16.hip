@@ -442,16 +442,22 @@ template <int NW, bool BIAS, int HD, bool PRE>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 64 ? 4 : 3, HD == 64 ? 4 : 3))) void attn_fwd_bf16_flat_kernel(AttnArgs a) {
   constexpr int NJ = HD / 16;                                    // QK MFMAs per 32-key tile
   constexpr int ND = HD / 32;                                    // 32-wide slabs of d = O accumulators
-  constexpr int KTILE = HD == 128 ? kKTileS : kTS * 64;          // elements
-  constexpr int TILES = HD == 128 ? kStageS : 2 * kTS * 64;      // the K and the V tile of a slot
+  // Head dim 64: 64-key tiles (two 32-key blocks per ring slot, the LDS of a 32-key tile at head dim 128) in a 2-slot
+  // ring: half the barriers and tile bookkeeping per key of a kernel whose softmax already outweighs its MFMAs.
+  constexpr int TS = HD == 128 ? kTS : 64;                       // keys per tile
+  constexpr int NB = TS / 32;                                    // 32-key blocks per tile
+  constexpr int SLOTS = HD == 128 ? kSlotsS : 2;
+  constexpr int KTILE = HD == 128 ? kKTileS : TS * 64;           // elements
+  constexpr int QTILE = HD == 128 ? kKTileS : 32 * 64;           // a wave's 32 Q rows, staged like a K tile
+  constexpr int TILES = HD == 128 ? kStageS : 2 * TS * 64;       // the K and the V tile of a slot
   // with a bias, a slot also carries the tile's 32 bias values (f32) behind its tiles: a register load inside the
   // loop would be waited for in issue order, i.e. behind the loads of the tile after next
-  constexpr int STAGE = TILES + (BIAS ? 4 * kTS : 0);  // 64 floats: one per lane of the load that brings them
+  constexpr int STAGE = TILES + (BIAS ? 128 : 0);  // 64 floats: one per lane of the load that brings them
   constexpr int RPI = HD == 128 ? 4 : 8;                          // rows one load instruction fills
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
   constexpr int BM = NW * 32;
-  constexpr int GPW = (kTS / RPI) / NW;  // row groups per wave, tile and tensor
+  constexpr int GPW = (TS / RPI) / NW;  // row groups per wave, tile and tensor
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -467,11 +473,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
   const __bf16* kp = a.k + b * a.k_sb + h * a.k_sh;
   const __bf16* vp = a.v + b * a.v_sb + h * a.v_sh;
   const int q0 = qt * BM + wave * 32;
-  const int nt = (a.Skv + kTS - 1) / kTS;
+  const int nt = (a.Skv + TS - 1) / TS;
   const float c = a.c;
   // with a bias the logits are brought to log2 units (scale folded, bias added) right after the MFMAs
   const float cs = BIAS ? 1.0f : c;
   const float* bias_row = BIAS ? a.bias + b * a.bias_sb : nullptr;
+  [[maybe_unused]] const int bias_cols = (a.Skv + 31) / 32 * 32;  // entries the caller's bias rows are sure to hold
 
   bf16x8 qf[NJ];  // filled from LDS below: the wave's 32 Q rows arrive like a K tile, by whole-row loads
 
@@ -489,10 +496,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
     const unsigned Vs = Ks + KTILE * 2u;
     // every wave fetches the same values to the same place (a load more per wave and tile, counted in the loop's
     // s_waitcnt): lane l and lane l + 32 the bias of key l of the tile; the ring runs up to two tiles past the end
-    if constexpr (BIAS) lds_dma4(bias_row + (kt < nt ? kt : nt - 1) * kTS, (unsigned)l32 * 4u, Ks + TILES * 2u);
-    if (kt * kTS + kTS <= a.Skv) {
-      const __bf16* kt0 = kp + (int64_t)(kt * kTS + RPI * wave) * a.k_ss;
-      const __bf16* vt0 = vp + (int64_t)(kt * kTS + RPI * wave) * a.v_ss;
+    if constexpr (BIAS) {  // (a 64-key tile may reach past the padded bias row, whose length is a multiple of 32)
+      int col = (kt < nt ? kt : nt - 1) * TS + (TS == 64 ? lane : l32);
+      col = col < bias_cols ? col : bias_cols - 1;
+      lds_dma4(bias_row, (unsigned)col * 4u, Ks + TILES * 2u);
+    }
+    if (kt * TS + TS <= a.Skv) {
+      const __bf16* kt0 = kp + (int64_t)(kt * TS + RPI * wave) * a.k_ss;
+      const __bf16* vt0 = vp + (int64_t)(kt * TS + RPI * wave) * a.v_ss;
 #pragma unroll
       for (int i = 0; i < GPW; ++i) {
         lds_dma16(kt0 + (int64_t)(RPI * NW * i) * a.k_ss, kofs, Ks + (unsigned)((wave + NW * i) * KGS) * 2u);
@@ -502,7 +513,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
 #pragma unroll
       for (int i = 0; i < GPW; ++i) {
         const int g = wave + NW * i;
-        int kk = kt * kTS + RPI * g + grow;
+        int kk = kt * TS + RPI * g + grow;
         kk = kk < a.Skv ? kk : a.Skv - 1;
         lds_dma16(kp + (int64_t)kk * a.k_ss + kcol, Ks + (unsigned)(g * KGS) * 2u);
         lds_dma16(vp + (int64_t)kk * a.v_ss + vcol, Vs + (unsigned)(g * VGS) * 2u);
@@ -545,6 +556,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
 
   auto tile = [&](int t, int slot, auto masked) __attribute__((always_inline)) {
     const __bf16* base = smem + slot * STAGE;
+#pragma unroll
+   for (int blk = 0; blk < NB; ++blk) {
+    constexpr int kBlk = 32 * 64;  // a 32-key block of a head-dim-64 tile: 32 rows of 64 elements, in K and in V
+    const bool first = t == 0 && blk == 0;
     // ---- S^T = K.Q^T: one chain of MFMAs; the other waves of the SIMD fill the gaps between them.  A wave in an
     // MFMA phase issues ahead of the SIMD's waves in their softmax phase (1-2 % on short key sequences).
     __builtin_amdgcn_s_setprio(1);
@@ -553,19 +568,19 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
     for (int i = 0; i < 16; ++i) S[i] = 0.f;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + k_off[j]);
+      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + k_off[j] + blk * kBlk);
       S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[j], (PRE && j == 0) ? negm : S, 0, 0, 0);
     }
     if constexpr (BIAS) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const f32x4 bv = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(base + TILES) + 8 * g + 4 * hh);
+        const f32x4 bv = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(base + TILES) + 32 * blk + 8 * g + 4 * hh);
 #pragma unroll
         for (int e = 0; e < 4; ++e) S[4 * g + e] = __builtin_fmaf(S[4 * g + e], c, bv[e] * kLog2e);
       }
     }
     if constexpr (decltype(masked)::value) {
-      const int kv_base = t * kTS + 4 * hh;
+      const int kv_base = t * TS + 32 * blk + 4 * hh;
 #pragma unroll
       for (int i = 0; i < 16; ++i)
         if (kv_base + 8 * (i >> 2) + (i & 3) >= a.Skv) S[i] = -INFINITY;
@@ -591,15 +606,15 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
       return lsum;
     };
     float lsum = soft(mc);
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lsum <= kTrig)) != 0 || (PRE && t == 0), 0)) {
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lsum <= kTrig)) != 0 || (PRE && first), 0)) {
       float mloc = S[0];
 #pragma unroll
       for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, S[i]);
       mloc = xhalf_max(mloc);
       float alpha;
       if constexpr (PRE) {  // S holds logits minus the old reference: shift them and the chains' start value
-        const float dm = t == 0 ? mloc : fmaxf(mloc, 0.f);
-        alpha = t == 0 ? 0.f : __builtin_amdgcn_exp2f(-dm);
+        const float dm = first ? mloc : fmaxf(mloc, 0.f);
+        alpha = first ? 0.f : __builtin_amdgcn_exp2f(-dm);
         mc += dm;
 #pragma unroll
         for (int i = 0; i < 16; ++i) { S[i] -= dm; negm[i] = -mc; }
@@ -622,10 +637,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
     // ---- O^T += V^T.P^T
 #pragma unroll
     for (int jv = 0; jv < 2 * ND; ++jv) {
-      const __bf16* vsrc = base + v_off[jv % ND] + (jv / ND) * kVH;
+      const __bf16* vsrc = base + v_off[jv % ND] + (jv / ND) * kVH + blk * kBlk;
       const bf16x8 vf = read_vt(vsrc, vsrc + kV8);
       O[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P[jv / ND], O[jv % ND], 0, 0, 0);
     }
+   }
   };
 
   // ---- Q fragments.  A lane's registers hold 16-byte pieces of ONE row, so loading them straight from global memory
@@ -635,29 +651,32 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
   // with the K fragment offsets.  Each wave stages and reads only its own rows.
   dma(0, 0);
   {
-    const unsigned Qs = smem_addr + (unsigned)(STAGE + wave * KTILE) * 2u;
+    const unsigned Qs = smem_addr + (unsigned)(STAGE + wave * QTILE) * 2u;
 #pragma unroll
-    for (int g = 0; g < kTS / RPI; ++g) {
+    for (int g = 0; g < 32 / RPI; ++g) {
       int row = q0 + RPI * g + grow;
       row = row < a.Sq ? row : a.Sq - 1;
       const int qcol = HD == 128 ? kcol : ((lane & 7) ^ ((4 * (g & 1) + (grow >> 1)) & 7)) * 8;
       lds_dma16(qp + (int64_t)row * a.q_ss + qcol, Qs + (unsigned)(g * KGS) * 2u);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the wave's own Q rows (and its share of tile 0) are in LDS
-    const __bf16* qs = smem + STAGE + wave * KTILE;
+    const __bf16* qs = smem + STAGE + wave * QTILE;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) qf[j] = *reinterpret_cast<const bf16x8*>(qs + k_off[j]);
   }
-  __syncthreads();  // every wave holds its fragments: the staging area is ring slots 1 and 2 again
-  dma(1, 1);
-  int slot = 0, fill = 2;
+  __syncthreads();  // every wave holds its fragments: the staging area is ring slots again
+  // SLOTS - 1 tiles are requested ahead of the one being worked on
+#pragma unroll
+  for (int i = 1; i < SLOTS - 1; ++i) dma(i, i);
+  int slot = 0, fill = SLOTS - 1;
   for (int t = 0; t < nt - 1; ++t) {
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * GPW + (BIAS ? 1 : 0)));  // vmcnt: this wave's share of tile t has landed
+    // vmcnt: this wave's share of tile t has landed (the SLOTS - 2 tiles requested after it may still be in flight)
+    __builtin_amdgcn_s_waitcnt(0x0F70 | ((SLOTS - 2) * (2 * GPW + (BIAS ? 1 : 0))));
     __syncthreads();                                  // ... and everyone's; slot `fill` (tile t-1) is free
-    dma(fill, t + 2);
+    dma(fill, t + SLOTS - 1);
     tile(t, slot, std::false_type{});
-    slot = slot == kSlotsS - 1 ? 0 : slot + 1;
-    fill = fill == kSlotsS - 1 ? 0 : fill + 1;
+    slot = slot == SLOTS - 1 ? 0 : slot + 1;
+    fill = fill == SLOTS - 1 ? 0 : fill + 1;
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
@@ -666,7 +685,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
   if (a.o_run) {  // ring step: merged into the f32 carry, row by row
     store_row<ND>(a, O, xhalf_sum(l), mc, b, h, q0 + l32, hh);
   } else {
-    static_assert(NW * 32 * (HD * 2 + 16) <= kSlotsS * STAGE * 2, "the output staging tiles must fit the ring's LDS");
+    static_assert(NW * 32 * (HD * 2 + 16) <= SLOTS * STAGE * 2, "the output staging tiles must fit the ring's LDS");
     __syncthreads();  // every wave has finished reading the ring: its LDS now stages the output tiles
     store_rows_through_lds<ND>(a, O, xhalf_sum(l), mc, b, h, q0, lane, smem_raw + wave * 32 * (HD * 2 + 16));
   }
@@ -676,8 +695,9 @@ template <int NW, bool BIAS, int HD = 128>
 static int launch_flat(hipStream_t st, AttnArgs a, int B) {
   constexpr int BM = NW * 32;
   // the ring, or ring slot 0 plus one K-shaped Q staging tile per wave, whichever is larger
-  constexpr int stage_el = (HD == 128 ? kStageS : 2 * kTS * 64) + (BIAS ? 4 * kTS : 0), ktile_el = HD == 128 ? kKTileS : kTS * 64;
-  constexpr int lds_bytes = (kSlotsS * stage_el > stage_el + NW * ktile_el ? kSlotsS * stage_el : stage_el + NW * ktile_el) * 2;
+  constexpr int slots = HD == 128 ? kSlotsS : 2;
+  constexpr int stage_el = (HD == 128 ? kStageS : 2 * 64 * 64) + (BIAS ? 128 : 0), qtile_el = HD == 128 ? kKTileS : 32 * 64;
+  constexpr int lds_bytes = (slots * stage_el > stage_el + NW * qtile_el ? slots * stage_el : stage_el + NW * qtile_el) * 2;
   a.nqt = (a.Sq + BM - 1) / BM;
   const int64_t total = (int64_t)B * a.H * a.nqt;
   if (total > (int64_t)0x7FFFFFF0) return MDATTN_E_UNSUPPORTED;
