@@ -254,29 +254,38 @@ def main():
     cross = {"Skv": w.cross_kv, "kernel_ms": cms, "TFLOP/s": cfl / (cms * 1e-3) / 1e12,
              "GB/s": (2 * S * H * D * 2 + 2 * w.cross_kv * H * D * 2 + H * S * 4) / (cms * 1e-3) / 1e9}
 
-  # backward of one attention call of the workload (one KV chunk for the ring shards), with the plain softmax scale
+  # backward of one attention call of the workload (one KV chunk for the ring shards), on the operands the training path
+  # hands it: q from the prologue with scale * log2(e) folded in (the configuration of the headline forward), and, for
+  # comparison, on plain q with the softmax scale as an argument
   backward = None
   if args.with_backward and not fp8:
     if D != 128:
       raise SystemExit("--with-backward: the backward kernels are built for head dim 128")
-    if w.norm == "fullrow":
-      qb, kb = ops.norm_rope_fullrow(q_in, k_in, wq, wk, cos, sin, H)
-    elif w.norm == "rows":
-      qb, kb = ops.norm_rope_rows(q_in, wq, cos, sin, heads=H, mode="interleaved"), ops.norm_rope_rows(k_in, wk, cos, sin, heads=H, mode="interleaved")
-    else:
-      qb, kb = ops.norm_rope_perhead(q4, k4, wq, wk, cos, sin)
     vb = v[:, :Skv]
-    ob, lb = ops.flash_attention(qb, kb, vb, scale=w.scale, return_lse=True)
     dout = randn(1, S, H, D)
-    for _ in range(2):
-      ops.flash_attention_backward(qb, kb, vb, ob, dout, lb, scale=w.scale)
-    e0, e1 = ev(), ev()
-    e0.record()
-    for _ in range(5):
-      ops.flash_attention_backward(qb, kb, vb, ob, dout, lb, scale=w.scale)
-    e1.record()
-    torch.cuda.synchronize()
-    bms = e0.elapsed_time(e1) / 5
+
+    def time_backward(qb, kb, sc):
+      ob, lb = ops.flash_attention(qb, kb, vb, scale=sc, return_lse=True)
+      for _ in range(2):
+        ops.flash_attention_backward(qb, kb, vb, ob, dout, lb, scale=sc)
+      e0, e1 = ev(), ev()
+      e0.record()
+      for _ in range(5):
+        ops.flash_attention_backward(qb, kb, vb, ob, dout, lb, scale=sc)
+      e1.record()
+      torch.cuda.synchronize()
+      return e0.elapsed_time(e1) / 5, (qb, kb, ob, lb)
+
+    qf, kf = prologue()
+    bms, (qb, kb, ob, lb) = time_backward(qf, kf[:, :Skv] if kf.shape[1] != Skv else kf, att_scale)
+    if w.norm == "fullrow":
+      qp, kp = ops.norm_rope_fullrow(q_in, k_in, wq, wk, cos, sin, H)
+    elif w.norm == "rows":
+      qp, kp = ops.norm_rope_rows(q_in, wq, cos, sin, heads=H, mode="interleaved"), ops.norm_rope_rows(k_in, wk, cos, sin, heads=H, mode="interleaved")
+    else:
+      qp, kp = ops.norm_rope_perhead(q4, k4, wq, wk, cos, sin)
+    bms_plain, _ = time_backward(qp, kp, w.scale)
+    del qp, kp
     # the five matrix products of the backward pass: S, dP, dV, dK, dQ (the two passes execute seven: S and dP are formed in both)
     bfl = 2.5 * O.attention_flops(1, H, S, Skv, D)
     btf = bfl / (bms * 1e-3) / 1e12
@@ -305,7 +314,9 @@ def main():
       del dqf
     backward = {"Sq": S, "Skv": Skv, "ms": bms, "TFLOP/s": btf, "bound": "mfma", "peak": 2500.0, "frac": btf / 2500.0,
                 "frac_executed": btf * 7.0 / 5.0 / 2500.0,
-                "flop_counted": bfl, "note": "5 matrix products counted, 7 executed (two atomic-free passes: dq; dk and dv)"}
+                "flop_counted": bfl, "ms_plain_scale": bms_plain,
+                "note": "5 matrix products counted, 7 executed (two atomic-free passes: dq; dk and dv); ms: q carries scale * log2(e) "
+                        "from the prologue, as in the headline forward; ms_plain_scale: plain q, softmax scale as an argument"}
     if probe:
       backward["single_pass_dq_atomics_probe"] = probe
 

@@ -109,8 +109,19 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
   constexpr int kBD = HD, kBGK = L::GA, kBGV = L::GB, kBTileA = L::TileA, kBTileB = L::TileB;
   constexpr int kBStage = bwd_slot_elems<MODE, HD, BIAS>();  // MODE 3: a second transposed-read tile (dout)
   constexpr bool AUX = MODE != 0 || BIAS;
-  constexpr int LA = MODE == 0 && HD == 128 ? 4 : 0;  // fragment look-ahead (the dk / dv pass has no registers for a window)
+#ifndef MDATTN_BWD_LA
+#define MDATTN_BWD_LA 4
+#endif
+  constexpr int LA = MODE == 0 && HD == 128 ? MDATTN_BWD_LA : 0;  // fragment look-ahead (the dk / dv pass has no registers for a window)
   static_assert(LA == 0 || (HAS2 && !BOTH && LA <= 2 * ND), "the window covers the three-product passes");
+#ifndef MDATTN_BWD_LA1
+#define MDATTN_BWD_LA1 2
+#endif
+#ifndef MDATTN_BWD_LA3
+#define MDATTN_BWD_LA3 6
+#endif
+  constexpr int LA3 = BOTH && HD == 128 ? (BIAS ? 4 : MDATTN_BWD_LA3) : 0;
+  constexpr int LA1 = BOTH && HD == 128 ? MDATTN_BWD_LA1 : 0;  // merged pass: look-ahead over the chains' row reads only
   constexpr int kBAux = L::Stage + (BOTH ? L::TileB : 0);    // where a slot's f32 values start (elements)
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -312,6 +323,17 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
         win[n % LA] = frag(n + LA);
         __builtin_amdgcn_sched_barrier(0);
       }
+    } else if constexpr (LA1 > 0) {  // a window over the row reads of the two chains only
+      bf16x8 w1[LA1];
+#pragma unroll
+      for (int n = 0; n < LA1; ++n) w1[n] = frag(n);
+#pragma unroll
+      for (int n = 0; n < 2 * NJ; ++n) {
+        if (n < NJ) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1[n % LA1], ef1[n % NJ], S, 0, 0, 0);
+        else dP = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1[n % LA1], ef2[n % NJ], dP, 0, 0, 0);
+        if (n + LA1 < 2 * NJ) w1[n % LA1] = frag(n + LA1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     } else {
 #pragma unroll
       for (int j = 0; j < NJ; ++j) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(j), ef1[j], S, 0, 0, 0);
@@ -370,6 +392,24 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
       W[hb] = __builtin_bit_cast(bf16x8, u32x4{wpk[0], wpk[1], wpk[2], wpk[3]});
       if constexpr (BOTH) Wp[hb] = __builtin_bit_cast(bf16x8, u32x4{ppk[0], ppk[1], ppk[2], ppk[3]});
     }
+    if constexpr (LA3 > 0) {  // merged pass: a window over the transposing reads of both accumulations
+      auto frag3 = [&](int n) __attribute__((always_inline)) {
+        const int jv = n >> 1;
+        const __bf16* src = base + v_off[jv % ND] + (jv / ND) * L::VH + ((n & 1) ? kBTileB : 0);
+        return read_vt_b(src, src + L::V8);
+      };
+      bf16x8 w3[LA3];
+#pragma unroll
+      for (int n = 0; n < LA3; ++n) w3[n] = frag3(n);
+#pragma unroll
+      for (int n = 0; n < 4 * ND; ++n) {
+        const int jv = n >> 1;
+        if (n & 1) acc2[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w3[n % LA3], Wp[jv / ND], acc2[jv % ND], 0, 0, 0);
+        else acc[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w3[n % LA3], W[jv / ND], acc[jv % ND], 0, 0, 0);
+        if (n + LA3 < 4 * ND) w3[n % LA3] = frag3(n + LA3);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else
 #pragma unroll
     for (int jv = 0; jv < 2 * ND; ++jv) {
       const __bf16* src = base + v_off[jv % ND] + (jv / ND) * L::VH;
@@ -482,7 +522,9 @@ int launch_bwd_as(hipStream_t st, BwdArgs a, int B) {
 // MFMAs in log2 units and take -lse as the chain's start value instead of a multiply-add each.
 template <int MODE, int HD, bool BIAS>
 int launch_bwd(hipStream_t st, const BwdArgs& a, int B) {
-  if constexpr (!BIAS) {
+  // (not for the merged pass at head dim 128: there the start values come from LDS, a read that the chain's first
+  // MFMA then waits for, and the multiply-add version measured 3 % faster)
+  if constexpr (!BIAS && !(MODE == 3 && HD == 128)) {
     if (a.c > 1.0f - 1e-6f && a.c < 1.0f + 1e-6f) return launch_bwd_as<MODE, HD, false, true>(st, a, B);
   }
   return launch_bwd_as<MODE, HD, BIAS, false>(st, a, B);
