@@ -259,8 +259,8 @@ def main():
   # comparison, on plain q with the softmax scale as an argument
   backward = None
   if args.with_backward and not fp8:
-    if D != 128:
-      raise SystemExit("--with-backward: the backward kernels are built for head dim 128")
+    if D not in (64, 128):
+      raise SystemExit("--with-backward: the backward kernels are built for head dims 64 and 128")
     vb = v[:, :Skv]
     dout = randn(1, S, H, D)
 
