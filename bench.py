@@ -76,6 +76,9 @@ def main():
                   help="with --with-backward: also time the f32 atomic adds that a single-pass backward (five matrix products "
                        "instead of seven) would issue for dq at this shape, per wave and reduced per workgroup; reported inside "
                        "the `backward` object")
+  ap.add_argument("--with-mask", action="store_true",
+                  help="fp8 workloads: also time the attention with a key padding mask (1000 keys excluded), beside the "
+                       "unmasked call with the same softmax, for power-of-two and for arbitrary scales; reported inside `roofline_exp2`")
   ap.add_argument("--with-backward", action="store_true",
                   help="also time the backward pass (dq, dk, dv) of the workload's attention, outside the timed steps; "
                        "reported as a `backward` object beside the headline")
@@ -233,6 +236,28 @@ def main():
     fp8_exp2 = {"bound": "mfma", "achieved": efl / (ems * 1e-3) / 1e12, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                 "frac": efl / (ems * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, "traffic": None, "kernel": "attn_fwd_fp8_kernel<4,1> (softmax_mode exp2)",
                 "kernel_ms": ems, "flop_per_launch": efl}
+    if args.with_mask:
+      # the same call with a key padding mask (the last 1000 keys excluded), with power-of-two scales and with
+      # arbitrary ones, each beside its unmasked twin
+      keep = torch.ones((1, Skv), dtype=torch.bool, device=dev)
+      keep[:, Skv - 1000:] = False
+      kb = ops.key_mask_bias(keep)
+
+      def t5(fn):
+        fn()
+        e0, e1 = ev(), ev()
+        e0.record()
+        for _ in range(5):
+          fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / 5
+
+      fp8_exp2["masked"] = {
+          "masked_keys": 1000, "unmasked_ms": ems,
+          "masked_ms": t5(lambda: ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=ops.FOLDED_SCALE, key_bias=kb)),
+          "unmasked_arbitrary_scale_ms": t5(lambda: ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=0.1)),
+          "masked_arbitrary_scale_ms": t5(lambda: ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=0.1, key_bias=kb))}
     del q8, k8, v8
 
   # configs[2] also names the cross-attention of the same Q against 512 text tokens (no RoPE): reported beside the
