@@ -23,7 +23,7 @@ from . import ops
 
 __all__ = [
     "KERNEL_REGISTRY", "register_kernel", "AttentionOp", "hip_flash_kernel", "hip_flash_fp8_kernel",
-    "hip_norm_rope", "hip_norm_rope_ltx2", "hip_flash_attention_autograd", "HIP_KERNEL_NAMES",
+    "hip_norm_rope", "hip_norm_rope_qkv", "hip_norm_rope_ltx2", "hip_flash_attention_autograd", "HIP_KERNEL_NAMES",
 ]
 
 KERNEL_REGISTRY = {}
@@ -193,6 +193,35 @@ class _HipNormRopeFullrow(torch.autograd.Function):
     return dq, dk, dwq.to(wq.dtype), (dwk.to(wk.dtype) if k is not None else None), None, None, None, None, None, None
 
 
+class _HipNormRopeQkv(torch.autograd.Function):
+  """The prologue over a fused q|k|v projection output with its HIP backward: the q | k blocks of the gradient buffer
+  are written by mdattn_norm_rope_fullrow_bwd (which also returns their bias gradients), v's block is its output
+  gradient (v only gains a bias, whose gradient is the token sum)."""
+
+  @staticmethod
+  def forward(ctx, qkv, bias, wq, wk, cos, sin, heads, eps, out_layout, q_mul):
+    q_out, k_out, v_out = ops.norm_rope_qkv(qkv, wq, wk, cos, sin, heads, bias, eps, out_layout, q_mul)
+    ctx.save_for_backward(qkv, bias, wq, wk, cos, sin)
+    ctx.cfg = (heads, eps, q_mul)
+    return q_out, k_out, v_out
+
+  @staticmethod
+  def backward(ctx, gq, gk, gv):
+    qkv, bias, wq, wk, cos, sin = ctx.saved_tensors
+    heads, eps, q_mul = ctx.cfg
+    b, s, n3 = qkv.shape
+    n = n3 // 3
+    dqkv = torch.empty((b, s, n3), dtype=torch.bfloat16, device=qkv.device)
+    res = ops.norm_rope_fullrow_backward(qkv[:, :, :n], qkv[:, :, n:2 * n], wq, wk, cos, sin, heads, gq.to(torch.bfloat16),
+                                         gk.to(torch.bfloat16), eps, q_mul, bias=None if bias is None else bias[:2 * n].contiguous(),
+                                         dq=dqkv[:, :, :n], dk=dqkv[:, :, n:2 * n])
+    dqkv[:, :, 2 * n:].unflatten(2, (heads, n // heads)).copy_(gv)
+    dbias = None
+    if bias is not None:
+      dbias = torch.cat([res[4], gv.float().sum(dim=(0, 1)).reshape(n)]).to(bias.dtype)
+    return dqkv, dbias, res[2].to(wq.dtype), res[3].to(wk.dtype), None, None, None, None, None, None
+
+
 class _HipNormRopePerhead(torch.autograd.Function):
   """The Flux prologue with its HIP backward (attention_flax.py:2989-3020)."""
 
@@ -235,6 +264,22 @@ def _norm_rope_rows(x, w, cos, sin, heads, mode, eps):
   if _wants_grad(x, w):
     return _HipNormRopeRows.apply(x, w, cos, sin, heads, mode, eps)
   return ops.norm_rope_rows(x, w, cos, sin, heads=heads, mode=mode, eps=eps)
+
+
+def hip_norm_rope_qkv(qkv, wq, wk, freqs_cis, heads: int, bias=None, eps: float = 1e-6, out_layout: str = "bshd",
+                      q_mul: float = 1.0, inplace: bool = False):
+  """The fused prologue over the output of ONE q|k|v projection `[B,S,3*H*D]` (the three projections of
+  attention_flax.py:2653-2663 run as one GEMM): bias adds, norm_q / norm_k, head split and rotation in one launch;
+  returns (q, k, v) logical [B,S,H,D] for `hip_flash`.  `bias`: the three Linear biases [3*H*D] when the GEMM ran
+  without them.  Differentiable with respect to qkv, bias and the norm weights; `inplace=True` (the fused buffer
+  itself becomes the three operands) is for inference only, since the backward needs the projection output."""
+  b, s, n3 = qkv.shape
+  cos, sin = _split_table(freqs_cis, s, n3 // 3 // heads)
+  if _wants_grad(qkv, wq, wk, bias):
+    if inplace:
+      raise ValueError("inplace=True overwrites the projection output that the backward pass needs")
+    return _HipNormRopeQkv.apply(qkv, bias, wq, wk, cos, sin, heads, eps, out_layout, q_mul)
+  return ops.norm_rope_qkv(qkv, wq, wk, cos, sin, heads, bias, eps, out_layout, q_mul, inplace)
 
 
 def hip_norm_rope_ltx2(query, key, norm_q_scale, norm_k_scale, heads: int, rotary_emb=None, k_rotary_emb=None,

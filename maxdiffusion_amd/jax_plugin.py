@@ -307,20 +307,54 @@ def hip_norm_rope_qkv(qkv, wq, wk, cos, sin, heads: int, bias=None, eps: float =
   """The prologue over the output of one fused q|k|v projection: qkv bf16 [B,S,3*H*D] (column blocks q | k | v);
   bias bf16 [3*H*D] or None (the Linear biases, when the GEMM ran without them) -> (q, k, v) [B,S,H,D] bf16.  Without
   a bias v is a slice of the fused buffer (XLA fuses the reshape; nothing is copied by the custom call).  One launch in
-  place of the three bias adds, norm_q / norm_k, _unflatten_heads and _apply_rope of attention_flax.py:2653-2677."""
+  place of the three bias adds, norm_q / norm_k, _unflatten_heads and _apply_rope of attention_flax.py:2653-2677.
+  Differentiable with respect to qkv, wq, wk and bias: the backward runs mdattn_norm_rope_fullrow_bwd on the q | k
+  blocks (with their biases) and passes v's gradient through (its bias gradient is the token sum)."""
   jax, jnp = _require_jax()
   b, s, n3 = qkv.shape
   n = n3 // 3
   d = n // heads
   rope, has_bias = cos is not None, bias is not None
   dummy = jnp.zeros((8,), jnp.float32)
-  out = jax.ShapeDtypeStruct((b, s, heads, d), jnp.bfloat16)
-  v_out = out if has_bias else jax.ShapeDtypeStruct((8,), jnp.bfloat16)
-  call = jax.ffi.ffi_call("mdattn_norm_rope_qkv", (out, out, v_out), vmap_method="sequential")
-  q_out, k_out, v_res = call(qkv, bias if has_bias else wq, wq, wk, cos if rope else dummy, sin if rope else dummy,
-                             eps=_f32(eps), q_mul=_f32(q_mul), heads=_i64(heads), rope=_i64(rope), has_bias=_i64(has_bias),
-                             has_v=_i64(has_bias))
-  return q_out, k_out, (v_res if has_bias else qkv[:, :, 2 * n:].reshape(b, s, heads, d))
+  cos_, sin_ = (cos, sin) if rope else (dummy, dummy)
+
+  def forward(qkv, wq, wk, bias_):
+    out = jax.ShapeDtypeStruct((b, s, heads, d), jnp.bfloat16)
+    v_out = out if has_bias else jax.ShapeDtypeStruct((8,), jnp.bfloat16)
+    call = jax.ffi.ffi_call("mdattn_norm_rope_qkv", (out, out, v_out), vmap_method="sequential")
+    q_out, k_out, v_res = call(qkv, bias_, wq, wk, cos_, sin_, eps=_f32(eps), q_mul=_f32(q_mul), heads=_i64(heads),
+                               rope=_i64(rope), has_bias=_i64(has_bias), has_v=_i64(has_bias))
+    return q_out, k_out, (v_res if has_bias else qkv[:, :, 2 * n:].reshape(b, s, heads, d))
+
+  @jax.custom_vjp
+  def prologue(qkv, wq, wk, bias_):
+    return forward(qkv, wq, wk, bias_)
+
+  def fwd(qkv, wq, wk, bias_):
+    return forward(qkv, wq, wk, bias_), (qkv, wq, wk, bias_)
+
+  def bwd(res, g):
+    qkv, wq, wk, bias_ = res
+    gq, gk, gv = g
+    cols = 2 * n * (2 if has_bias else 1)
+    rows = jax.ShapeDtypeStruct((b, s, n), jnp.bfloat16)
+    vec = jax.ShapeDtypeStruct((n,), jnp.float32)
+    results = (rows, rows, vec, vec, jax.ShapeDtypeStruct((2 * n,) if has_bias else (8,), jnp.float32),
+               jax.ShapeDtypeStruct((_partial_rows_floats(b * s, cols),), jnp.float32))
+    call = jax.ffi.ffi_call("mdattn_norm_rope_fullrow_bwd", results, vmap_method="sequential")
+    dq, dk, dwq, dwk, dbias_qk, _ = call(qkv[:, :, :n], qkv[:, :, n:2 * n], gq.astype(jnp.bfloat16), gk.astype(jnp.bfloat16), wq, wk,
+                                         cos_, sin_, bias_[:2 * n] if has_bias else wq, eps=_f32(eps), q_mul=_f32(q_mul),
+                                         heads=_i64(heads), rope=_i64(rope), has_k=_i64(1), has_bias=_i64(has_bias))
+    gv_rows = gv.astype(jnp.bfloat16).reshape(b, s, n)
+    dqkv = jnp.concatenate([dq, dk, gv_rows], axis=2)
+    if has_bias:
+      dbias = jnp.concatenate([dbias_qk, gv.astype(jnp.float32).sum(axis=(0, 1)).reshape(n)]).astype(bias_.dtype)
+    else:
+      dbias = jnp.zeros(bias_.shape, bias_.dtype)  # the stand-in operand (wq) receives a zero cotangent
+    return dqkv, dwq.astype(wq.dtype), dwk.astype(wk.dtype), dbias
+
+  prologue.defvjp(fwd, bwd)
+  return prologue(qkv, wq, wk, bias if has_bias else wq)
 
 
 def hip_norm_rope_perhead(q, k, wq, wk, cos, sin, eps: float = 1e-6, wq_txt=None, wk_txt=None, n_txt: int = 0, q_mul: float = 1.0):

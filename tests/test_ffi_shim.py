@@ -99,9 +99,14 @@ class _FakeArray:
   def transpose(self, *axes):
     return _FakeArray(tuple(self.shape[a] for a in axes), self.dtype)
 
-  def __getitem__(self, idx):  # slicing of the last axis only: x[:, :, a:]
-    a = idx[-1].start or 0
-    return _FakeArray(self.shape[:-1] + (self.shape[-1] - a,), self.dtype)
+  def __getitem__(self, idx):  # slicing of the last axis only: x[:, :, a:b], x[a:b]
+    sl = idx[-1] if isinstance(idx, tuple) else idx
+    a, b = sl.start or 0, self.shape[-1] if sl.stop is None else sl.stop
+    return _FakeArray(self.shape[:-1] + (b - a,), self.dtype)
+
+  def sum(self, axis):
+    axes = (axis,) if isinstance(axis, int) else tuple(axis)
+    return _FakeArray(tuple(n for i, n in enumerate(self.shape) if i not in axes), self.dtype)
 
 
 @pytest.fixture
@@ -115,6 +120,13 @@ def fake_jax(monkeypatch):
   for name in ("bfloat16", "float32", "bool_", "float8_e4m3fn"):
     setattr(jnp, name, name)
   jnp.zeros = lambda shape, dtype: _FakeArray(shape, dtype)
+
+  def concatenate(parts, axis=0):
+    shape = list(parts[0].shape)
+    shape[axis] = sum(x.shape[axis] for x in parts)
+    return _FakeArray(shape, parts[0].dtype)
+
+  jnp.concatenate = concatenate
   jax.ShapeDtypeStruct = lambda shape, dtype: _FakeArray(shape, dtype)
 
   def ffi_call(target, results, **kw):
@@ -135,7 +147,8 @@ def fake_jax(monkeypatch):
 
     def __call__(self, *a):  # run forward AND backward so that both custom calls are recorded
       out, res = self.fwd(*a)
-      self.bwd(res, out)
+      cot = self.bwd(res, out)
+      calls.append({"primals": tuple(x.shape for x in a), "cotangents": tuple(x.shape for x in cot)})
       return out
 
   jax.custom_vjp = _CustomVjp
@@ -198,7 +211,7 @@ def test_python_wrappers_follow_the_bind_lines(fake_jax):
       assert c["operands"][i].shape == c["results"][o].shape
   assert seen == set(P.FFI_TARGETS), sorted(set(P.FFI_TARGETS) - seen)
   # the text-token weights of Flux's double blocks reach the custom call (operands 4 and 5) with n_txt
-  ph = [c for c in fake_jax if c["target"] == "mdattn_norm_rope_perhead"][0]
+  ph = [c for c in fake_jax if c.get("target") == "mdattn_norm_rope_perhead"][0]
   assert ph["attrs"]["n_txt"] == 7 and ph["operands"][4] is wd and ph["operands"][5] is wd
   # the registry entries: rank-3 [B,S,H*D] in, [B,Sq,H*D] out, both names
   ctx = {"heads": H, "scale": 0.1, "attention_mask": None, "is_causal": False}
@@ -256,6 +269,27 @@ def test_registered_entry_is_differentiable(fake_jax):
   assert targets() == ["mdattn_norm_rope_fullrow", "mdattn_norm_rope_fullrow_bwd"]
   ws = [c for c in fake_jax if c.get("target") == "mdattn_norm_rope_fullrow_bwd"][0]["results"][-1]
   assert ws.shape == (min(B * S, P.NORM_ROPE_BWD_MAX_PARTIAL_ROWS) * 2 * H * D,)
+  # every custom_vjp returns one cotangent per primal, of the primal's shape
+  for c in fake_jax:
+    if "cotangents" in c:
+      assert c["cotangents"] == c["primals"], c
+  # the fused-projection form: its backward is the full-row backward on the q | k column blocks with their biases; the
+  # cotangent of the fused buffer is [dq | dk | gv], the bias's [dbias_q | dbias_k | sum of gv]
+  fake_jax.clear()
+  N = H * D
+  qkv, b3 = _FakeArray((B, S, 3 * N), bf), _FakeArray((3 * N,), bf)
+  assert [t.shape for t in P.hip_norm_rope_qkv(qkv, w, w, tab, tab, H, bias=b3)] == [(B, S, H, D)] * 3
+  assert targets() == ["mdattn_norm_rope_qkv", "mdattn_norm_rope_fullrow_bwd"]
+  bwd = [c for c in fake_jax if c.get("target") == "mdattn_norm_rope_fullrow_bwd"][0]
+  assert [o.shape for o in bwd["operands"][:4]] == [(B, S, N), (B, S, N), (B, S, H, D), (B, S, H, D)]
+  assert bwd["operands"][8].shape == (2 * N,) and bwd["attrs"]["has_bias"] == 1 and bwd["attrs"]["has_k"] == 1
+  assert [r.shape for r in bwd["results"]] == [(B, S, N), (B, S, N), (N,), (N,), (2 * N,), (min(B * S, 1024) * 4 * N,)]
+  vjp = [c for c in fake_jax if "cotangents" in c][0]
+  assert vjp["cotangents"] == ((B, S, 3 * N), (N,), (N,), (3 * N,)) == vjp["primals"]
+  fake_jax.clear()
+  P.hip_norm_rope_qkv(qkv, w, w, None, None, H)                      # no bias, norm only: v is a slice, workspace 2N columns
+  bwd = [c for c in fake_jax if c.get("target") == "mdattn_norm_rope_fullrow_bwd"][0]
+  assert bwd["attrs"]["has_bias"] == 0 and bwd["attrs"]["rope"] == 0 and bwd["results"][-1].shape == (min(B * S, 1024) * 2 * N,)
 
 
 def test_install_registers_both_kernel_names(fake_jax, monkeypatch, tmp_path):

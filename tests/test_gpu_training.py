@@ -76,6 +76,48 @@ def test_wan_prologue_and_attention_end_to_end(dev, rank4, masked):
     assert not v.grad[0, 40:].any()
 
 
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_fused_projection_prologue_and_attention_end_to_end(dev, with_bias):
+  """One fused q|k|v projection output [B,S,3*H*D] (the three Linears of attention_flax.py:2653-2663 as one GEMM, their
+  biases added by the prologue): gradients for the fused buffer, the biases and the norm weights."""
+  B, H, D, grid = 2, 3, 128, (2, 5, 9)
+  S, N = grid[0] * grid[1] * grid[2], 3 * 128
+  scale = D**-0.5
+  xqkv = O.normal_bf16((B, S, 3 * N), 0)
+  xb = (0.5 * O.normal_bf16((3 * N,), 1)).astype(np.float32)
+  wq, wk = O.norm_weight(N, 3), O.norm_weight(N, 4)
+  g = O.normal_bf16((B, S, N), 5)
+  cos, sin = O.wan_rope_table(grid, D)
+
+  qkv, tq, tk = (_leaf(x, dev) for x in (xqkv, wq, wk))
+  tb = _leaf(xb, dev) if with_bias else None
+  freqs = torch.complex(torch.from_numpy(cos), torch.from_numpy(sin)).to(dev)[None, None]
+  qn, kn, vn = A.hip_norm_rope_qkv(qkv, tq, tk, freqs, H, bias=tb)
+  assert qn.requires_grad and kn.requires_grad and vn.requires_grad
+  op = A.AttentionOp(attention_kernel="hip_flash", scale=scale, heads=H, dim_head=D)
+  out = op.apply_attention(qn.permute(0, 2, 1, 3), kn.permute(0, 2, 1, 3), vn.permute(0, 2, 1, 3))
+  (out.float() * to_dev_bf16(g, dev).float()).sum().backward()
+  with pytest.raises(ValueError, match="inplace"):
+    A.hip_norm_rope_qkv(qkv, tq, tk, freqs, H, bias=tb, inplace=True)
+
+  rqkv, rwq, rwk = (torch.tensor(x, dtype=torch.float64, requires_grad=True) for x in (xqkv, wq, wk))
+  xb16 = to_dev_bf16(xb, "cpu").double().numpy() if with_bias else np.zeros(3 * N)  # the bias as the kernel sees it: bf16
+  rb = torch.tensor(xb16, dtype=torch.float64, requires_grad=True)
+  u = rqkv + rb
+  yq = _rope_complex(torch.nn.functional.rms_norm(u[..., :N], (N,), rwq, eps=1e-6).reshape(B, S, H, D), cos, sin).transpose(1, 2)
+  yk = _rope_complex(torch.nn.functional.rms_norm(u[..., N:2 * N], (N,), rwk, eps=1e-6).reshape(B, S, H, D), cos, sin).transpose(1, 2)
+  ro = torch.nn.functional.scaled_dot_product_attention(yq, yk, u[..., 2 * N:].reshape(B, S, H, D).transpose(1, 2), scale=scale)
+  ro = ro.transpose(1, 2).reshape(B, S, N)
+  (ro * torch.tensor(g, dtype=torch.float64)).sum().backward()
+  _check(out, ro, "forward")
+  checks = [(qkv, rqkv, "d qkv"), (tq, rwq, "d wq"), (tk, rwk, "d wk")] + ([(tb, rb, "d bias")] if with_bias else [])
+  for got, ref, name in checks:
+    assert got.grad is not None and got.grad.dtype == got.dtype and got.grad.shape == got.shape
+    _check(got.grad, ref.grad, name)
+  for blk, name in ((slice(0, N), "q"), (slice(N, 2 * N), "k"), (slice(2 * N, 3 * N), "v")):  # each column block on its own
+    _check(qkv.grad[..., blk], rqkv.grad[..., blk], "d qkv block " + name)
+
+
 def test_flux_prologue_and_attention_end_to_end(dev):
   B, H, D, n_txt = 1, 4, 128, 7
   ids = O.flux_ids(n_txt, 5, 6)
