@@ -112,7 +112,9 @@ __device__ __forceinline__ void attn_bwd_body(const BwdArgs& a) {
 #ifndef MDATTN_BWD_LA
 #define MDATTN_BWD_LA 4
 #endif
-  constexpr int LA = MODE == 0 && HD == 128 ? MDATTN_BWD_LA : 0;  // fragment look-ahead (the dk / dv pass has no registers for a window)
+  // fragment look-ahead of the dq pass over its whole read stream (head dim 64, at three waves per SIMD, has room for
+  // two: 1 % on one machine, A/B); the merged pass windows its two MFMA phases separately, LA1 and LA3 below
+  constexpr int LA = MODE == 0 ? (HD == 128 ? MDATTN_BWD_LA : 2) : 0;
   static_assert(LA == 0 || (HAS2 && !BOTH && LA <= 2 * ND), "the window covers the three-product passes");
 #ifndef MDATTN_BWD_LA1
 #define MDATTN_BWD_LA1 2
