@@ -106,3 +106,47 @@ def test_captured_forward_and_static_backward_replay_to_the_eager_result(dev):
     assert torch.equal(out_c, out) and torch.equal(lse_c, lse), f"replay {rep}: forward differs"
     for i, (g, w) in enumerate(zip(grads, want)):
       assert torch.equal(g, w), f"replay {rep}: gradient {i} differs from the eager result"
+
+
+def test_captured_training_step_with_the_prologue_backward(dev):
+  """Prologue -> attention -> attention backward -> prologue backward in one captured graph: the backward entry points
+  enqueue kernels only (their workspaces are the caller's; the weight gradients come from a two-stage sum, no atomics,
+  so every replay reproduces the eager gradients bit for bit)."""
+  H, grid = 3, (2, 6, 11)
+  S, N = grid[0] * grid[1] * grid[2], 3 * 128
+  q, k, v, do = (to_dev_bf16(O.normal_bf16((2, S, N), s), dev) for s in (0, 1, 2, 5))
+  wq, wk = (to_dev_bf16(O.norm_weight(N, s), dev) for s in (3, 4))
+  cos, sin = (torch.from_numpy(t).to(dev) for t in O.wan_rope_table(grid, 128))
+  q_mul = ops.folded_q_mul(128)
+
+  def step():
+    qn, kn = ops.norm_rope_fullrow(q, k, wq, wk, cos, sin, H, q_mul=q_mul)
+    v4, do4 = v.view(2, S, H, 128), do.view(2, S, H, 128)
+    out, lse = ops.flash_attention(qn, kn, v4, scale=ops.FOLDED_SCALE, return_lse=True)
+    dqn, dkn, dv = ops.flash_attention_backward(qn, kn, v4, out, do4, lse, scale=ops.FOLDED_SCALE)
+    dq, dk, dwq, dwk = ops.norm_rope_fullrow_backward(q, k, wq, wk, cos, sin, H, dqn, dkn, q_mul=q_mul)
+    return out, dv, dq, dk, dwq, dwk
+
+  want = [t.clone() for t in step()]
+  torch.cuda.synchronize()
+  assert all(bool(torch.isfinite(t.float()).all()) and float(t.float().abs().max()) > 0 for t in want)
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):  # warm-up on the capture stream (also: the prologue backward sizes its grid on first use)
+    step()
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    captured = step()
+  for rep in range(3):
+    for t in captured:
+      t.fill_(float(rep) + 0.25)
+    # eager work between the replays: another prologue backward of a different shape
+    x = to_dev_bf16(O.normal_bf16((1, 37 + rep, N), 50 + rep), dev)
+    ops.norm_rope_fullrow_backward(x, x, wq, wk, None, None, H, x.view(1, -1, H, 128), x.view(1, -1, H, 128))
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    for i, (g, w) in enumerate(zip(captured, want)):
+      assert torch.equal(g, w), f"replay {rep}: output {i} differs from the eager result"
