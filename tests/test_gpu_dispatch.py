@@ -98,3 +98,37 @@ def test_reference_splash_test_shape_head_dim_64(dev):
   print(f"B=8 S=4096 H=10 D=64: ||hip_flash - f32 attention||_2 = {diff_norm:.3f}, max-abs {mx:.2e}", flush=True)
   assert diff_norm < 1.0 and mx <= 2e-2
   assert float(diff.norm() / ref.norm()) <= 1.5e-2
+
+
+def test_wan_i2v_cross_attention_block(dev):
+  """The Wan image-to-video cross-attention (attention_flax.py:2690-2777): the same tokens attend to the text states
+  (normed q, no mask) and to the image embeddings (raw q; 257 real image tokens padded to 384, the padding excluded by
+  encoder_attention_mask_img), and the two results are added.  Prologue hooks in norm-only mode, `hip_flash` twice,
+  against the f32 oracle with the padded keys removed."""
+  B, H, D, S, T, real, padded = 2, 4, 128, 300, 512, 257, 384
+  N = H * D
+  scale = D**-0.5
+  xq, xkt, xvt = O.normal_bf16((B, S, N), 0), O.normal_bf16((B, T, N), 1), O.normal_bf16((B, T, N), 2)
+  xki, xvi = O.normal_bf16((B, padded, N), 3), O.normal_bf16((B, padded, N), 4)
+  wq, wk, wki = O.norm_weight(N, 5), O.norm_weight(N, 6), O.norm_weight(N, 7)
+  q, kt, vt, ki, vi, tq, tk, tki = (to_dev_bf16(x, dev) for x in (xq, xkt, xvt, xki, xvi, wq, wk, wki))
+  keep = torch.zeros((B, padded), dtype=torch.bool, device=dev)
+  keep[:, :real] = True
+
+  op = A.AttentionOp(mesh=None, attention_kernel="hip_flash", scale=scale, heads=H, dim_head=D, dtype=torch.bfloat16)
+  q_text, _ = A.hip_norm_rope(q, None, tq, None, None, H)        # norm_q on the queries (norm only: no rotary table)
+  k_text, _ = A.hip_norm_rope(kt, None, tk, None, None, H)       # norm_k on the text keys
+  k_img, _ = A.hip_norm_rope(ki, None, tki, None, None, H)       # norm_added_k on the image keys
+  out_text = op.apply_attention(q_text.reshape(B, S, N), k_text.reshape(B, T, N), vt)
+  out_img = op.apply_attention(q, k_img.reshape(B, padded, N), vi, attention_mask=keep)
+  got = to_np(out_text + out_img)
+
+  for b in range(B):
+    hsd = lambda x: np.ascontiguousarray(x.reshape(x.shape[0], H, D).transpose(1, 0, 2))
+    qn = O.bf16_round(O.rmsnorm(xq[b], wq))
+    o_t, _ = O.attention(hsd(qn), hsd(O.bf16_round(O.rmsnorm(xkt[b], wk))), hsd(xvt[b]), scale)
+    o_i, _ = O.attention(hsd(xq[b]), hsd(O.bf16_round(O.rmsnorm(xki[b, :real], wki))), hsd(xvi[b, :real]), scale)
+    want = (O.bf16_round(o_t) + O.bf16_round(o_i)).transpose(1, 0, 2).reshape(S, N)
+    mx, mean = err_stats(got[b], want)
+    print(f"i2v cross-attention, batch {b}: max-abs {mx:.3e} mean-abs {mean:.3e} rel-l2 {rel_l2(got[b], want):.3e}")
+    assert mx <= 4e-2 and mean <= 4e-3 and rel_l2(got[b], want) <= 2e-2  # the sum of two bf16 outputs: twice the single-call bars
