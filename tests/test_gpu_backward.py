@@ -268,3 +268,33 @@ def test_backward_seeded_sweep_of_shapes_layouts_masks_and_scale_kinds(dev):
       rel, mx = float((g - r).norm()) / den, float((g - r).abs().max() / r.abs().max())
       # sharper logits (x2, x4) put more weight on fewer probabilities: the bf16 rounding of P and dS weighs more
       assert rel <= (6e-3 if mult == 1.0 else 1e-2) and mx <= (1.5e-2 if mult == 1.0 else 3e-2), f"{what} {name}: rel-l2 {rel:.2e} max {mx:.2e}"
+
+
+@pytest.mark.parametrize("D", [128, 64])
+def test_backward_over_kv_chunks_with_the_merged_lse(dev, D):
+  """The backward of a ring / chunked forward: every KV chunk is differentiated against the MERGED (out, lse) of the
+  whole key range; dq is the sum over the chunks and each chunk's dk / dv are the slices of the unsplit gradients
+  (the reference's ring backward does exactly this, kernels/splash_attention/ring_attention_kernel.py:1134-1230)."""
+  B, H, Sq, Skv = 2, 3, 200, 333
+  cuts = [0, 96, 231, Skv]  # ragged chunks
+  q, do = (to_dev_bf16(O.normal_bf16((B, Sq, H, D), s), dev) for s in (0, 3))
+  k, v = (to_dev_bf16(O.normal_bf16((B, Skv, H, D), s), dev) for s in (1, 2))
+  scale = D**-0.5
+  # forward chunk by chunk through the fused merge, as a ring does
+  o_run, l_run = ops.new_merge_state(B, Sq, H, D, dev)
+  for a, b in zip(cuts[:-1], cuts[1:]):
+    ops.flash_attention_merge(q, k[:, a:b], v[:, a:b], o_run, l_run, scale=scale)
+  out = ops.finalize(o_run)
+  out1, lse1 = ops.flash_attention(q, k, v, scale=scale, return_lse=True)
+  assert float((l_run - lse1).abs().max()) <= 1e-3
+  dq1, dk1, dv1 = ops.flash_attention_backward(q, k, v, out1, do, lse1, scale=scale)
+  dq = torch.zeros_like(dq1, dtype=torch.float32)
+  dk, dv = torch.empty_like(dk1), torch.empty_like(dv1)
+  for a, b in zip(cuts[:-1], cuts[1:]):
+    dq_c, dk_c, dv_c = ops.flash_attention_backward(q, k[:, a:b].contiguous(), v[:, a:b].contiguous(), out, do, l_run, scale=scale)
+    dq += dq_c.float()
+    dk[:, a:b], dv[:, a:b] = dk_c, dv_c
+  for got, want, name in ((dq, dq1, "dq"), (dk, dk1, "dk"), (dv, dv1, "dv")):
+    rl = rel_l2(to_np(got.to(torch.bfloat16)), to_np(want))
+    print(f"D={D} {name}: chunked vs unsplit rel-l2 {rl:.3e}", flush=True)
+    assert rl <= 1e-2, name  # bf16 roundings of the merged out and of the partial dq
