@@ -257,7 +257,7 @@ int mdattn_key_mask_bias(void* stream, const void* keep, float* bias, int B, int
                          float masked_value);
 
 /*
- * Per-tensor absmax quantisation bf16 -> OCP float8 e4m3fn (BASELINE configs[4]; no reference
+ * Per-tensor absmax quantisation bf16 -> OCP float8 e4m3fn (the benchmark's fp8 configuration; no reference
  * counterpart: the reference's fp8 is qwix quantisation of dense layers, pipelines/wan/wan_pipeline.py:581-626).
  *   x_bf16 [n] contiguous, x_fp8 [n] bytes,
  *   premul       constant multiplied into x before the (single) rounding to e4m3; 1.0f = none.  For q,

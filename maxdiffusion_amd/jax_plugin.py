@@ -131,7 +131,7 @@ def hip_quant_e4m3(x, premul: float = 1.0, pow2_scale: bool = False):
 
 
 def hip_flash_attention_fp8(q, k, v, scale: float, layout: int, softmax: str = "byte_grid", keep_mask=None):
-  """BASELINE configs[4]: quantises bf16 q, k, v per tensor (q carries scale * log2(e), q and k scales are powers of
+  """The fp8 configuration of the benchmark (Wan-14B self-attention in e4m3): quantises bf16 q, k, v per tensor (q carries scale * log2(e), q and k scales are powers of
   two) and runs the fp8-e4m3 kernel.  softmax "byte_grid" (fastest; use `out`) or "exp2" (exact lse, mergeable);
   keep_mask [B,Skv] bool: masked keys are excluded (exact exponentials).
   Returns (out [B,Sq,H,D] bf16, lse [B,H,Sq] f32)."""
@@ -478,7 +478,7 @@ def hip_flash_kernel(q, k, v, context):
 
 
 def hip_flash_fp8_kernel(q, k, v, context):
-  """The KERNEL_REGISTRY entry `hip_flash_fp8` (BASELINE configs[4]): per-tensor e4m3 q, k, v on the device, then the
+  """The KERNEL_REGISTRY entry `hip_flash_fp8` (the benchmark's fp8 configuration): per-tensor e4m3 q, k, v on the device, then the
   fp8 kernel; a [B,Skv] attention_mask is honoured like hip_flash honours it."""
   _, jnp = _require_jax()
   if context.get("is_causal"):

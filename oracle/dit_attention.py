@@ -49,7 +49,7 @@ Pinning status of each function (what fixes it besides its own formula):
                                  equals `attention` bit for bit.  (What XLA-CPU does inside einsum / softmax
                                  is fixed by no reference test or fixture; the flow restated is the one the
                                  source's dtypes prescribe, attention_flax.py:1546-1564.)
-  attention_fp8_emulated         no reference counterpart (BASELINE configs[4]).  Pinned by a scalar brute-force
+  attention_fp8_emulated         no reference counterpart (the benchmark's fp8 configuration).  Pinned by a scalar brute-force
                                  loop over rows, tiles and keys with torch.float8_e4m3fn casts (both scale
                                  kinds, both softmax forms, profiles that move the reference points), and by
                                  what the mathematics fixes: with exp2 the lse equals the f64 lse of the
@@ -522,7 +522,7 @@ def merge_scan_ring(outs, lses):
 
 
 def ring_replay(q, k_chunks, v_chunks, scale: float, dtype=np.float64):
-  """One Q shard against successive KV chunks, merged in LSE space (BASELINE configs[3])."""
+  """One Q shard against successive KV chunks, merged in LSE space (the benchmark's ring-shard configuration)."""
   o_run = np.zeros(q.shape, dtype)
   lse_run = np.full(q.shape[:-1], LSE_INIT, dtype)
   for kc, vc in zip(k_chunks, v_chunks):

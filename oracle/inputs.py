@@ -36,7 +36,7 @@ class Workload:
 
 
 WORKLOADS = {
-    # BASELINE.json configs[0..4]
+    # the five benchmark configurations: Wan-1.3B, Flux-dev, Wan-14B (self + 512-key cross), its ring shard, its fp8 form
     "wan1.3b": Workload("wan1.3b", 12, 128, 4680, 4680, "fullrow", "wan", (3, 30, 52)),
     "flux-dev": Workload("flux-dev", 24, 128, 4608, 4608, "perhead", "flux", (512, 64, 64)),
     "wan14b": Workload("wan14b", 40, 128, 75600, 75600, "fullrow", "wan", (21, 45, 80), cross_kv=512),

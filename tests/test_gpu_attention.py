@@ -1,6 +1,6 @@
 """Parity of the bf16 flash-attention forward (HIP, through the C ABI) against the CPU oracle.
 
-Bars (BASELINE north star): out max-abs <= 2e-2 and mean-abs <= 2e-3 against an f32/f64 reference,
+Bars (the benchmark's stated tolerances): out max-abs <= 2e-2 and mean-abs <= 2e-3 against an f32/f64 reference,
 LSE within 1e-3.  With N(0,1) inputs |out| is ~1e-2, so those absolute bars alone would pass an
 all-zero output: every case also checks the relative L2 error, and sharpened inputs are included."""
 import math

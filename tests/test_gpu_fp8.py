@@ -1,4 +1,4 @@
-"""fp8-e4m3 attention forward (HIP, through the C ABI): BASELINE configs[4].
+"""fp8-e4m3 attention forward (HIP, through the C ABI): the benchmark's fp8 configuration.
 
 No reference implementation of fp8 attention exists, so the bar is the north star's: cosine similarity
 >= 0.995 against the bf16 `dot_product` result (here the f32 oracle on the same bf16 inputs).  The

@@ -1,6 +1,6 @@
 """Parity of the fused RMSNorm + RoPE HIP kernels (through the C ABI) against the CPU oracle.
 
-Bars (BASELINE north star): max-abs <= 2e-2 and mean-abs <= 2e-3 against the f32/f64 oracle.
+Bars (the benchmark's stated tolerances): max-abs <= 2e-2 and mean-abs <= 2e-3 against the f32/f64 oracle.
 The kernel computes in f32 and rounds once, so the observed error is one bf16 rounding."""
 import numpy as np
 import pytest

@@ -93,7 +93,7 @@ def test_golden_ltx2(dev):
 
 @pytest.mark.parametrize("layout", ["bshd", "bhsd"])
 def test_wan13b_full_size(dev, layout):
-  """BASELINE configs[0] whole: every token of the Wan-1.3B shape, both tensors, against the f64 oracle."""
+  """The Wan-1.3B benchmark shape whole: every token of the Wan-1.3B shape, both tensors, against the f64 oracle."""
   w = O.WORKLOADS["wan1.3b"]
   H, D, S = w.heads, w.head_dim, w.seq
   q, k = O.normal_bf16((1, S, H * D), 0), O.normal_bf16((1, S, H * D), 1)
@@ -114,7 +114,7 @@ def test_wan13b_full_size(dev, layout):
 
 
 def test_flux_dev_full_size(dev):
-  """BASELINE configs[1] whole: 512 text + 4096 image tokens x 24 heads, separate text weights."""
+  """The Flux-dev benchmark shape whole: 512 text + 4096 image tokens x 24 heads, separate text weights."""
   w = O.WORKLOADS["flux-dev"]
   n_txt, rows, cols = w.grid
   ids = O.flux_ids(n_txt, rows, cols)
@@ -135,7 +135,7 @@ def test_flux_dev_full_size(dev):
 
 
 def test_wan14b_full_size_sampled_rows(dev):
-  """BASELINE configs[2] at full size: the input gradients on a deterministic sample of token rows against the f64
+  """The Wan-14B benchmark shape at full size: the input gradients on a deterministic sample of token rows against the f64
   oracle (a row's gradient depends on that row only); the weight gradients, sums over all 75,600 tokens, against the
   same formula evaluated by torch in f64 on the GPU from the kernel-independent inputs (test harness only)."""
   w = O.WORKLOADS["wan14b"]
