@@ -319,6 +319,28 @@ def test_folded_scale_ragged_and_sharp(dev, variant, var, sq, skv, mult):
   _check(out, lse, ro, rl, f"folded scale, variant {var} Sq={sq} Skv={skv} x{mult}")
 
 
+@pytest.mark.parametrize("sq,skv,mult", [(1, 1, 1.0), (40, 32, 1.0), (40, 33, 1.0), (31, 64, 1.0), (31, 65, 1.0), (257, 127, 1.0),
+                                         (300, 333, 1.0), (100, 4097, 1.0), (500, 700, 6.0)])
+def test_folded_scale_head_dim_64(dev, sq, skv, mult):
+  """The same at head dim 64 (the flat schedule's 64-key tiles, two 32-key blocks per tile: the first block of a row
+  always sets the reference point, the second must not)."""
+  H = 3
+  q = (np.random.default_rng(0).standard_normal((1, sq, H, 64)) * mult).astype(np.float32)
+  k, v = O.normal_bf16((1, skv, H, 64), 1), O.normal_bf16((1, skv, H, 64), 2)
+  out, lse, ro, rl = _folded_run(q, k, v, dev)
+  _check(out, lse, ro, rl, f"folded scale, head dim 64 Sq={sq} Skv={skv} x{mult}")
+
+
+@pytest.mark.parametrize("profile", ["ascending", "descending", "plateau", "late_spike"])
+def test_folded_scale_reference_point_moves_head_dim_64(dev, profile):
+  H, sq, skv = 2, 150, 1500
+  qs, ks = zip(*(structured_logits(sq, skv, 64, profile, seed=5 + h) for h in range(H)))
+  q, k = np.stack(qs, 1)[None], np.stack(ks, 1)[None]
+  v = O.normal_bf16((1, skv, H, 64), 2)
+  out, lse, ro, rl = _folded_run(q, k, v, dev)
+  _check(out, lse, ro, rl, f"folded scale, head dim 64, {profile}", lse_abs=2e-3 if profile == "late_spike" else LSE_ABS)
+
+
 @pytest.mark.parametrize("profile", ["ascending", "descending", "plateau", "late_spike", "all_far_below_zero"])
 def test_folded_scale_reference_point_moves(dev, variant, profile):
   variant(1)
