@@ -55,7 +55,9 @@ def main():
   ap.add_argument("--gpus", type=int, default=1)
   ap.add_argument("--steps", type=int, default=10)
   ap.add_argument("--warmup", type=int, default=3)
-  ap.add_argument("--workload", default="wan14b")
+  ap.add_argument("--workload", default=None,
+                  help="default wan14b; a run without this option also reports the backward blocks of --with-backward "
+                       "(a failure there is reported in the block and does not cost the headline line)")
   ap.add_argument("--cpu-rows", type=int, default=16384, help="query rows of the CPU-baseline slice (0: skip)")
   ap.add_argument("--traffic-probe", action="store_true",
                   help="also launch one 1 GiB device copy: the plain copy kernel of known size that scales rocprofv3's "
@@ -83,6 +85,10 @@ def main():
                   help="also time the backward pass (dq, dk, dv) of the workload's attention, outside the timed steps; "
                        "reported as a `backward` object beside the headline")
   args = ap.parse_args()
+  default_run = args.workload is None  # the plain `python bench.py [--gpus 1 --steps K --warmup W]` form
+  args.workload = args.workload or "wan14b"
+  explicit_backward = args.with_backward
+  args.with_backward = args.with_backward or default_run
   if args.gpus != 1:
     print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
     sys.exit(2)
@@ -284,66 +290,77 @@ def main():
   # comparison, on plain q with the softmax scale as an argument
   backward = None
   if args.with_backward and not fp8:
-    if D not in (64, 128):
-      raise SystemExit("--with-backward: the backward kernels are built for head dims 64 and 128")
-    vb = v[:, :Skv]
-    dout = randn(1, S, H, D)
 
-    def time_backward(qb, kb, sc):
-      ob, lb = ops.flash_attention(qb, kb, vb, scale=sc, return_lse=True)
-      for _ in range(2):
-        ops.flash_attention_backward(qb, kb, vb, ob, dout, lb, scale=sc)
-      e0, e1 = ev(), ev()
-      e0.record()
-      for _ in range(5):
-        ops.flash_attention_backward(qb, kb, vb, ob, dout, lb, scale=sc)
-      e1.record()
-      torch.cuda.synchronize()
-      return e0.elapsed_time(e1) / 5, (qb, kb, ob, lb)
+    def measure_backward():
+      if D not in (64, 128):
+        raise SystemExit("--with-backward: the backward kernels are built for head dims 64 and 128")
+      vb = v[:, :Skv]
+      dout = randn(1, S, H, D)
 
-    qf, kf = prologue()
-    bms, (qb, kb, ob, lb) = time_backward(qf, kf[:, :Skv] if kf.shape[1] != Skv else kf, att_scale)
-    if w.norm == "fullrow":
-      qp, kp = ops.norm_rope_fullrow(q_in, k_in, wq, wk, cos, sin, H)
-    elif w.norm == "rows":
-      qp, kp = ops.norm_rope_rows(q_in, wq, cos, sin, heads=H, mode="interleaved"), ops.norm_rope_rows(k_in, wk, cos, sin, heads=H, mode="interleaved")
-    else:
-      qp, kp = ops.norm_rope_perhead(q4, k4, wq, wk, cos, sin)
-    bms_plain, _ = time_backward(qp, kp, w.scale)
-    del qp, kp
-    # the five matrix products of the backward pass: S, dP, dV, dK, dQ (the two passes execute seven: S and dP are formed in both)
-    bfl = 2.5 * O.attention_flops(1, H, S, Skv, D)
-    btf = bfl / (bms * 1e-3) / 1e12
-    probe = None
-    if args.atomic_probe:
-      import ctypes
-
-      fn = _lib.load().mdattn_probe_dq_atomics
-      fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 5
-      fn.restype = ctypes.c_int
-      dqf = torch.zeros((H, S // 32 * 32, D), dtype=torch.float32, device=dev)
-      probe = {}
-      for per_wave, key in ((1, "per_wave_ms"), (0, "per_workgroup_ms")):
-        run = lambda: _lib.check(fn(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), ctypes.c_void_p(dqf.data_ptr()), H, S, Skv, D, per_wave), "probe")
-        run()
+      def time_backward(qb, kb, sc):
+        ob, lb = ops.flash_attention(qb, kb, vb, scale=sc, return_lse=True)
+        for _ in range(2):
+          ops.flash_attention_backward(qb, kb, vb, ob, dout, lb, scale=sc)
         e0, e1 = ev(), ev()
         e0.record()
-        for _ in range(3):
-          run()
+        for _ in range(5):
+          ops.flash_attention_backward(qb, kb, vb, ob, dout, lb, scale=sc)
         e1.record()
         torch.cuda.synchronize()
-        probe[key] = e0.elapsed_time(e1) / 3
-      n_add = H * (Skv // 256) * (S // 32) * 32 * D  # per workgroup and query tile: one 32 x D partial
-      probe.update({"atomic_adds_per_workgroup_mode": n_add, "atomic_adds_per_wave_mode": 8 * n_add,
-                    "note": "f32 atomic adds of the dq partials of a key-outer single pass, nothing else in the launch"})
-      del dqf
-    backward = {"Sq": S, "Skv": Skv, "ms": bms, "TFLOP/s": btf, "bound": "mfma", "peak": 2500.0, "frac": btf / 2500.0,
-                "frac_executed": btf * 7.0 / 5.0 / 2500.0,
-                "flop_counted": bfl, "ms_plain_scale": bms_plain,
-                "note": "5 matrix products counted, 7 executed (two atomic-free passes: dq; dk and dv); ms: q carries scale * log2(e) "
-                        "from the prologue, as in the headline forward; ms_plain_scale: plain q, softmax scale as an argument"}
-    if probe:
-      backward["single_pass_dq_atomics_probe"] = probe
+        return e0.elapsed_time(e1) / 5, (qb, kb, ob, lb)
+
+      qf, kf = prologue()
+      bms, (qb, kb, ob, lb) = time_backward(qf, kf[:, :Skv] if kf.shape[1] != Skv else kf, att_scale)
+      if w.norm == "fullrow":
+        qp, kp = ops.norm_rope_fullrow(q_in, k_in, wq, wk, cos, sin, H)
+      elif w.norm == "rows":
+        qp, kp = ops.norm_rope_rows(q_in, wq, cos, sin, heads=H, mode="interleaved"), ops.norm_rope_rows(k_in, wk, cos, sin, heads=H, mode="interleaved")
+      else:
+        qp, kp = ops.norm_rope_perhead(q4, k4, wq, wk, cos, sin)
+      bms_plain, _ = time_backward(qp, kp, w.scale)
+      del qp, kp
+      # the five matrix products of the backward pass: S, dP, dV, dK, dQ (the two passes execute seven: S and dP are formed in both)
+      bfl = 2.5 * O.attention_flops(1, H, S, Skv, D)
+      btf = bfl / (bms * 1e-3) / 1e12
+      probe = None
+      if args.atomic_probe:
+        import ctypes
+
+        fn = _lib.load().mdattn_probe_dq_atomics
+        fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 5
+        fn.restype = ctypes.c_int
+        dqf = torch.zeros((H, S // 32 * 32, D), dtype=torch.float32, device=dev)
+        probe = {}
+        for per_wave, key in ((1, "per_wave_ms"), (0, "per_workgroup_ms")):
+          run = lambda: _lib.check(fn(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), ctypes.c_void_p(dqf.data_ptr()), H, S, Skv, D, per_wave), "probe")
+          run()
+          e0, e1 = ev(), ev()
+          e0.record()
+          for _ in range(3):
+            run()
+          e1.record()
+          torch.cuda.synchronize()
+          probe[key] = e0.elapsed_time(e1) / 3
+        n_add = H * (Skv // 256) * (S // 32) * 32 * D  # per workgroup and query tile: one 32 x D partial
+        probe.update({"atomic_adds_per_workgroup_mode": n_add, "atomic_adds_per_wave_mode": 8 * n_add,
+                      "note": "f32 atomic adds of the dq partials of a key-outer single pass, nothing else in the launch"})
+        del dqf
+      backward = {"Sq": S, "Skv": Skv, "ms": bms, "TFLOP/s": btf, "bound": "mfma", "peak": 2500.0, "frac": btf / 2500.0,
+                  "frac_executed": btf * 7.0 / 5.0 / 2500.0,
+                  "flop_counted": bfl, "ms_plain_scale": bms_plain,
+                  "note": "5 matrix products counted, 7 executed (two atomic-free passes: dq; dk and dv); ms: q carries scale * log2(e) "
+                          "from the prologue, as in the headline forward; ms_plain_scale: plain q, softmax scale as an argument"}
+      if probe:
+        backward["single_pass_dq_atomics_probe"] = probe
+      return backward
+
+    if default_run and not explicit_backward:
+      try:
+        backward = measure_backward()
+      except Exception as e:  # the optional block must not cost the headline line
+        backward = {"error": f"{type(e).__name__}: {e}"}
+    else:
+      backward = measure_backward()
 
   # the key range split F ways inside one launch, then merged: what a key split could buy small grids
   key_split = None
@@ -407,34 +424,45 @@ def main():
   # backward of the prologue (input and weight gradients from the saved inputs and the gradients of its outputs)
   prologue_backward = None
   if args.with_backward:
-    gq, gk = randn(1, S, H, D), randn(1, S, H, D)
-    if w.norm == "fullrow":
-      runb = lambda: ops.norm_rope_fullrow_backward(q_in, k_in, wq, wk, cos, sin, H, gq, gk, q_mul=q_mul)
-      nlaunch, pb_bytes = 1, 6 * S * H * D * 2 + 2 * S * (D // 2) * 4 + 2 * H * D * (2 + 4)
-      kname_b = "norm_rope_fullrow_bwd_kernel"
-    elif w.norm == "rows":
-      runb = lambda: (ops.norm_rope_rows_backward(q_in, wq, gq, cos, sin, heads=H, mode="interleaved"),
-                      ops.norm_rope_rows_backward(k_in, wk, gk, cos, sin, heads=H, mode="interleaved"))
-      nlaunch, pb_bytes = 2, 6 * S * H * D * 2 + 2 * 2 * S * H * D * 4 + 2 * H * D * (4 + 4)
-      kname_b = "norm_rope_rows_bwd_kernel (two launches: q, k)"
+
+    def measure_prologue_backward():
+      gq, gk = randn(1, S, H, D), randn(1, S, H, D)
+      if w.norm == "fullrow":
+        runb = lambda: ops.norm_rope_fullrow_backward(q_in, k_in, wq, wk, cos, sin, H, gq, gk, q_mul=q_mul)
+        nlaunch, pb_bytes = 1, 6 * S * H * D * 2 + 2 * S * (D // 2) * 4 + 2 * H * D * (2 + 4)
+        kname_b = "norm_rope_fullrow_bwd_kernel"
+      elif w.norm == "rows":
+        runb = lambda: (ops.norm_rope_rows_backward(q_in, wq, gq, cos, sin, heads=H, mode="interleaved"),
+                        ops.norm_rope_rows_backward(k_in, wk, gk, cos, sin, heads=H, mode="interleaved"))
+        nlaunch, pb_bytes = 2, 6 * S * H * D * 2 + 2 * 2 * S * H * D * 4 + 2 * H * D * (4 + 4)
+        kname_b = "norm_rope_rows_bwd_kernel (two launches: q, k)"
+      else:
+        runb = lambda: ops.norm_rope_perhead_backward(q4, k4, wq, wk, cos, sin, gq, gk, q_mul=q_mul)
+        nlaunch, pb_bytes = 1, 6 * S * H * D * 2 + 2 * S * (D // 2) * 4 + 2 * D * (2 + 4)
+        kname_b = "norm_rope_perhead_bwd_kernel"
+      for _ in range(2):
+        runb()
+      e0, e1 = ev(), ev()
+      e0.record()
+      for _ in range(reps):
+        runb()
+      e1.record()
+      torch.cuda.synchronize()
+      pbms = e0.elapsed_time(e1) / reps
+      prologue_backward = {"bound": "hbm", "achieved": pb_bytes / (pbms * 1e-3) / 1e9, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                           "frac": pb_bytes / (pbms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "traffic": None, "kernel": kname_b,
+                           "ms": pbms, "bytes_per_call": pb_bytes,
+                           "note": "saved inputs and output gradients read once, input gradients written once (bf16), tables, weights and "
+                                   "f32 weight gradients; the time includes the second-stage column sum and the workspace allocation"}
+      return prologue_backward
+
+    if default_run and not explicit_backward:
+      try:
+        prologue_backward = measure_prologue_backward()
+      except Exception as e:  # the optional block must not cost the headline line
+        prologue_backward = {"error": f"{type(e).__name__}: {e}"}
     else:
-      runb = lambda: ops.norm_rope_perhead_backward(q4, k4, wq, wk, cos, sin, gq, gk, q_mul=q_mul)
-      nlaunch, pb_bytes = 1, 6 * S * H * D * 2 + 2 * S * (D // 2) * 4 + 2 * D * (2 + 4)
-      kname_b = "norm_rope_perhead_bwd_kernel"
-    for _ in range(2):
-      runb()
-    e0, e1 = ev(), ev()
-    e0.record()
-    for _ in range(reps):
-      runb()
-    e1.record()
-    torch.cuda.synchronize()
-    pbms = e0.elapsed_time(e1) / reps
-    prologue_backward = {"bound": "hbm", "achieved": pb_bytes / (pbms * 1e-3) / 1e9, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                         "frac": pb_bytes / (pbms * 1e-3) / 1e9 / PEAK_HBM_GBPS, "traffic": None, "kernel": kname_b,
-                         "ms": pbms, "bytes_per_call": pb_bytes,
-                         "note": "saved inputs and output gradients read once, input gradients written once (bf16), tables, weights and "
-                                 "f32 weight gradients; the time includes the second-stage column sum and the workspace allocation"}
+      prologue_backward = measure_prologue_backward()
 
   flops = O.attention_flops(1, H, S, Skv * ring, D)
   att_ms = sum(t_att) / len(t_att)
