@@ -338,7 +338,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
         const float dm = (BLK) == 0 ? mloc : fmaxf(mloc, 0.f);                                                \
         alpha = (BLK) == 0 ? 0.f : __builtin_amdgcn_exp2f(-dm);                                               \
         mc += dm;                                                                                             \
-        _Pragma("unroll") for (int i = 0; i < 16; ++i) { SC[i] -= dm; SN[i] -= dm; negm[i] = -mc; }           \
+        _Pragma("unroll") for (int i = 0; i < 16; ++i) { SC[i] -= dm; SN[i] -= dm; negm[i] -= dm; }           \
       } else {                                                                                                \
         const float mnew = fmaxf(m, mloc);                                                                    \
         alpha = __builtin_amdgcn_exp2f((m - mnew) * c); /* exactly 1 for rows that keep m */                  \
@@ -619,7 +619,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
         alpha = first ? 0.f : __builtin_amdgcn_exp2f(-dm);
         mc += dm;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { S[i] -= dm; negm[i] = -mc; }
+        for (int i = 0; i < 16; ++i) { S[i] -= dm; negm[i] -= dm; }
       } else {
         const float mnew = fmaxf(m, mloc);
         alpha = __builtin_amdgcn_exp2f((m - mnew) * cs);
