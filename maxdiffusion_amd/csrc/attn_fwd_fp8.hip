@@ -298,12 +298,14 @@ __device__ __forceinline__ void fp8_body(const Fp8Args& a, const float c, char* 
     // every output row holds the sums, over both halves of the row's keys) instead of two decodes and four adds per
     // four logits (1.3 % faster at head dim 128, 6 % at 64).  A byte 0x7F still poisons the sum with its NaN.
     auto rowsum = [&]() __attribute__((always_inline)) {
-      const int one4 = 0x38383838;  // four e4m3 ones
-      const i32x8 ones = {one4, one4, one4, one4, one4, one4, one4, one4};
+      // the ones as FP4 (E2M1: 1.0 = 0b0010), the operand bytes as e4m3: the instruction takes the two formats
+      // independently, and a lane's 32 FP4 ones are four registers where e4m3 ones are eight
+      const int one8 = 0x22222222;  // eight E2M1 ones
+      const i32x8 ones = {one8, one8, one8, one8, 0, 0, 0, 0};
       f32x16 z;
 #pragma unroll
       for (int i = 0; i < 16; ++i) z[i] = 0.f;
-      z = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pk, z, 0, 0, 0, 0, 0, 0);
+      z = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pk, z, 4, 0, 0, 0, 0, 0);
       return z[0];
     };
     if constexpr (CODE) ls = rowsum();
