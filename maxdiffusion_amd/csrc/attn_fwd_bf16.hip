@@ -425,6 +425,12 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
   store_row<4>(a, O, xhalf_sum(l), mc, b, h, q0 + l32, hh);
 }
 
+#ifndef MDATTN_FLAT_PAIRWISE
+#define MDATTN_FLAT_PAIRWISE 1
+#endif
+#ifndef MDATTN_FLAT_LA128
+#define MDATTN_FLAT_LA128 2
+#endif
 // ---------------------------------------------------------------------------------------------------
 // Second schedule: no software pipelining inside a wave.  Four waves per workgroup, 32-key tiles in a
 // 3-slot ring (50 KB of LDS) and at most 168 VGPRs, so that three workgroups share a CU and three waves
@@ -556,11 +562,27 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
       v_off[sg] = KTILE + (4 * hh + vxr) * 64 + (sg ^ vx) * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
   }
 
+  // A tile's fragment reads as one stream (per 32-key block: NJ row reads of K, then 2*ND transposing reads of V) with a
+  // window of LA fragments running ahead of the MFMAs, pinned by scheduling barriers: left to itself the compiler
+  // waits for every read right before its MFMA.
+  constexpr int LA = HD == 128 ? MDATTN_FLAT_LA128 : 0;
+  constexpr int FPB = NJ + 2 * ND, NFRAG = NB * FPB;
   auto tile = [&](int t, int slot, auto masked) __attribute__((always_inline)) {
     const __bf16* base = smem + slot * STAGE;
+    constexpr int kBlk = 32 * 64;  // a 32-key block of a head-dim-64 tile: 32 rows of 64 elements, in K and in V
+    auto frag = [&](int n) __attribute__((always_inline)) {
+      const int fb = n / FPB, r = n % FPB;
+      if (r < NJ) return *reinterpret_cast<const bf16x8*>(base + k_off[r] + fb * kBlk);
+      const __bf16* vsrc = base + v_off[(r - NJ) % ND] + ((r - NJ) / ND) * kVH + fb * kBlk;
+      return read_vt(vsrc, vsrc + kV8);
+    };
+    [[maybe_unused]] bf16x8 win[LA > 0 ? LA : 1];
+    if constexpr (LA > 0) {
+#pragma unroll
+      for (int n = 0; n < LA; ++n) win[n] = frag(n);
+    }
 #pragma unroll
    for (int blk = 0; blk < NB; ++blk) {
-    constexpr int kBlk = 32 * 64;  // a 32-key block of a head-dim-64 tile: 32 rows of 64 elements, in K and in V
     const bool first = t == 0 && blk == 0;
     // ---- S^T = K.Q^T: one chain of MFMAs; the other waves of the SIMD fill the gaps between them.  A wave in an
     // MFMA phase issues ahead of the SIMD's waves in their softmax phase (1-2 % on short key sequences).
@@ -570,8 +592,15 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
     for (int i = 0; i < 16; ++i) S[i] = 0.f;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + k_off[j] + blk * kBlk);
-      S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[j], (PRE && j == 0) ? negm : S, 0, 0, 0);
+      if constexpr (LA > 0) {
+        const int n = blk * FPB + j;
+        S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(win[n % LA], qf[j], (PRE && j == 0) ? negm : S, 0, 0, 0);
+        if (n + LA < NFRAG) win[n % LA] = frag(n + LA);
+        __builtin_amdgcn_sched_barrier(0);
+      } else {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + k_off[j] + blk * kBlk);
+        S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[j], (PRE && j == 0) ? negm : S, 0, 0, 0);
+      }
     }
     if constexpr (BIAS) {
 #pragma unroll
@@ -597,6 +626,21 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
       float lsum = 0.f;
 #pragma unroll
       for (int hb = 0; hb < 2; ++hb) {
+#if MDATTN_FLAT_PAIRWISE
+        // two logits at a time, packed as soon as they exist: 16 f32 probabilities never live at once, which is what
+        // leaves this kernel registers for a fragment window
+        unsigned pk[4];
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          const float x0 = __builtin_amdgcn_exp2f(PRE ? S[8 * hb + e] : __builtin_fmaf(S[8 * hb + e], cs, -rf));
+          const float x1 = __builtin_amdgcn_exp2f(PRE ? S[8 * hb + e + 1] : __builtin_fmaf(S[8 * hb + e + 1], cs, -rf));
+          lsum += x0;
+          lsum += x1;
+          pk[e >> 1] = pack2(x0, x1);
+          asm volatile("" : "+v"(pk[e >> 1]), "+v"(lsum));
+        }
+        P[hb] = __builtin_bit_cast(bf16x8, u32x4{pk[0], pk[1], pk[2], pk[3]});
+#else
         float p[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -604,6 +648,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
           lsum += p[e];
         }
         P[hb] = __builtin_bit_cast(bf16x8, pack8(p));
+#endif
       }
       return lsum;
     };
@@ -639,9 +684,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
     // ---- O^T += V^T.P^T
 #pragma unroll
     for (int jv = 0; jv < 2 * ND; ++jv) {
-      const __bf16* vsrc = base + v_off[jv % ND] + (jv / ND) * kVH + blk * kBlk;
-      const bf16x8 vf = read_vt(vsrc, vsrc + kV8);
-      O[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P[jv / ND], O[jv % ND], 0, 0, 0);
+      if constexpr (LA > 0) {
+        const int n = blk * FPB + NJ + jv;
+        O[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(win[n % LA], P[jv / ND], O[jv % ND], 0, 0, 0);
+        if (n + LA < NFRAG) win[n % LA] = frag(n + LA);
+        __builtin_amdgcn_sched_barrier(0);
+      } else {
+        const __bf16* vsrc = base + v_off[jv % ND] + (jv / ND) * kVH + blk * kBlk;
+        const bf16x8 vf = read_vt(vsrc, vsrc + kV8);
+        O[jv % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, P[jv / ND], O[jv % ND], 0, 0, 0);
+      }
     }
    }
   };
