@@ -368,15 +368,25 @@ __device__ __forceinline__ void fp8_body(const Fp8Args& a, const float c, char* 
     }
     l += ls;
     // ---- O^T += V^T.P^T
-#pragma unroll
-    for (int sl = 0; sl < NSL; ++sl) {
+    // The V^T operand of slab sl + 1 is requested before the MFMA of slab sl is issued (the 16 registers of the logits
+    // are free by now), pinned by scheduling barriers: the compiler's own order reads each operand into one
+    // buffer and waits for it right before its MFMA.
+    auto vfrag = [&](int sl) __attribute__((always_inline)) {
       const char* vsrc = Ks + v_off[sl];
       const i32x2 r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_ptr)(vsrc));
       const i32x2 r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_ptr)(vsrc + 16 * kVS8));
       const i32x2 r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_ptr)(vsrc + 32 * kVS8));
       const i32x2 r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_ptr)(vsrc + 48 * kVS8));
-      const i32x8 vf = {r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
-      O[sl] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pk, O[sl], 0, 0, 0, 0, 0, 0);
+      return i32x8{r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
+    };
+    i32x8 vw[2];
+    vw[0] = vfrag(0);
+#pragma unroll
+    for (int sl = 0; sl < NSL; ++sl) {
+      if (sl + 1 < NSL) vw[(sl + 1) & 1] = vfrag(sl + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      O[sl] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vw[sl & 1], pk, O[sl], 0, 0, 0, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
