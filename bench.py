@@ -74,6 +74,11 @@ def main():
   ap.add_argument("--hbm-probe", action="store_true",
                   help="also time the runtime's own streaming kernels on tensors of the prologue's size (copy, two-input add, "
                        "fill, sum): what this machine's memory system gives plain kernels, for scale; reported as `hbm_probe`")
+  ap.add_argument("--mfma-probe", action="store_true",
+                  help="also run the library's MFMA rate probe: MFMA 32x32x16 bf16 back to back on the workload's kind of "
+                       "operands (N(0,1) rounded to bf16) and on zeros, alone and with the LDS reads / softmax instructions of "
+                       "an attention loop beside them; reported as `mfma_probe` (what this machine sustains, against the "
+                       "published peak)")
   ap.add_argument("--atomic-probe", action="store_true",
                   help="with --with-backward: also time the f32 atomic adds that a single-pass backward (five matrix products "
                        "instead of seven) would issue for dq at this shape, per wave and reduced per workgroup; reported inside "
@@ -421,6 +426,43 @@ def main():
                  "note": "torch's own elementwise / reduction kernels on bf16 tensors of the prologue's size"}
     del a_, b_, c_
 
+  mfma_probe = None
+  if args.mfma_probe:
+    import ctypes
+
+    fn = _lib.load().mdattn_probe_mfma_rate
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    fn.restype = ctypes.c_int
+    p_iters, p_grid = 20000, 4096  # 2 workgroups of 4 waves per CU at a time, 8 rounds: about 50 ms per launch
+    src = torch.randn(32768, device=dev).to(torch.bfloat16)  # 16384 words
+    sink = torch.empty(p_grid * 256, dtype=torch.float32, device=dev)
+    rows = []
+    for mode, what in ((0, "MFMA only, operands in registers"), (1, "A operand from LDS for every MFMA"),
+                       (2, "A operand from LDS for every second MFMA"),
+                       (16, "registers; 1 exp2, 1 add, 1/2 pack per MFMA (head dim 128's softmax)"),
+                       (17, "LDS every MFMA; head dim 128's softmax"), (18, "LDS every second MFMA; head dim 128's softmax"),
+                       (4, "registers; 2 exp2, 2 add, 1 pack per MFMA (head dim 64's softmax)"),
+                       (5, "LDS every MFMA; head dim 64's softmax"), (6, "LDS every second MFMA; head dim 64's softmax"),
+                       (8, "MFMA only, all operands zero"), (9, "LDS every MFMA, all operands zero")):
+      run = lambda: _lib.check(fn(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), mode, p_iters, p_grid,
+                                  ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(sink.data_ptr())), "mfma probe")
+      for _ in range(2):
+        run()
+      e0, e1 = ev(), ev()
+      e0.record()
+      for _ in range(3):
+        run()
+      e1.record()
+      torch.cuda.synchronize()
+      ms = e0.elapsed_time(e1) / 3
+      tf = p_grid * 4 * p_iters * 8 * 32768 / (ms * 1e-3) / 1e12  # 32 x 32 x 16 x 2 FLOP per MFMA and wave
+      rows.append({"mode": mode, "what": what, "ms": ms, "TFLOP/s": tf, "frac_of_peak": tf / 2500.0,
+                   "GHz_of_a_full_pipe": tf / 2500.0 * 2.4})
+    mfma_probe = {"peak": 2500.0, "unit": "TFLOP/s", "rows": rows,
+                  "note": "MFMA 32x32x16 bf16 back to back, 2 waves per SIMD, 4 accumulators per wave; the published peak is "
+                          "1024 SIMDs x one MFMA per 32 clocks x 2.4 GHz"}
+    del src, sink
+
   # backward of the prologue (input and weight gradients from the saved inputs and the gradients of its outputs)
   prologue_backward = None
   if args.with_backward:
@@ -520,6 +562,8 @@ def main():
     out["key_split"] = key_split
   if hbm_probe:
     out["hbm_probe"] = hbm_probe
+  if mfma_probe:
+    out["mfma_probe"] = mfma_probe
   if args.cpu_rows > 0:
     out["cpu_baseline"] = cpu_baseline(w, args.cpu_rows)
   print(json.dumps(out), flush=True)

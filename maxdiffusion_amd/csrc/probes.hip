@@ -7,6 +7,15 @@
 // the workgroup), without it the workgroup adds one partial per query tile, as if its eight waves had reduced theirs
 // first (each wave adds an eighth).  The time of the launch is a lower bound of what the atomics would add to a
 // backward pass that saved its two duplicate matrix products.
+//
+// mdattn_probe_mfma_rate: what the chip sustains on MFMA 32x32x16 bf16 issued back to back (two waves per SIMD, four
+// independent accumulators per wave, nothing to wait for), alone and with the LDS reads and vector instructions an
+// attention loop issues beside its MFMAs.  The shader clock is managed against a power limit, so the published peak
+// (every SIMD starting an MFMA every 32 clocks at 2.4 GHz) is an upper bound that random operands do not reach; the
+// probe gives the bound that applies to a given instruction mix and operand content.  `mode` bits: 1 = the A operand
+// of every MFMA is read from LDS (1 KB per MFMA, as the K / V fragments are), 2 = of every second MFMA (two MFMAs
+// share a fragment), 4 = two exp2, two adds and one bf16 pack per MFMA (the softmax of head dim 64), 16 = half of
+// that (head dim 128), 8 = all operands zero instead of the caller's data.
 #include "mdattn_common.h"
 
 namespace mdattn {
@@ -26,7 +35,75 @@ __global__ __launch_bounds__(512) void probe_dq_atomics_kernel(float* dq, int Sq
     t = t + 1 == nqt ? 0 : t + 1;
   }
 }
+
+template <int MODE>
+__global__ __launch_bounds__(256, 2) void probe_mfma_rate_kernel(const unsigned* src, float* out, int iters) {
+  __shared__ __attribute__((aligned(16))) unsigned smem[32768 / 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < 32768 / 4; i += 256) smem[i] = (MODE & 8) ? 0u : src[i];
+  __syncthreads();
+  bf16x8 bfr[4], afr[4];
+  for (int j = 0; j < 4; ++j) {
+    u32x4 t, u;
+    for (int e = 0; e < 4; ++e) {
+      t[e] = (MODE & 8) ? 0u : src[8192 + (j * 64 + lane) * 4 + e];
+      u[e] = (MODE & 8) ? 0u : src[12288 + (j * 64 + lane) * 4 + e];
+    }
+    bfr[j] = __builtin_bit_cast(bf16x8, t);
+    afr[j] = __builtin_bit_cast(bf16x8, u);
+  }
+  f32x16 acc[4];
+  for (int j = 0; j < 4; ++j)
+    for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+  float vs = 0.f, x = (MODE & 8) ? 0.f : 0.001f * lane;
+  unsigned pk = 0;
+  const u32x4* lds = reinterpret_cast<const u32x4*>(smem) + lane + wave * 512;  // 8 KB per wave, read 1 KB at a time
+  bf16x8 win[2];
+  win[0] = __builtin_bit_cast(bf16x8, lds[0]);
+  win[1] = __builtin_bit_cast(bf16x8, lds[64]);
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if constexpr ((MODE & 1) != 0) {  // a window of two reads runs ahead of the MFMAs, as in the attention kernels
+        acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(win[j & 1], bfr[j & 3], acc[j & 3], 0, 0, 0);
+        win[j & 1] = __builtin_bit_cast(bf16x8, lds[((j + 2) & 7) * 64]);
+      } else if constexpr ((MODE & 2) != 0) {
+        acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(win[(j >> 1) & 1], bfr[j & 3], acc[j & 3], 0, 0, 0);
+        if (j & 1) win[(j >> 1) & 1] = __builtin_bit_cast(bf16x8, lds[(((j >> 1) + 2) & 3) * 64]);
+      } else {
+        acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[j & 3], bfr[j & 3], acc[j & 3], 0, 0, 0);
+      }
+      if ((MODE & 4) || ((MODE & 16) && (j & 1))) {
+        const float e0 = __builtin_amdgcn_exp2f(x), e1 = __builtin_amdgcn_exp2f(-x);
+        vs += e0;
+        vs += e1;
+        pk ^= pack2(e0, e1);
+        asm volatile("" : "+v"(vs), "+v"(pk), "+v"(x));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  float r = vs + __builtin_bit_cast(float, pk & 0x3fffffffu);
+  for (int j = 0; j < 4; ++j)
+    for (int i = 0; i < 16; ++i) r += acc[j][i];
+  out[blockIdx.x * 256 + tid] = r;
+}
 }  // namespace mdattn
+
+// src: 16384 words of operand data (bf16 pairs); out: grid * 256 floats.  Every wave issues 8 * iters MFMAs.
+extern "C" int mdattn_probe_mfma_rate(void* stream, int mode, int iters, int grid, const unsigned* src, float* out) {
+  if (!src || !out || iters <= 0 || grid <= 0) return MDATTN_E_BADARG;
+  hipStream_t st = (hipStream_t)stream;
+#define MDATTN_PROBE_CASE(M) \
+  case M: MDATTN_LAUNCH(mdattn::probe_mfma_rate_kernel<M>, dim3(grid), dim3(256), 0, st, src, out, iters); break;
+  switch (mode) {
+    MDATTN_PROBE_CASE(0) MDATTN_PROBE_CASE(1) MDATTN_PROBE_CASE(2) MDATTN_PROBE_CASE(4) MDATTN_PROBE_CASE(5) MDATTN_PROBE_CASE(6)
+    MDATTN_PROBE_CASE(16) MDATTN_PROBE_CASE(17) MDATTN_PROBE_CASE(18) MDATTN_PROBE_CASE(8) MDATTN_PROBE_CASE(9)
+    default: return MDATTN_E_BADARG;
+  }
+#undef MDATTN_PROBE_CASE
+  return mdattn::launch_status();
+}
 
 extern "C" int mdattn_probe_dq_atomics(void* stream, float* dq, int H, int Sq, int Skv, int D, int per_wave) {
   if (!dq || H <= 0 || Sq < 32 || Skv < 256 || D <= 0 || D % 16) return MDATTN_E_BADARG;
