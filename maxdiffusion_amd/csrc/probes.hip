@@ -88,9 +88,69 @@ __global__ __launch_bounds__(256, 2) void probe_mfma_rate_kernel(const unsigned*
     for (int i = 0; i < 16; ++i) r += acc[j][i];
   out[blockIdx.x * 256 + tid] = r;
 }
+
+// The same for the fp8 MFMA (32x32x64 f8f6f4 on e4m3 operands: four times the FLOP of the bf16 instruction in twice its
+// clocks).  MODE bit 1: the A operand (2 KB) of every MFMA is read from
+// LDS; bit 4: four exp2, four adds and two 4-byte packs per MFMA (an fp8 attention loop's softmax at head dim 128);
+// bit 8: operands zero.
+template <int MODE>
+__global__ __launch_bounds__(256, 2) void probe_mfma_rate_fp8_kernel(const unsigned* src, float* out, int iters) {
+  __shared__ __attribute__((aligned(16))) unsigned smem[65536 / 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < 65536 / 4; i += 256) smem[i] = (MODE & 8) ? 0u : src[i & 16383];
+  __syncthreads();
+  i32x8 bfr[4], afr[4];
+  for (int j = 0; j < 4; ++j)
+    for (int e = 0; e < 8; ++e) {
+      bfr[j][e] = (MODE & 8) ? 0 : (int)src[(j * 64 + lane) * 8 + e];
+      afr[j][e] = (MODE & 8) ? 0 : (int)src[4096 + (j * 64 + lane) * 8 + e];
+    }
+  f32x16 acc[4];
+  for (int j = 0; j < 4; ++j)
+    for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+  float vs = 0.f, x = (MODE & 8) ? 0.f : 0.001f * lane;
+  unsigned pk = 0;
+  const u32x4* lds = reinterpret_cast<const u32x4*>(smem) + lane + wave * 1024;  // 16 KB per wave, read 2 KB at a time
+  auto rd = [&](int f) __attribute__((always_inline)) {
+    const u32x4 lo = lds[f * 128], hi = lds[f * 128 + 64];
+    return i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+  };
+  i32x8 win[2];
+  win[0] = rd(0);
+  win[1] = rd(1);
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if constexpr ((MODE & 1) != 0) {
+        acc[j & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(win[j & 1], bfr[j & 3], acc[j & 3], 0, 0, 0, 0, 0, 0);
+        win[j & 1] = rd((j + 2) & 7);
+      } else {
+        acc[j & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(afr[j & 3], bfr[j & 3], acc[j & 3], 0, 0, 0, 0, 0, 0);
+      }
+      if constexpr ((MODE & 4) != 0) {
+        const float e0 = __builtin_amdgcn_exp2f(x), e1 = __builtin_amdgcn_exp2f(-x);
+        vs += e0;
+        vs += e1;
+        pk = (unsigned)__builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, (int)pk, false);
+        asm volatile("" : "+v"(vs), "+v"(pk), "+v"(x));
+        const float e2 = __builtin_amdgcn_exp2f(x), e3 = __builtin_amdgcn_exp2f(-x);
+        vs += e2;
+        vs += e3;
+        pk = (unsigned)__builtin_amdgcn_cvt_pk_fp8_f32(e2, e3, (int)pk, true);
+        asm volatile("" : "+v"(vs), "+v"(pk), "+v"(x));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  float r = vs + __builtin_bit_cast(float, pk & 0x3f3f3f3fu);
+  for (int j = 0; j < 4; ++j)
+    for (int i = 0; i < 16; ++i) r += acc[j][i];
+  out[blockIdx.x * 256 + tid] = r;
+}
 }  // namespace mdattn
 
-// src: 16384 words of operand data (bf16 pairs); out: grid * 256 floats.  Every wave issues 8 * iters MFMAs.
+// src: 16384 words of operand data (bf16 pairs, or fp8 quadruples for modes >= 32); out: grid * 256 floats.  Every wave
+// issues 8 * iters MFMAs.
 extern "C" int mdattn_probe_mfma_rate(void* stream, int mode, int iters, int grid, const unsigned* src, float* out) {
   if (!src || !out || iters <= 0 || grid <= 0) return MDATTN_E_BADARG;
   hipStream_t st = (hipStream_t)stream;
@@ -99,6 +159,10 @@ extern "C" int mdattn_probe_mfma_rate(void* stream, int mode, int iters, int gri
   switch (mode) {
     MDATTN_PROBE_CASE(0) MDATTN_PROBE_CASE(1) MDATTN_PROBE_CASE(2) MDATTN_PROBE_CASE(4) MDATTN_PROBE_CASE(5) MDATTN_PROBE_CASE(6)
     MDATTN_PROBE_CASE(16) MDATTN_PROBE_CASE(17) MDATTN_PROBE_CASE(18) MDATTN_PROBE_CASE(8) MDATTN_PROBE_CASE(9)
+#define MDATTN_PROBE_CASE8(M) \
+  case 32 + M: MDATTN_LAUNCH(mdattn::probe_mfma_rate_fp8_kernel<M>, dim3(grid), dim3(256), 0, st, src, out, iters); break;
+    MDATTN_PROBE_CASE8(0) MDATTN_PROBE_CASE8(1) MDATTN_PROBE_CASE8(4) MDATTN_PROBE_CASE8(5) MDATTN_PROBE_CASE8(8)
+#undef MDATTN_PROBE_CASE8
     default: return MDATTN_E_BADARG;
   }
 #undef MDATTN_PROBE_CASE
