@@ -88,6 +88,19 @@ def _mask_bias(context, qv, kv):
   return ops.key_mask_bias(mask)
 
 
+def _pad_head_dim(qv, kv, vv):
+  """Head dims below 128 other than 64 are zero-padded to the next size the kernels take (64 or 128), as the
+  reference's flash wrappers pad them to 128 (attention_flax.py:223-259, `_pad_data_for_flash`): zero columns of q and
+  k add nothing to a logit, zero columns of v give output columns that the caller of this helper slices off.  Returns
+  the (possibly padded) views and the original head dim.  One more pass over each tensor; gradients flow through the
+  pad.  Head dims above 128 are left alone: the kernel entry rejects them."""
+  d = qv.shape[-1]
+  if d in (64, 128) or d > 128:
+    return qv, kv, vv, d
+  extra = (64 if d < 64 else 128) - d
+  return tuple(torch.nn.functional.pad(t, (0, extra)) for t in (qv, kv, vv)) + (d,)
+
+
 def _dense(t: torch.Tensor) -> torch.Tensor:
   """A view whose memory is dense in some axis order (the backward kernels write gradients with the operand's strides)."""
   return t if t.is_contiguous() or t.permute(0, 2, 1, 3).is_contiguous() else t.contiguous()
@@ -140,12 +153,13 @@ def hip_flash_kernel(q, k, v, context):
   # [B,Skv] keep-mask (attention_flax.py:1926-1939): masked keys are excluded, as the flash wrappers do with
   # segment ids (:390-438); rows without a kept key return 0 (:1552-1554)
   bias = _mask_bias(context, qv, kv)
+  qv, kv, vv, d0 = _pad_head_dim(qv, kv, vv)
   if torch.is_grad_enabled() and (qv.requires_grad or kv.requires_grad or vv.requires_grad):
     out = hip_flash_attention_autograd(qv, kv, vv, context["scale"], bias)
   else:
     out = ops.flash_attention(qv, kv, vv, scale=context["scale"], key_bias=bias)
   b, s, h, d = out.shape
-  out = out.reshape(b, s, h * d)
+  out = out[..., :d0].reshape(b, s, h * d0)
   return out.to(q.dtype) if cast else out
 
 
@@ -154,7 +168,8 @@ def hip_flash_fp8_kernel(q, k, v, context):
   """fp8-e4m3 variant: per-tensor absmax quantisation of q, k, v on the device, then the fp8 kernel."""
   _reject_unsupported(context)
   heads = context["heads"]
-  qv, kv, vv = (_as_bshd(t, heads).to(torch.bfloat16).contiguous() for t in (q, k, v))
+  qv, kv, vv, d0 = _pad_head_dim(*(_as_bshd(t, heads).to(torch.bfloat16) for t in (q, k, v)))
+  qv, kv, vv = qv.contiguous(), kv.contiguous(), vv.contiguous()
   # the softmax scale rides on q's quantisation (one rounding either way) and the q and k scales are powers of two:
   # the kernel then applies the whole logit scale inside its MFMAs; the registry entry returns `out` only, so it asks
   # for the softmax without exponentials (P's e4m3 byte straight from the logit: a piecewise-linear exponential
@@ -165,7 +180,7 @@ def hip_flash_fp8_kernel(q, k, v, context):
   # a [B,Skv] keep-mask goes in as an additive key bias (exact-exponential softmax), as for hip_flash
   out = ops.flash_attention_fp8(q8, k8, v8, sq, sk, sv, scale=ops.FOLDED_SCALE, softmax="byte_grid", key_bias=_mask_bias(context, qv, kv))
   b, s, h, d = out.shape
-  return out.reshape(b, s, h * d).to(q.dtype)
+  return out[..., :d0].reshape(b, s, h * d0).to(q.dtype)
 
 
 

@@ -458,6 +458,19 @@ def _as_rank4(q, k, v, heads: int):
   return q, k, v, 1
 
 
+def _pad_head_dim(q4, k4, v4):
+  """Head dims below 128 other than 64: zero-padded to the next size the kernels take (64 or 128), as the reference's
+  flash wrappers pad to 128 (attention_flax.py:223-259); returns the arrays and the original head dim, to which the
+  caller slices the output.  jnp.pad and the slice are differentiable, so the custom_vjp inside sees padded shapes."""
+  _, jnp = _require_jax()
+  d = q4.shape[-1]
+  if d in (64, 128) or d > 128:
+    return q4, k4, v4, d
+  extra = (64 if d < 64 else 128) - d
+  widths = ((0, 0), (0, 0), (0, 0), (0, extra))
+  return jnp.pad(q4, widths), jnp.pad(k4, widths), jnp.pad(v4, widths), d
+
+
 def hip_flash_kernel(q, k, v, context):
   """The KERNEL_REGISTRY entry `hip_flash`: fn(q, k, v, context) -> [B, Sq, H*D] in q's dtype.  The function is a
   jax.custom_vjp (forward custom call with lse, backward custom calls): the trainer differentiates straight through
@@ -469,12 +482,13 @@ def hip_flash_kernel(q, k, v, context):
   if context.get("is_causal"):
     raise NotImplementedError("hip_flash is non-causal")
   q4, k4, v4, layout = _as_rank4(q, k, v, context["heads"])
+  q4, k4, v4, d0 = _pad_head_dim(q4, k4, v4)
   dt = q.dtype
   out = hip_flash_attention_vjp(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"],
                                 keep_mask=context.get("attention_mask"), layout=layout,
                                 residual_checkpoint_name=context.get("residual_checkpoint_name"))
   b, sq, h, d = out.shape
-  return out.reshape(b, sq, h * d).astype(dt)
+  return out[..., :d0].reshape(b, sq, h * d0).astype(dt)
 
 
 def hip_flash_fp8_kernel(q, k, v, context):
@@ -484,11 +498,12 @@ def hip_flash_fp8_kernel(q, k, v, context):
   if context.get("is_causal"):
     raise NotImplementedError("hip_flash is non-causal")
   q4, k4, v4, layout = _as_rank4(q, k, v, context["heads"])
+  q4, k4, v4, d0 = _pad_head_dim(q4, k4, v4)
   dt = q.dtype
   out, _ = hip_flash_attention_fp8(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"], layout,
                                    keep_mask=context.get("attention_mask"))
   b, sq, h, d = out.shape
-  return out.reshape(b, sq, h * d).astype(dt)
+  return out[..., :d0].reshape(b, sq, h * d0).astype(dt)
 
 
 def install():

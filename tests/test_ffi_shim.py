@@ -127,6 +127,7 @@ def fake_jax(monkeypatch):
     return _FakeArray(shape, parts[0].dtype)
 
   jnp.concatenate = concatenate
+  jnp.pad = lambda x, widths: _FakeArray(tuple(n + lo + hi for n, (lo, hi) in zip(x.shape, widths)), x.dtype)
   jax.ShapeDtypeStruct = lambda shape, dtype: _FakeArray(shape, dtype)
 
   def ffi_call(target, results, **kw):
@@ -254,6 +255,16 @@ def test_registered_entry_is_differentiable(fake_jax):
   fake_jax.clear()
   P.hip_flash_kernel(q3, k3, k3, dict(ctx, attention_mask=_FakeArray((B, Skv), "bool_")))
   assert targets() == ["mdattn_key_mask_bias", "mdattn_fwd_bf16_bias", "mdattn_bwd_bf16_bias"]
+  # head dims below 128 other than 64 are zero-padded to 64 / 128 around the custom calls (the reference pads to 128,
+  # attention_flax.py:223-259) and the output is cut back: rank 3 and rank 4, both registry names
+  for d, padded in ((40, 64), (80, 128), (64, 64)):
+    fake_jax.clear()
+    qd, kd = _FakeArray((B, S, H * d), bf), _FakeArray((B, Skv, H * d), bf)
+    assert P.hip_flash_kernel(qd, kd, kd, ctx).shape == (B, S, H * d)
+    fwd, bwd = [c for c in fake_jax if "target" in c]
+    assert fwd["operands"][0].shape == (B, S, H, padded) and bwd["operands"][1].shape == (B, Skv, H, padded)
+    assert P.hip_flash_kernel(_FakeArray((B, H, S, d), bf), _FakeArray((B, H, Skv, d), bf), _FakeArray((B, H, Skv, d), bf), ctx).shape == (B, S, H * d)
+    assert P.hip_flash_fp8_kernel(qd, kd, kd, ctx).shape == (B, S, H * d)
   # the static-scratch backward only where 2*B*H*ceil32(Sq) fits its array; beyond, the workspace form
   fake_jax.clear()
   P.hip_flash_attention_vjp(_FakeArray((B, S, H, D), bf), _FakeArray((B, Skv, H, D), bf), _FakeArray((B, Skv, H, D), bf), 0.1, static_scratch=True)

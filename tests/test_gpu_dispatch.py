@@ -132,3 +132,51 @@ def test_wan_i2v_cross_attention_block(dev):
     mx, mean = err_stats(got[b], want)
     print(f"i2v cross-attention, batch {b}: max-abs {mx:.3e} mean-abs {mean:.3e} rel-l2 {rel_l2(got[b], want):.3e}")
     assert mx <= 4e-2 and mean <= 4e-3 and rel_l2(got[b], want) <= 2e-2  # the sum of two bf16 outputs: twice the single-call bars
+
+
+@pytest.mark.parametrize("D", [40, 80, 96, 8])
+def test_head_dims_below_128_are_zero_padded(dev, D):
+  """The reference's flash wrappers pad head dims below 128 with zeros (attention_flax.py:223-259), so its registry
+  takes SD-1.x style heads of 40 / 80 as well; `hip_flash` pads to the next size its kernels take (64 or 128) and cuts
+  the output back.  Forward against the oracle at the true head dim (rank 3, rank 4, with a key mask), gradients
+  against torch autograd through an f32 attention on the same inputs."""
+  H, S, T = 3, 200, 77
+  q, k, v = O.normal_bf16((1, S, H * D), 0), O.normal_bf16((1, T, H * D), 1), O.normal_bf16((1, T, H * D), 2)
+  hsd = lambda x, n: np.ascontiguousarray(x.reshape(n, H, D).transpose(1, 0, 2))
+  op = A.AttentionOp(mesh=None, attention_kernel="hip_flash", scale=D**-0.5, heads=H, dim_head=D, dtype=torch.bfloat16)
+  qd, kd, vd = (to_dev_bf16(x, dev) for x in (q, k, v))
+  got = op.apply_attention(qd, kd, vd)
+  assert got.shape == (1, S, H * D) and got.dtype == torch.bfloat16
+  ro, _ = O.attention(hsd(q, S), hsd(k, T), hsd(v, T), D**-0.5)
+  mx, mean = err_stats(hsd(to_np(got), S), ro)
+  assert mx <= 2e-2 and mean <= 2e-3, (D, mx, mean)
+  to4 = lambda t, n: t.view(1, n, H, D).permute(0, 2, 1, 3).contiguous()
+  assert torch.equal(op.apply_attention(to4(qd, S), to4(kd, T), to4(vd, T)), got)
+  keep = np.random.default_rng(7).random((1, T)) < 0.6
+  gm = op.apply_attention(qd, kd, vd, attention_mask=torch.from_numpy(keep).to(dev))
+  rm, _ = O.attention(hsd(q, S), hsd(k, T), hsd(v, T), D**-0.5, kv_mask=keep[0])
+  mx, mean = err_stats(hsd(to_np(gm), S), rm)
+  assert mx <= 2e-2 and mean <= 2e-3, ("masked", D, mx, mean)
+  # gradients flow through the pad and the slice
+  ql, kl, vl = (t.clone().requires_grad_(True) for t in (qd, kd, vd))
+  g = to_dev_bf16(O.normal_bf16((1, S, H * D), 9), dev)
+  op.apply_attention(ql, kl, vl).backward(g)
+  qf, kf, vf = (t.float().view(1, -1, H, D).permute(0, 2, 1, 3).detach().requires_grad_(True) for t in (qd, kd, vd))
+  ref = torch.softmax(qf @ kf.transpose(-1, -2) * D**-0.5, dim=-1) @ vf
+  ref.backward(g.float().view(1, S, H, D).permute(0, 2, 1, 3))
+  for name, a, b in (("dq", ql.grad, qf.grad), ("dk", kl.grad, kf.grad), ("dv", vl.grad, vf.grad)):
+    assert a.shape == (1, a.shape[1], H * D)
+    want = b.permute(0, 2, 1, 3).reshape(a.shape)
+    err = float((a.float() - want).abs().max())
+    scale = float(want.abs().max())
+    assert err <= 2e-2 * max(1.0, scale), (D, name, err, scale)
+
+
+def test_fp8_registry_entry_pads_head_dims_too(dev):
+  H, S, D = 2, 300, 80
+  q, k, v = (to_dev_bf16(O.normal_bf16((1, S, H * D), s), dev) for s in (0, 1, 2))
+  mk = lambda name: A.AttentionOp(mesh=None, attention_kernel=name, scale=D**-0.5, heads=H, dim_head=D, dtype=torch.bfloat16)
+  got, want = mk("hip_flash_fp8").apply_attention(q, k, v), mk("hip_flash").apply_attention(q, k, v)
+  assert got.shape == want.shape == (1, S, H * D)
+  a, b = got.float().flatten(), want.float().flatten()
+  assert float(torch.dot(a, b) / (a.norm() * b.norm())) >= 0.995
