@@ -359,8 +359,9 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
     l += lsum;                                                                                                \
   }
 
-  // ring bookkeeping: period t uses slot t%4 (K(t), V(t-1)) and looks ahead into slot (t+1)%4
-  int s_cur = 0, s_nxt = 1, s_nn = 2, s_fill = 3;
+  // ring bookkeeping: period t uses slot t%4 (K(t), V(t-1)) and looks ahead into slot (t+1)%4.  The loop over periods is
+  // unrolled four times, one copy per ring slot, so that every fragment address is a lane constant plus a compile-time
+  // offset: the stream carries no address arithmetic.
   // fragments the first iteration's first QK / PV MFMA expect in the windows
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): Q fragments and this wave's share of slots 0..2
   __syncthreads();
@@ -379,7 +380,8 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
     kofs_i[i] = kofs + (unsigned)(4 * NW * i * (int)a.k_ss) * 2u;
     vofs_i[i] = vofs + (unsigned)(4 * NW * i * (int)a.v_ss) * 2u;
   }
-  for (int t = 0; t <= nt; ++t) {
+  auto period = [&](int t, auto slot_c) __attribute__((always_inline)) {
+    constexpr int s_cur = decltype(slot_c)::value, s_nxt = (s_cur + 1) & 3, s_fill = (s_cur + 3) & 3;
     // every wave's loads into slot s_nxt (issued two periods ago) have landed once all waves pass the
     // barrier: only the loads of the previous period (2 * 16 / NW per wave) may still be in flight.
     // Slot s_fill was last read in period t-1 and now receives K(t+3), V(t+2).
@@ -413,11 +415,15 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
     vdma += kBN * a.v_ss;
     // iteration 2t: softmax(2t), PV(2t-1), QK(2t+1)
     MDATTN_ITER(Sb, Sa, Pb, Pa, Kc1, Kn0, Vc1, Vn0, 2 * t)
-    const int tmp = s_cur;
-    s_cur = s_nxt;
-    s_nxt = s_nn;
-    s_nn = s_fill;
-    s_fill = tmp;
+  };
+  for (int t = 0; t <= nt; t += 4) {
+    period(t, std::integral_constant<int, 0>{});
+    if (t + 1 > nt) break;
+    period(t + 1, std::integral_constant<int, 1>{});
+    if (t + 2 > nt) break;
+    period(t + 2, std::integral_constant<int, 2>{});
+    if (t + 3 > nt) break;
+    period(t + 3, std::integral_constant<int, 3>{});
   }
 #undef MDATTN_ITER
 
@@ -567,7 +573,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
   // waits for every read right before its MFMA.
   constexpr int LA = HD == 128 ? MDATTN_FLAT_LA128 : 0;
   constexpr int FPB = NJ + 2 * ND, NFRAG = NB * FPB;
-  auto tile = [&](int t, int slot, auto masked) __attribute__((always_inline)) {
+  auto tile = [&](int t, auto slot, auto masked) __attribute__((always_inline)) {  // slot: int or integral_constant
     const __bf16* base = smem + slot * STAGE;
     constexpr int kBlk = 32 * 64;  // a 32-key block of a head-dim-64 tile: 32 rows of 64 elements, in K and in V
     auto frag = [&](int n) __attribute__((always_inline)) {
@@ -722,19 +728,33 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
   // SLOTS - 1 tiles are requested ahead of the one being worked on
 #pragma unroll
   for (int i = 1; i < SLOTS - 1; ++i) dma(i, i);
-  int slot = 0, fill = SLOTS - 1;
-  for (int t = 0; t < nt - 1; ++t) {
+  auto step = [&](int t, auto slot, int fill) __attribute__((always_inline)) {
     // vmcnt: this wave's share of tile t has landed (the SLOTS - 2 tiles requested after it may still be in flight)
     __builtin_amdgcn_s_waitcnt(0x0F70 | ((SLOTS - 2) * (2 * GPW + (BIAS ? 1 : 0))));
     __syncthreads();                                  // ... and everyone's; slot `fill` (tile t-1) is free
     dma(fill, t + SLOTS - 1);
     tile(t, slot, std::false_type{});
-    slot = slot == SLOTS - 1 ? 0 : slot + 1;
-    fill = fill == SLOTS - 1 ? 0 : fill + 1;
+  };
+  if constexpr (HD == 64) {
+    // Two copies of the loop body, one per ring slot: the slot is a compile-time constant in each, every fragment
+    // address a lane constant plus an immediate offset, and the address arithmetic per tile is gone from a kernel that
+    // is bound by vector issue (1 % at 32 heads x 13,376 tokens; at head dim 128 the copies cost registers and lose).
+    for (int t = 0; t < nt - 1; t += 2) {
+      step(t, std::integral_constant<int, 0>{}, 1);
+      if (t + 1 >= nt - 1) break;
+      step(t + 1, std::integral_constant<int, 1>{}, 0);
+    }
+  } else {
+    int slot = 0, fill = SLOTS - 1;
+    for (int t = 0; t < nt - 1; ++t) {
+      step(t, slot, fill);
+      slot = slot == SLOTS - 1 ? 0 : slot + 1;
+      fill = fill == SLOTS - 1 ? 0 : fill + 1;
+    }
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
-  tile(nt - 1, slot, std::true_type{});
+  tile(nt - 1, (nt - 1) % SLOTS, std::true_type{});
 
   if (a.o_run) {  // ring step: merged into the f32 carry, row by row
     store_row<ND>(a, O, xhalf_sum(l), mc, b, h, q0 + l32, hh);
