@@ -165,8 +165,12 @@ def hip_flash_kernel(q, k, v, context):
 
 @register_kernel("hip_flash_fp8")
 def hip_flash_fp8_kernel(q, k, v, context):
-  """fp8-e4m3 variant: per-tensor absmax quantisation of q, k, v on the device, then the fp8 kernel."""
+  """fp8-e4m3 variant: per-tensor absmax quantisation of q, k, v on the device, then the fp8 kernel.  Forward only:
+  called with inputs that require a gradient while autograd is recording, it raises instead of returning a result that
+  would silently carry no gradient (train through `hip_flash`)."""
   _reject_unsupported(context)
+  if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+    raise NotImplementedError("hip_flash_fp8 has no backward pass: use hip_flash for training, or call it under torch.no_grad()")
   heads = context["heads"]
   qv, kv, vv, d0 = _pad_head_dim(*(_as_bshd(t, heads).to(torch.bfloat16) for t in (q, k, v)))
   qv, kv, vv = qv.contiguous(), kv.contiguous(), vv.contiguous()

@@ -120,6 +120,14 @@ def test_cpu_tensors_are_refused_not_computed():
     _call(q, q, q, "hip_flash", heads=2, dim_head=128)
 
 
+def test_fp8_entry_refuses_to_be_differentiated():
+  q = torch.zeros(1, 8, 2 * 128, dtype=torch.bfloat16, requires_grad=True)
+  with pytest.raises(NotImplementedError, match="no backward"):
+    _call(q, q, q, "hip_flash_fp8", heads=2, dim_head=128)
+  with torch.no_grad(), pytest.raises(ValueError, match="no CPU path"):  # without autograd it goes on to the kernels
+    _call(q, q, q, "hip_flash_fp8", heads=2, dim_head=128)
+
+
 def test_attention_op_mirrors_constructor_and_call():
   op = A.AttentionOp(mesh=None, attention_kernel="fake", scale=0.5, heads=2, dim_head=4, dtype=torch.bfloat16)
   q = torch.zeros(1, 8, 8)
