@@ -67,20 +67,20 @@ def test_ring_replay_small_unequal_chunks(dev):
 
 
 @pytest.mark.parametrize("layout", ["bshd", "bhsd"])
-@pytest.mark.parametrize("variant", [0, 1, 3])
-def test_fused_ring_step_equals_attention_then_merge(dev, request, layout, variant):
+@pytest.mark.parametrize("variant,D", [(0, 128), (1, 128), (3, 128), (0, 64)])
+def test_fused_ring_step_equals_attention_then_merge(dev, request, layout, variant, D):
   """mdattn_fwd_bf16_merge (attention + merge in the attention kernel's epilogue) against the two separate calls
-  and against the oracle, with ragged chunks, through both schedules and both layouts of the carry."""
+  and against the oracle, with ragged chunks, through both schedules and both layouts of the carry, at both head dims."""
   ops.set_fwd_schedule(variant)
   request.addfinalizer(lambda: ops.set_fwd_schedule(0))
   H, Sq = 3, 333
-  q = O.normal_bf16((1, Sq, H, 128), 0)
+  q = O.normal_bf16((1, Sq, H, D), 0)
   sizes = [4200, 1, 63, 777, 3100]
-  ks = [O.normal_bf16((1, n, H, 128), 10 + i) for i, n in enumerate(sizes)]
-  vs = [O.normal_bf16((1, n, H, 128), 20 + i) for i, n in enumerate(sizes)]
+  ks = [O.normal_bf16((1, n, H, D), 10 + i) for i, n in enumerate(sizes)]
+  vs = [O.normal_bf16((1, n, H, D), 20 + i) for i, n in enumerate(sizes)]
   qd = to_dev_bf16(q, dev)
-  o_f, l_f = ops.new_merge_state(1, Sq, H, 128, dev, layout=layout)
-  o_s, l_s = ops.new_merge_state(1, Sq, H, 128, dev, layout=layout)
+  o_f, l_f = ops.new_merge_state(1, Sq, H, D, dev, layout=layout)
+  o_s, l_s = ops.new_merge_state(1, Sq, H, D, dev, layout=layout)
   for kc, vc in zip(ks, vs):
     kd, vd = to_dev_bf16(kc, dev), to_dev_bf16(vc, dev)
     ops.flash_attention_merge(qd, kd, vd, o_f, l_f)
@@ -89,11 +89,11 @@ def test_fused_ring_step_equals_attention_then_merge(dev, request, layout, varia
   # the separate path rounds each chunk's output to bf16 before the merge, the fused one does not
   assert float((o_f - o_s).abs().max()) < 8e-3
   assert float((l_f - l_s).abs().max()) < 1e-5
-  ro, rl = O.attention(hsd(q), hsd(np.concatenate(ks, 1)), hsd(np.concatenate(vs, 1)), 128**-0.5)
+  ro, rl = O.attention(hsd(q), hsd(np.concatenate(ks, 1)), hsd(np.concatenate(vs, 1)), D**-0.5)
   out = to_np(ops.finalize(o_f))
   mx, mean = err_stats(hsd(out), ro)
   mx_s = err_stats(hsd(to_np(ops.finalize(o_s))), ro)[0]
-  print(f"fused ring step ({layout}, variant {variant}): max-abs {mx:.3e} (separate calls {mx_s:.3e}) mean-abs {mean:.3e}")
+  print(f"fused ring step ({layout}, variant {variant}, D={D}): max-abs {mx:.3e} (separate calls {mx_s:.3e}) mean-abs {mean:.3e}")
   assert mx < 2e-2 and mean < 2e-3 and rel_l2(hsd(out), ro) < 1.5e-2
   assert err_stats(to_np(l_f)[0], rl)[0] < 1e-3
 
