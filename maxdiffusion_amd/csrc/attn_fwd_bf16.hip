@@ -444,7 +444,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
 // pipe busy.  Same tile layouts, same fragment reads, same arithmetic as the pipelined kernel.
 // Head dim 64 (template HD) uses 128-byte rows: one load instruction fills 8 rows, K chunk c of row r sits at
 // position c ^ ((r >> 1) & 7), V chunk c at c ^ 4*((r >> 1) & 1), both unpadded and conflict-free for the
-// same two read patterns; its 109-128 VGPRs and 32 KB of LDS (64-key tiles, two 32-key blocks per slot, in a 2-slot
+// same two read patterns; its 104-128 VGPRs and 32 KB of LDS (64-key tiles, two 32-key blocks per slot, in a 2-slot
 // ring) let four workgroups share a CU (four waves per SIMD: 3 % faster than three at 32 heads x 13,376 tokens, where
 // the softmax per MFMA FLOP is twice that of head dim 128).
 constexpr int kTS = 32;                               // keys per tile
