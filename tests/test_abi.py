@@ -53,6 +53,41 @@ def test_build_id_and_schedule_hook(lib):
   assert lib.mdattn_set_fwd_schedule(0) == 0
 
 
+def test_header_is_plain_c_and_a_c_program_links_against_the_library(lib, tmp_path):
+  """The boundary is a C ABI: include/mdattn.h compiles as C99 and as C++11 with the host compilers (no HIP, no torch
+  type in it), and a C program that calls the host-only entry points links against libmdattn.so and runs."""
+  import shutil
+  import subprocess
+
+  from maxdiffusion_amd import build
+
+  gcc, gxx = shutil.which("gcc"), shutil.which("g++")
+  if not gcc or not gxx:
+    pytest.skip("no host C / C++ compiler")
+  inc = os.path.dirname(HEADER)
+  src = tmp_path / "abi.c"
+  src.write_text(
+      '#include <stdio.h>\n#include <string.h>\n#include "mdattn.h"\n'
+      "int main(void) {\n"
+      "  mdattn_strides s; memset(&s, 0, sizeof s);\n"
+      "  if (mdattn_version() != MDATTN_VERSION) return 2;\n"
+      '  if (strcmp(mdattn_strerror(MDATTN_OK), "ok") != 0) return 3;\n'
+      "  /* a null operand is refused on the host: no kernel is launched */\n"
+      "  if (mdattn_fwd_bf16(0, 0, 0, 0, 0, 0, 1, 1, 1, 1, 128, &s, &s, &s, &s, 1.0f) != MDATTN_E_BADARG) return 4;\n"
+      '  printf("%s\\n", mdattn_build_id());\n'
+      "  return 0;\n}\n")
+  subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", f"-I{inc}", str(src)], check=True)
+  cxx = tmp_path / "abi.cc"
+  cxx.write_text('#include "mdattn.h"\nint main() { return mdattn_version() == MDATTN_VERSION ? 0 : 1; }\n')
+  subprocess.run([gxx, "-std=c++11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", f"-I{inc}", str(cxx)], check=True)
+  exe = tmp_path / "abi"
+  libdir = os.path.dirname(build.LIB_PATH)
+  subprocess.run([gcc, "-std=c99", f"-I{inc}", str(src), "-o", str(exe), f"-L{libdir}", "-l:libmdattn.so", f"-Wl,-rpath,{libdir}"], check=True)
+  r = subprocess.run([str(exe)], capture_output=True, text=True)
+  assert r.returncode == 0, (r.returncode, r.stderr)
+  assert r.stdout.strip() == build.source_id()
+
+
 def test_stale_library_is_refused(monkeypatch):
   from maxdiffusion_amd import _lib, build
 
