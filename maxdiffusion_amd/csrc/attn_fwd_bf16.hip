@@ -319,7 +319,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_bf16_kernel(AttnArgs a) {
             asm volatile("" : "+v"(pe));                                                                      \
           } else {                                                                                            \
             unsigned pk = pack2(pe, x);                                                                       \
-            lsum += pe + x;                                                                                   \
+            lsum = e == 1 ? pe + x : lsum + (pe + x); /* no add of the initial zero */                        \
             asm volatile("" : "+v"(pk), "+v"(lsum));                                                          \
             PC[e >> 3][(e >> 1) & 3] = pk;                                                                    \
           }                                                                                                   \
@@ -640,7 +640,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(HD == 6
         for (int e = 0; e < 8; e += 2) {
           const float x0 = __builtin_amdgcn_exp2f(PRE ? S[8 * hb + e] : __builtin_fmaf(S[8 * hb + e], cs, -rf));
           const float x1 = __builtin_amdgcn_exp2f(PRE ? S[8 * hb + e + 1] : __builtin_fmaf(S[8 * hb + e + 1], cs, -rf));
-          lsum += x0;
+          lsum = (hb == 0 && e == 0) ? x0 : lsum + x0;  // no add of the initial zero
           lsum += x1;
           pk[e >> 1] = pack2(x0, x1);
           asm volatile("" : "+v"(pk[e >> 1]), "+v"(lsum));
