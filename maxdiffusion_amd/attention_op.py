@@ -88,6 +88,11 @@ def _mask_bias(context, qv, kv):
   return ops.key_mask_bias(mask)
 
 
+# From this many keys on, the registry entry folds the softmax scale into q before the call (see hip_flash_kernel): the
+# pass over q costs what the multiply per logit costs at about 8,000 keys.
+FOLD_SCALE_MIN_KEYS = 16384
+
+
 def _pad_head_dim(qv, kv, vv):
   """Head dims below 128 other than 64 are zero-padded to the next size the kernels take (64 or 128), as the
   reference's flash wrappers pad them to 128 (attention_flax.py:223-259, `_pad_data_for_flash`): zero columns of q and
@@ -154,10 +159,19 @@ def hip_flash_kernel(q, k, v, context):
   # segment ids (:390-438); rows without a kept key return 0 (:1552-1554)
   bias = _mask_bias(context, qv, kv)
   qv, kv, vv, d0 = _pad_head_dim(qv, kv, vv)
+  scale = context["scale"]
   if torch.is_grad_enabled() and (qv.requires_grad or kv.requires_grad or vv.requires_grad):
-    out = hip_flash_attention_autograd(qv, kv, vv, context["scale"], bias)
+    out = hip_flash_attention_autograd(qv, kv, vv, scale, bias)
   else:
-    out = ops.flash_attention(qv, kv, vv, scale=context["scale"], key_bias=bias)
+    c = scale * math.log2(math.e)
+    if bias is None and kv.shape[1] >= FOLD_SCALE_MIN_KEYS and abs(c - 1.0) > 1e-6:
+      # Long key sequences: q * (scale * log2 e), rounded to bf16 once, then scale = ln 2, on which the kernels drop the
+      # multiply per logit (3.5 % of the launch at head dim 128, 7 % at 64) for one pass over q.  The reference's flash
+      # wrappers round the same factors into their operands (k * scale and q * log2 e in bf16,
+      # attention_flax.py:1783, :610).  Callers that apply the fused prologue with q_mul arrive here with scale = ln 2
+      # already and skip this.
+      qv, scale = qv * c, ops.FOLDED_SCALE
+    out = ops.flash_attention(qv, kv, vv, scale=scale, key_bias=bias)
   b, s, h, d = out.shape
   out = out[..., :d0].reshape(b, s, h * d0)
   return out.to(q.dtype) if cast else out

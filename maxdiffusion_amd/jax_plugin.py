@@ -50,6 +50,7 @@ BWD_STATIC_MAX_FLOATS = 8 * 1024 * 1024  # MDATTN_BWD_STATIC_MAX_FLOATS of inclu
 NORM_ROPE_BWD_MAX_PARTIAL_ROWS = 1024    # mdattn_norm_rope_bwd_workspace_floats(rows, columns) = min(rows, 1024) * columns
 
 FOLDED_SCALE = math.log(2.0)  # see ops.FOLDED_SCALE: scale * log2(e) == 1, the softmax scale rides on q
+FOLD_SCALE_MIN_KEYS = 16384   # from this many keys on, hip_flash_kernel folds the scale into q itself
 
 _installed = False
 
@@ -484,8 +485,16 @@ def hip_flash_kernel(q, k, v, context):
   q4, k4, v4, layout = _as_rank4(q, k, v, context["heads"])
   q4, k4, v4, d0 = _pad_head_dim(q4, k4, v4)
   dt = q.dtype
-  out = hip_flash_attention_vjp(q4.astype(jnp.bfloat16), k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), context["scale"],
-                                keep_mask=context.get("attention_mask"), layout=layout,
+  scale, mask = context["scale"], context.get("attention_mask")
+  q4 = q4.astype(jnp.bfloat16)
+  c = scale * math.log2(math.e)
+  if mask is None and k4.shape[2 if layout else 1] >= FOLD_SCALE_MIN_KEYS and abs(c - 1.0) > 1e-6:
+    # long key sequences: q * (scale * log2 e) in bf16 (XLA fuses the multiply into q's producer) and scale = ln 2, on
+    # which forward and backward kernels drop the multiply per logit; the reference rounds the same factors into its
+    # operands (attention_flax.py:1783, :610).  Autodiff scales dq back through the multiply.
+    q4, scale = q4 * c, FOLDED_SCALE
+  out = hip_flash_attention_vjp(q4, k4.astype(jnp.bfloat16), v4.astype(jnp.bfloat16), scale,
+                                keep_mask=mask, layout=layout,
                                 residual_checkpoint_name=context.get("residual_checkpoint_name"))
   b, sq, h, d = out.shape
   return out[..., :d0].reshape(b, sq, h * d0).astype(dt)

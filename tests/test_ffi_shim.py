@@ -265,6 +265,18 @@ def test_registered_entry_is_differentiable(fake_jax):
     assert fwd["operands"][0].shape == (B, S, H, padded) and bwd["operands"][1].shape == (B, Skv, H, padded)
     assert P.hip_flash_kernel(_FakeArray((B, H, S, d), bf), _FakeArray((B, H, Skv, d), bf), _FakeArray((B, H, Skv, d), bf), ctx).shape == (B, S, H * d)
     assert P.hip_flash_fp8_kernel(qd, kd, kd, ctx).shape == (B, S, H * d)
+  # long key sequences: the entry multiplies q by scale * log2(e) itself and hands the kernels scale = ln 2 (forward
+  # and backward then run without a multiply per logit); not with a key mask, not when the caller's scale is ln 2 already
+  long_k = _FakeArray((B, P.FOLD_SCALE_MIN_KEYS, H * D), bf)
+  for c, want in ((ctx, P.FOLDED_SCALE), (dict(ctx, scale=P.FOLDED_SCALE), P.FOLDED_SCALE),
+                  (dict(ctx, attention_mask=_FakeArray((B, P.FOLD_SCALE_MIN_KEYS), "bool_")), 0.1)):
+    fake_jax.clear()
+    P.hip_flash_kernel(q3, long_k, long_k, c)
+    scales = {float(x["attrs"]["scale"]) for x in fake_jax if "target" in x and "scale" in x["attrs"]}
+    assert scales == {float(np.float32(want))}, (scales, want)
+  fake_jax.clear()
+  P.hip_flash_kernel(q3, k3, k3, ctx)  # 60 keys: the caller's scale goes through
+  assert {float(x["attrs"]["scale"]) for x in fake_jax if "target" in x} == {float(np.float32(0.1))}
   # the static-scratch backward only where 2*B*H*ceil32(Sq) fits its array; beyond, the workspace form
   fake_jax.clear()
   P.hip_flash_attention_vjp(_FakeArray((B, S, H, D), bf), _FakeArray((B, Skv, H, D), bf), _FakeArray((B, Skv, H, D), bf), 0.1, static_scratch=True)

@@ -180,3 +180,26 @@ def test_fp8_registry_entry_pads_head_dims_too(dev):
   assert got.shape == want.shape == (1, S, H * D)
   a, b = got.float().flatten(), want.float().flatten()
   assert float(torch.dot(a, b) / (a.norm() * b.norm())) >= 0.995
+
+
+def test_registry_folds_the_scale_into_q_on_long_key_sequences(dev):
+  """From FOLD_SCALE_MIN_KEYS keys on (no mask, no autograd) `hip_flash` multiplies q by scale * log2(e) itself and
+  calls the kernels with scale = ln 2; below, and for a caller that already carries the factor, the scale goes through
+  unchanged.  Either way the result meets the bars against the oracle."""
+  from maxdiffusion_amd import ops
+
+  H, S, D = 2, 300, 128
+  for skv, scale, want in ((A.FOLD_SCALE_MIN_KEYS + 77, D**-0.5, ops.FOLDED_SCALE), (A.FOLD_SCALE_MIN_KEYS - 1, D**-0.5, D**-0.5),
+                           (A.FOLD_SCALE_MIN_KEYS, ops.FOLDED_SCALE, ops.FOLDED_SCALE)):
+    q, k, v = O.normal_bf16((1, S, H * D), 0), O.normal_bf16((1, skv, H * D), 1), O.normal_bf16((1, skv, H * D), 2)
+    if scale == ops.FOLDED_SCALE:  # what the fused prologue hands over with q_mul
+      q = O.bf16_round(q * np.float32(ops.folded_q_mul(D)))
+    op = A.AttentionOp(mesh=None, attention_kernel="hip_flash", scale=scale, heads=H, dim_head=D, dtype=torch.bfloat16)
+    with mock.patch.object(A.ops, "flash_attention", wraps=ops.flash_attention) as spy:
+      got = op.apply_attention(to_dev_bf16(q, dev), to_dev_bf16(k, dev), to_dev_bf16(v, dev))
+    assert spy.call_args.kwargs["scale"] == want, (skv, scale, spy.call_args.kwargs["scale"])
+    hsd = lambda x, n: np.ascontiguousarray(x.reshape(n, H, D).transpose(1, 0, 2))
+    ro, _ = O.attention(hsd(q, S), hsd(k, skv), hsd(v, skv), scale)
+    mx, mean = err_stats(hsd(to_np(got), S), ro)
+    print(f"Skv={skv} scale={scale:.4f}: max-abs {mx:.3e} mean-abs {mean:.3e}")
+    assert mx <= 2e-2 and mean <= 2e-3 and rel_l2(hsd(to_np(got), S), ro) <= 1.5e-2, (skv, mx, mean)
