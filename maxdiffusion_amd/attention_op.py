@@ -88,8 +88,9 @@ def _mask_bias(context, qv, kv):
   return ops.key_mask_bias(mask)
 
 
-# From this many keys on, the registry entry folds the softmax scale into q before the call (see hip_flash_kernel): the
-# pass over q costs what the multiply per logit costs at about 8,000 keys.
+# From this many keys on at head dim 128 (half as many at head dim 64, where the multiply weighs twice as much), the
+# registry entry folds the softmax scale into q before the call (see hip_flash_kernel): the pass over q costs what the
+# multiply per logit costs at about 9,000 (4,000) keys.
 FOLD_SCALE_MIN_KEYS = 16384
 
 
@@ -164,7 +165,7 @@ def hip_flash_kernel(q, k, v, context):
     out = hip_flash_attention_autograd(qv, kv, vv, scale, bias)
   else:
     c = scale * math.log2(math.e)
-    if bias is None and kv.shape[1] >= FOLD_SCALE_MIN_KEYS and abs(c - 1.0) > 1e-6:
+    if bias is None and kv.shape[1] * 128 >= FOLD_SCALE_MIN_KEYS * qv.shape[-1] and abs(c - 1.0) > 1e-6:
       # Long key sequences: q * (scale * log2 e), rounded to bf16 once, then scale = ln 2, on which the kernels drop the
       # multiply per logit (3.5 % of the launch at head dim 128, 7 % at 64) for one pass over q.  The reference's flash
       # wrappers round the same factors into their operands (k * scale and q * log2 e in bf16,

@@ -50,7 +50,7 @@ BWD_STATIC_MAX_FLOATS = 8 * 1024 * 1024  # MDATTN_BWD_STATIC_MAX_FLOATS of inclu
 NORM_ROPE_BWD_MAX_PARTIAL_ROWS = 1024    # mdattn_norm_rope_bwd_workspace_floats(rows, columns) = min(rows, 1024) * columns
 
 FOLDED_SCALE = math.log(2.0)  # see ops.FOLDED_SCALE: scale * log2(e) == 1, the softmax scale rides on q
-FOLD_SCALE_MIN_KEYS = 16384   # from this many keys on, hip_flash_kernel folds the scale into q itself
+FOLD_SCALE_MIN_KEYS = 16384   # from this many keys on (head dim 128; half at 64), hip_flash_kernel folds the scale into q itself
 
 _installed = False
 
@@ -488,7 +488,7 @@ def hip_flash_kernel(q, k, v, context):
   scale, mask = context["scale"], context.get("attention_mask")
   q4 = q4.astype(jnp.bfloat16)
   c = scale * math.log2(math.e)
-  if mask is None and k4.shape[2 if layout else 1] >= FOLD_SCALE_MIN_KEYS and abs(c - 1.0) > 1e-6:
+  if mask is None and k4.shape[2 if layout else 1] * 128 >= FOLD_SCALE_MIN_KEYS * k4.shape[-1] and abs(c - 1.0) > 1e-6:
     # long key sequences: q * (scale * log2 e) in bf16 (XLA fuses the multiply into q's producer) and scale = ln 2, on
     # which forward and backward kernels drop the multiply per logit; the reference rounds the same factors into its
     # operands (attention_flax.py:1783, :610).  Autodiff scales dq back through the multiply.
